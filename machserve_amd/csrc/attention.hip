@@ -1,0 +1,253 @@
+// Causal grouped-query attention of a mixed batch over a paged cache, on the matrix cores.
+//
+// Role in the reference: attn_paged_tiled_*_gqa and *_gqa_runs
+// (crates/mach-model/src/kernels.rs:1367-1496, 1650-1885): K/V tiles staged in LDS and
+// shared by the query heads of one KV head, online softmax with
+// m' = max(m, tile_max), acc = acc * exp(m - m') + sum exp(s - m') V.
+//
+// One block = 64 "flat rows" of one request and one KV head.  Flat row r of a request is
+// (token r / g, query head kvh * g + r % g), g = heads per KV head: a prompt portion of n
+// tokens has n * g rows, a decoded token g rows, and any g works the same way.  Each of the
+// four waves owns 16 flat rows.  Scores are computed transposed, S^T = K Q^T, so that a lane
+// holds four consecutive keys of one query row: row maxima and sums stay in the lane (plus
+// two cross-lane steps), and the probabilities are already laid out as the B operand of
+// O^T = V^T P^T.  V is stored transposed in its pages ([head_dim][page_size]) so that V^T
+// tiles load with contiguous 16-byte reads.
+//
+// Key tiles start at absolute multiples of BKV from key 0, whatever the portion, so a
+// row's result does not depend on how its request was cut into steps.
+//
+// Compiled once per MS_ATTN_ND (tile head size / 16); a smaller head size runs in the next
+// larger tile with the unused columns zero.
+#include "common.cuh"
+
+#ifndef MS_ATTN_ND
+#error "MS_ATTN_ND: head-size tile in units of 16"
+#endif
+
+namespace ms {
+
+constexpr int ND = MS_ATTN_ND;
+constexpr int HDT = ND * 16;             // head size of the tile
+constexpr int NKS = (HDT + 31) / 32;     // K steps of 32 over the head size
+#ifdef MS_ELEM_BF16
+constexpr int BKV = ND <= 8 ? 64 : 32;
+constexpr int EPC = 8;
+constexpr int KPAD = 8, VPAD = 8;
+#else
+constexpr int BKV = ND <= 4 ? 64 : (ND <= 8 ? 32 : 16);
+constexpr int EPC = 4;
+constexpr int KPAD = 4, VPAD = 4;
+#endif
+constexpr int NT = BKV / 16;             // 16-key score tiles per key tile
+constexpr int NTP = (NT + 1) / 2;        // pairs of score tiles = K steps of the PV product
+constexpr int K_LD = HDT + KPAD, V_LD = BKV + VPAD;
+constexpr int ROWS_PER_BLOCK = 64;
+constexpr float NEG_BIG = -1e30f;
+
+struct AttnArgs {
+    const elem_t* q;         // [T, H, hd]
+    const elem_t* kpool;     // [pages, KV, ps, hd]
+    const elem_t* vpool;     // [pages, KV, hd, ps]
+    elem_t* out;             // [T, H * hd]
+    const int* block_table;  // [S, table_stride]
+    const int* seq_q_start;  // [S] first row of the request in this step
+    const int* seq_q_len;    // [S] rows of the request in this step
+    const int* seq_pos0;     // [S] position of its first row
+    const int* work;         // [W, 2] (request index, first flat row)
+    int table_stride, H, KV, hd, ps, window;
+    float scale;
+};
+
+__device__ __forceinline__ float exp_f(float x) {
+#ifdef MS_ELEM_BF16
+    return __expf(x);
+#else
+    return expf(x);
+#endif
+}
+
+__global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
+    __shared__ __attribute__((aligned(16))) elem_t Ks[BKV * K_LD];
+    __shared__ __attribute__((aligned(16))) elem_t Vs[HDT * V_LD];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, grp = lane >> 4;
+    const int s = a.work[blockIdx.x * 2], r0 = a.work[blockIdx.x * 2 + 1];
+    const int kvh = blockIdx.y;
+    const int g = a.H / a.KV;
+    const int q_start = a.seq_q_start[s], q_len = a.seq_q_len[s], pos0 = a.seq_pos0[s];
+    const int R = q_len * g;
+    const int hd = a.hd, ps = a.ps;
+    const int* table = a.block_table + (size_t)s * a.table_stride;
+
+    // this lane's query row
+    const int row = r0 + wave * 16 + r16;
+    const bool valid = row < R;
+    const int tok = valid ? row / g : 0;
+    const int head = kvh * g + (valid ? row % g : 0);
+    const int pos = pos0 + tok;
+    const bool wave_active = r0 + wave * 16 < R;
+
+    // keys any row of the block may see
+    const int last_row = min(r0 + ROWS_PER_BLOCK, R) - 1;
+    const int kv_hi = pos0 + last_row / g + 1;
+    int kv_lo = 0;
+    if (a.window > 0) kv_lo = max(0, pos0 + r0 / g - a.window + 1);
+    const int lo_key = a.window > 0 ? pos - a.window + 1 : 0;
+
+    Frag qf[NKS];
+    {
+        const elem_t* qrow = a.q + ((size_t)(q_start + tok) * a.H + head) * hd;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            const int d0 = ks * 32 + grp * 8;
+            qf[ks] = (valid && d0 < hd) ? frag_load(qrow + d0) : frag_zero();
+        }
+    }
+
+    f32x4 acc_o[ND];
+#pragma unroll
+    for (int i = 0; i < ND; ++i) acc_o[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m_run = NEG_BIG, l_run = 0.f;
+
+    for (int kt0 = (kv_lo / BKV) * BKV; kt0 < kv_hi; kt0 += BKV) {
+        __syncthreads();  // the previous tile has been consumed
+        // K tile: [BKV keys][HDT]
+        constexpr int CPRK = HDT / EPC;
+        for (int c = tid; c < BKV * CPRK; c += 256) {
+            const int kl = c / CPRK, d0 = (c % CPRK) * EPC, key = kt0 + kl;
+            u32x4 v = {0, 0, 0, 0};
+            if (key < kv_hi && d0 < hd) {
+                const int page = table[key / ps];
+                if (page >= 0)
+                    v = *reinterpret_cast<const u32x4*>(a.kpool + (((size_t)page * a.KV + kvh) * ps + key % ps) * hd + d0);
+            }
+            *reinterpret_cast<u32x4*>(&Ks[kl * K_LD + d0]) = v;
+        }
+        // V^T tile: [HDT][BKV keys]
+        constexpr int CPRV = BKV / EPC;
+        for (int c = tid; c < HDT * CPRV; c += 256) {
+            const int d = c / CPRV, k0 = (c % CPRV) * EPC, key = kt0 + k0;
+            u32x4 v = {0, 0, 0, 0};
+            if (key < kv_hi && d < hd) {
+                const int page = table[key / ps];
+                if (page >= 0)
+                    v = *reinterpret_cast<const u32x4*>(a.vpool + (((size_t)page * a.KV + kvh) * hd + d) * ps + key % ps);
+            }
+            *reinterpret_cast<u32x4*>(&Vs[d * V_LD + k0]) = v;
+        }
+        __syncthreads();
+        if (!wave_active) continue;
+
+        // S^T = K Q^T: lane holds keys grp * 4 + i of tile nt for query row r16
+        f32x4 sc[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            sc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+                const int d0 = ks * 32 + grp * 8;
+                Frag kf = (d0 < HDT) ? frag_load(&Ks[(nt * 16 + r16) * K_LD + d0]) : frag_zero();
+                mma_16x16x32(sc[nt], kf, qf[ks]);
+            }
+        }
+        float tmax = NEG_BIG;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = kt0 + nt * 16 + grp * 4 + i;
+                const bool ok = valid && key <= pos && key >= lo_key;
+                const float v = ok ? sc[nt][i] * a.scale : -INFINITY;
+                sc[nt][i] = v;
+                tmax = fmaxf(tmax, v);
+            }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+        const float m_new = fmaxf(m_run, tmax);
+        const float alpha = exp_f(m_run - m_new);
+        float psum = 0.f;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float p = exp_f(sc[nt][i] - m_new);
+                sc[nt][i] = p;
+                psum += p;
+            }
+        psum += __shfl_xor(psum, 16, WAVE);
+        psum += __shfl_xor(psum, 32, WAVE);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc_o[dt][i] *= alpha;
+
+        // O^T += V^T P^T: the probabilities of two score tiles form one B fragment
+#pragma unroll
+        for (int pp = 0; pp < NTP; ++pp) {
+            Frag pf;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                pf.v[i] = from_f32<elem_t>(sc[2 * pp][i]);
+                pf.v[4 + i] = (2 * pp + 1 < NT) ? from_f32<elem_t>(sc[(2 * pp + 1 < NT) ? 2 * pp + 1 : 0][i]) : from_f32<elem_t>(0.f);
+            }
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt) {
+                Frag vf;
+                const elem_t* v0 = &Vs[(dt * 16 + r16) * V_LD + (2 * pp) * 16 + grp * 4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) vf.v[i] = v0[i];
+                if (2 * pp + 1 < NT) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) vf.v[4 + i] = v0[16 + i];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) vf.v[4 + i] = from_f32<elem_t>(0.f);
+                }
+                mma_16x16x32(acc_o[dt], vf, pf);
+            }
+        }
+    }
+
+    if (valid) {
+        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+        elem_t* orow = a.out + ((size_t)(q_start + tok) * a.H + head) * hd;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) {
+            const int d0 = dt * 16 + grp * 4;
+            if (d0 < hd) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) orow[d0 + i] = from_f32<elem_t>(acc_o[dt][i] * inv);
+            }
+        }
+    }
+}
+
+}  // namespace ms
+
+using namespace ms;
+
+#define MS_CAT2(a, b) a##b
+#define MS_CAT(a, b) MS_CAT2(a, b)
+
+// Attention of a mixed batch.  `work` lists (request index, first flat row) for every block
+// of 64 flat rows; see the file comment.  window = 0 means all keys.
+extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
+    const void* q, const void* kpool, const void* vpool, void* out, const int* block_table, int table_stride,
+    const int* seq_q_start, const int* seq_q_len, const int* seq_pos0, const int* work, int n_work, int H, int KV,
+    int hd, int ps, int window, float scale, hipStream_t stream) {
+    MS_REQUIRE(n_work > 0, "attention: no work");
+    MS_REQUIRE(hd % 16 == 0 && hd > 0 && hd <= HDT, "attention: head size %d does not fit this tile of %d", hd, HDT);
+    MS_REQUIRE(KV > 0 && H % KV == 0, "attention: %d heads are not a multiple of %d key/value heads", H, KV);
+    MS_REQUIRE(ps % 16 == 0 && ps > 0, "attention: page size %d must be a multiple of 16", ps);
+    MS_REQUIRE(window >= 0, "attention: window %d", window);
+    AttnArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, (elem_t*)out, block_table, seq_q_start,
+               seq_q_len, seq_pos0, work, table_stride, H, KV, hd, ps, window, scale};
+    hipLaunchKernelGGL(paged_attention_kernel, dim3((unsigned)n_work, (unsigned)KV), dim3(256), 0, stream, a);
+    return check_launch("paged_attention");
+}
+
+extern "C" int MS_CAT(ms_attention_rows_per_block_nd, MS_ATTN_ND)() { return ROWS_PER_BLOCK; }

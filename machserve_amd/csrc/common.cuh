@@ -1,0 +1,141 @@
+// Shared definitions of the gfx950 kernels: element type of this build, MFMA wrappers,
+// wave reductions and the error channel of the extern "C" entry points.
+//
+// One library is built per element type: MS_ELEM_BF16 (bfloat16 storage, 32-bit
+// accumulation) or MS_ELEM_F32 (everything in true 32-bit; its matrix products use the
+// full-precision v_mfma_f32_16x16x4_f32, never a reduced-precision mode).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#if defined(MS_ELEM_BF16) == defined(MS_ELEM_F32)
+#error "define exactly one of MS_ELEM_BF16, MS_ELEM_F32"
+#endif
+
+namespace ms {
+
+constexpr int WAVE = 64;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// ---- element type ---------------------------------------------------------------
+#ifdef MS_ELEM_BF16
+typedef __bf16 elem_t;
+constexpr bool kBf16 = true;
+#else
+typedef float elem_t;
+constexpr bool kBf16 = false;
+#endif
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(__bf16 v) { return (float)v; }
+
+// Round-to-nearest-even conversion of the compiler's own __bf16 cast.
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ __bf16 from_f32<__bf16>(float v) { return (__bf16)v; }
+
+// A fragment is 8 consecutive elements along the reduction dimension of one row of an
+// operand: for lane l of a wave, row l % 16 and elements (l / 16) * 8 .. + 8 of a chunk of
+// 32.  Both operands of a product use the same split, so the sum over the chunk is
+// complete whatever order the hardware takes the elements in.
+struct alignas(16) Frag {
+#ifdef MS_ELEM_BF16
+    bf16x8_t v;
+#else
+    float v[8];
+#endif
+};
+
+__device__ __forceinline__ Frag frag_zero() {
+    Frag f;
+#ifdef MS_ELEM_BF16
+    for (int i = 0; i < 8; ++i) f.v[i] = (__bf16)0.0f;
+#else
+    for (int i = 0; i < 8; ++i) f.v[i] = 0.0f;
+#endif
+    return f;
+}
+
+// Load 8 consecutive elements (16-byte aligned for bf16, 32-byte for float).
+__device__ __forceinline__ Frag frag_load(const elem_t* p) {
+    Frag f;
+#ifdef MS_ELEM_BF16
+    f.v = *reinterpret_cast<const bf16x8_t*>(p);
+#else
+    const f32x4* q = reinterpret_cast<const f32x4*>(p);
+    f32x4 a = q[0], b = q[1];
+    f.v[0] = a[0]; f.v[1] = a[1]; f.v[2] = a[2]; f.v[3] = a[3];
+    f.v[4] = b[0]; f.v[5] = b[1]; f.v[6] = b[2]; f.v[7] = b[3];
+#endif
+    return f;
+}
+
+__device__ __forceinline__ void frag_store(elem_t* p, const Frag& f) {
+#ifdef MS_ELEM_BF16
+    *reinterpret_cast<bf16x8_t*>(p) = f.v;
+#else
+    f32x4* q = reinterpret_cast<f32x4*>(p);
+    f32x4 a = {f.v[0], f.v[1], f.v[2], f.v[3]}, b = {f.v[4], f.v[5], f.v[6], f.v[7]};
+    q[0] = a; q[1] = b;
+#endif
+}
+
+// acc[16x16] += A[16 rows x 32] * B[16 cols x 32]^T, both given as fragments.
+// Result layout: lane l holds rows (l / 16) * 4 + i (i = 0..3) of column l % 16.
+__device__ __forceinline__ void mma_16x16x32(f32x4& acc, const Frag& a, const Frag& b) {
+#ifdef MS_ELEM_BF16
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
+#else
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v[i], b.v[i], acc, 0, 0, 0);
+#endif
+}
+
+// ---- reductions -----------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}
+
+// Sum over a block of NT threads (NT a multiple of 64, at most 1024); every thread gets
+// the result.  `scratch` holds at least NT / 64 floats.  The order of the partial sums is
+// fixed, so the result does not depend on timing.
+template <int NT> __device__ __forceinline__ float block_sum(float v, float* scratch) {
+    v = wave_sum(v);
+    const int w = threadIdx.x / WAVE;
+    __syncthreads();
+    if ((threadIdx.x & (WAVE - 1)) == 0) scratch[w] = v;
+    __syncthreads();
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < NT / WAVE; ++i) t += scratch[i];
+    return t;
+}
+
+// ---- error channel --------------------------------------------------------------
+// Entry points return 0 on success; otherwise ms_last_error() describes the refusal.
+void set_error(const char* fmt, ...);
+int check_launch(const char* what);
+
+#define MS_REQUIRE(cond, ...)            \
+    do {                                 \
+        if (!(cond)) {                   \
+            ::ms::set_error(__VA_ARGS__); \
+            return 1;                    \
+        }                                \
+    } while (0)
+
+__host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+}  // namespace ms

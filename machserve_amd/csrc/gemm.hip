@@ -1,0 +1,199 @@
+// out[M, N] = A[M, K] * W[N, K]^T on the matrix cores, with the epilogue fused:
+// bias add, residual accumulation into the 32-bit stream, or SiLU(gate) * up.
+//
+// Role in the reference: hipBLAS Sgemm / GemmEx plus separate add_bias, add and silu_mul
+// kernels (crates/mach-model/src/kernels.rs:5772-5798, 6416-6455, 131-160).
+//
+// Both operands are contiguous along K, so a 16x32 MFMA fragment of either is "row
+// l % 16, elements (l / 16) * 8 .. + 8": tiles go global -> registers -> LDS (padded rows,
+// conflict-free 16-byte reads) -> fragments.  Two LDS buffers, one barrier per K step.
+// Every output element is the sum over K in steps of 32 in ascending order whatever the
+// tile shape or the number of rows, so a row's result does not depend on its batch.
+#include "common.cuh"
+
+namespace ms {
+
+constexpr int BK = 32;
+#ifdef MS_ELEM_BF16
+constexpr int EPC = 8;   // elements per 16-byte chunk
+constexpr int KPAD = 8;  // row padding in elements: 80-byte rows
+#else
+constexpr int EPC = 4;
+constexpr int KPAD = 4;  // 144-byte rows
+#endif
+constexpr int LDS_LD = BK + KPAD;
+constexpr int CPR = BK / EPC;  // chunks per tile row
+
+enum EpiKind { EPI_STORE_F32 = 0, EPI_STORE_ELEM = 1, EPI_RESIDUAL = 2, EPI_SWIGLU = 3 };
+
+struct EpiArgs {
+    void* out;          // [M, ldo]
+    const float* bias;  // [N] or null
+    int ldo;
+    int n_out;          // SWIGLU: number of output columns (intermediate size)
+};
+
+__device__ __forceinline__ float silu_f(float g) {
+#ifdef MS_ELEM_BF16
+    return g / (1.0f + __expf(-g));
+#else
+    return g / (1.0f + expf(-g));
+#endif
+}
+
+template <int BM, int BN, int WM, int WN, int EPI>
+__global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A, const elem_t* __restrict__ W,
+                                                   int M, int N, int K, EpiArgs ep) {
+    static_assert(WM * WN == 4, "four waves");
+    constexpr int TM = BM / WM / 16, TN = BN / WN / 16;
+    constexpr int A_CHUNKS = BM * CPR / 256, W_CHUNKS = BN * CPR / 256;
+    static_assert(BM * CPR % 256 == 0 && BN * CPR % 256 == 0, "tile loads divide over the block");
+    __shared__ __attribute__((aligned(16))) elem_t As[2][BM * LDS_LD];
+    __shared__ __attribute__((aligned(16))) elem_t Ws[2][BN * LDS_LD];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int tiles_m = ceil_div(M, BM);
+    const int m0 = (blockIdx.x % tiles_m) * BM, n0 = (blockIdx.x / tiles_m) * BN;
+    const int r16 = lane & 15, grp = lane >> 4;
+
+    u32x4 ra[A_CHUNKS], rw[W_CHUNKS];
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) {
+            const int c = tid + i * 256, row = c / CPR, kk = k0 + (c % CPR) * EPC;
+            u32x4 v = {0, 0, 0, 0};
+            if (m0 + row < M && kk < K) v = *reinterpret_cast<const u32x4*>(A + (size_t)(m0 + row) * K + kk);
+            ra[i] = v;
+        }
+#pragma unroll
+        for (int i = 0; i < W_CHUNKS; ++i) {
+            const int c = tid + i * 256, row = c / CPR, kk = k0 + (c % CPR) * EPC;
+            u32x4 v = {0, 0, 0, 0};
+            if (n0 + row < N && kk < K) v = *reinterpret_cast<const u32x4*>(W + (size_t)(n0 + row) * K + kk);
+            rw[i] = v;
+        }
+    };
+    auto store_lds = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) {
+            const int c = tid + i * 256, row = c / CPR, cc = c % CPR;
+            *reinterpret_cast<u32x4*>(&As[buf][row * LDS_LD + cc * EPC]) = ra[i];
+        }
+#pragma unroll
+        for (int i = 0; i < W_CHUNKS; ++i) {
+            const int c = tid + i * 256, row = c / CPR, cc = c % CPR;
+            *reinterpret_cast<u32x4*>(&Ws[buf][row * LDS_LD + cc * EPC]) = rw[i];
+        }
+    };
+
+    f32x4 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    const int nk = ceil_div(K, BK);
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) load_global((kt + 1) * BK);
+        Frag fa[TM], fb[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[i] = frag_load(&As[buf][(wm * (BM / WM) + i * 16 + r16) * LDS_LD + grp * 8]);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[j] = frag_load(&Ws[buf][(wn * (BN / WN) + j * 16 + r16) * LDS_LD + grp * 8]);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) mma_16x16x32(acc[i][j], fa[i], fb[j]);
+        if (kt + 1 < nk) store_lds(buf ^ 1);
+        __syncthreads();
+    }
+
+    // Epilogue.  Lane holds rows grp * 4 + i of column r16 in each 16x16 tile.
+    const int row_base = m0 + wm * (BM / WM) + grp * 4;
+    const int col_base = n0 + wn * (BN / WN) + r16;
+    if constexpr (EPI == EPI_SWIGLU) {
+        static_assert(TN % 2 == 0, "gate and up tiles come in pairs");
+        elem_t* out = reinterpret_cast<elem_t*>(ep.out);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; j += 2) {
+                const int col = (col_base + j * 16 - r16) / 2 + r16;  // tiles 2t, 2t+1 -> output tile t
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int row = row_base + i * 16 + e;
+                    if (row < M && col < ep.n_out)
+                        out[(size_t)row * ep.ldo + col] = from_f32<elem_t>(silu_f(acc[i][j][e]) * acc[i][j + 1][e]);
+                }
+            }
+    } else {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int col = col_base + j * 16;
+                if (col >= N) continue;
+                const float b = ep.bias ? ep.bias[col] : 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int row = row_base + i * 16 + e;
+                    if (row >= M) continue;
+                    const size_t o = (size_t)row * ep.ldo + col;
+                    const float v = acc[i][j][e] + b;
+                    if constexpr (EPI == EPI_STORE_F32) reinterpret_cast<float*>(ep.out)[o] = v;
+                    else if constexpr (EPI == EPI_STORE_ELEM) reinterpret_cast<elem_t*>(ep.out)[o] = from_f32<elem_t>(v);
+                    else reinterpret_cast<float*>(ep.out)[o] += v;  // residual stream, 32-bit
+                }
+            }
+    }
+}
+
+template <int EPI>
+static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, EpiArgs ep, hipStream_t stream) {
+    MS_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: empty problem M=%d N=%d K=%d", M, N, K);
+    MS_REQUIRE(K % 8 == 0, "gemm: the reduction size K=%d must be a multiple of 8", K);
+    MS_REQUIRE((reinterpret_cast<uintptr_t>(A) & 15) == 0 && (reinterpret_cast<uintptr_t>(W) & 15) == 0,
+               "gemm: operands must be 16-byte aligned");
+#ifdef MS_ELEM_BF16
+    if (M > 64) {
+        const long blocks = (long)ceil_div(M, 128) * ceil_div(N, 128);
+        hipLaunchKernelGGL((gemm_kernel<128, 128, 2, 2, EPI>), dim3((unsigned)blocks), dim3(256), 0, stream, A, W, M, N, K, ep);
+        return check_launch("gemm 128x128");
+    }
+#endif
+    const long blocks = (long)ceil_div(M, 64) * ceil_div(N, 64);
+    hipLaunchKernelGGL((gemm_kernel<64, 64, 2, 2, EPI>), dim3((unsigned)blocks), dim3(256), 0, stream, A, W, M, N, K, ep);
+    return check_launch("gemm 64x64");
+}
+
+}  // namespace ms
+
+using namespace ms;
+
+// out[M, N] = a[M, K] w[N, K]^T (+ bias[N]); out is float when out_f32 != 0, else the element type.
+extern "C" int ms_linear(const void* a, const void* w, const float* bias, void* out, int out_f32, int M, int N, int K,
+                         hipStream_t stream) {
+    EpiArgs ep{out, bias, N, N};
+    if (out_f32) return launch_gemm<EPI_STORE_F32>((const elem_t*)a, (const elem_t*)w, M, N, K, ep, stream);
+    return launch_gemm<EPI_STORE_ELEM>((const elem_t*)a, (const elem_t*)w, M, N, K, ep, stream);
+}
+
+// x[M, N] += a[M, K] w[N, K]^T, x being the 32-bit residual stream.
+extern "C" int ms_linear_residual(const void* a, const void* w, float* x, int M, int N, int K, hipStream_t stream) {
+    EpiArgs ep{x, nullptr, N, N};
+    return launch_gemm<EPI_RESIDUAL>((const elem_t*)a, (const elem_t*)w, M, N, K, ep, stream);
+}
+
+// out[M, I] = silu(a g^T) * (a u^T) where w holds gate and up rows interleaved in blocks of 16:
+// rows [32 t, 32 t + 16) are gate rows [16 t, 16 t + 16), rows [32 t + 16, 32 t + 32) the same
+// up rows; w has 2 * ceil16(I) rows, the padding rows being zero.
+extern "C" int ms_linear_swiglu(const void* a, const void* w, void* out, int M, int I, int K, hipStream_t stream) {
+    const int n = 2 * ceil_div(I, 16) * 16;
+    EpiArgs ep{out, nullptr, I, I};
+    return launch_gemm<EPI_SWIGLU>((const elem_t*)a, (const elem_t*)w, M, n, K, ep, stream);
+}

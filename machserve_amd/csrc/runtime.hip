@@ -1,0 +1,32 @@
+// Error channel of the extern "C" entry points: a refused call returns non-zero and
+// leaves its reason here.  Role of `check` in crates/mach-kernel-sys/src/hip.rs:370.
+#include "common.cuh"
+#include <cstdarg>
+#include <cstdio>
+
+namespace ms {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+        return 2;
+    }
+    return 0;
+}
+
+}  // namespace ms
+
+extern "C" const char* ms_last_error() { return ms::g_error; }
+
+// 1 for the bfloat16 build, 0 for the 32-bit build.
+extern "C" int ms_elem_is_bf16() { return ms::kBf16 ? 1 : 0; }

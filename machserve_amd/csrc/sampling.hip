@@ -1,0 +1,212 @@
+// Token sampling on the GPU, one block per row of logits.
+//
+// Algorithm of the reference's sampler (crates/mach-model/src/sampling.rs:113-402 and its
+// CPU mirror 1169-1274): one SplitMix64 draw per row per call, also when greedy
+// (finalizer of the state, then state += golden ratio; u = top 24 bits / 2^24);
+// temperature <= 0 -> smallest index among the maxima; else p = exp((x - max) / T),
+// top-k as a threshold on the raw logit found by 30 bisection steps between the row's
+// minimum and maximum, top-p as a probability cut found by 30 bisection steps so that the
+// kept mass is >= p * total, then target = u * allowed mass and a walk in index order to
+// the first token whose cumulative mass exceeds the target.
+//
+// The walk here is in true index order: thread i owns the contiguous segment i of the row,
+// the segment masses are scanned in order, and the owner of the segment that holds the
+// target walks it.
+#include "common.cuh"
+
+namespace ms {
+
+constexpr int ST = 256;
+
+__device__ __forceinline__ unsigned long long mix64(unsigned long long z) {
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+    return z ^ (z >> 31);
+}
+
+struct SampleArgs {
+    const float* logits;  // [W, vocab]
+    const float* temperature;
+    const int* top_k;
+    const float* top_p;
+    unsigned long long* state;  // [W], advanced by one step
+    int* out_token;
+    float* out_logprob;
+    int vocab;
+};
+
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+    v = wave_max(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float t = scratch[0];
+    for (int i = 1; i < ST / WAVE; ++i) t = fmaxf(t, scratch[i]);
+    return t;
+}
+
+__global__ __launch_bounds__(ST) void sample_kernel(SampleArgs a) {
+    __shared__ float scratch[ST / WAVE];
+    __shared__ float seg[ST], seg_pref[ST];
+    __shared__ float s_u;
+    __shared__ int s_idx[ST / WAVE];
+    __shared__ float s_val[ST / WAVE];
+    __shared__ int s_found;
+    const int r = blockIdx.x, tid = threadIdx.x, V = a.vocab;
+    const float* row = a.logits + (size_t)r * V;
+    const float T = a.temperature[r];
+
+    if (tid == 0) {
+        unsigned long long st = a.state[r];
+        const unsigned long long z = mix64(st);
+        a.state[r] = st + 0x9E3779B97F4A7C15ULL;
+        s_u = (float)(z >> 40) * (1.0f / 16777216.0f);
+        s_found = -1;
+    }
+    __syncthreads();
+
+    const int seg_len = ceil_div(V, ST);
+    const int i0 = min(V, tid * seg_len), i1 = min(V, i0 + seg_len);
+
+    if (T <= 0.0f) {
+        // smallest index among the maxima: segments are in index order, strict > inside
+        float best = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int i = i0; i < i1; ++i)
+            if (bi == 0x7fffffff || row[i] > best) { best = row[i]; bi = i; }
+        // wave reduce (value desc, index asc)
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(best, o, WAVE);
+            const int oi = __shfl_xor(bi, o, WAVE);
+            if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+        }
+        if ((tid & 63) == 0) { s_val[tid >> 6] = best; s_idx[tid >> 6] = bi; }
+        __syncthreads();
+        if (tid == 0) {
+            for (int w = 1; w < ST / WAVE; ++w)
+                if (s_val[w] > best || (s_val[w] == best && s_idx[w] < bi)) { best = s_val[w]; bi = s_idx[w]; }
+            a.out_token[r] = bi;
+            a.out_logprob[r] = 0.0f;
+        }
+        return;
+    }
+
+    float mx = -INFINITY, mn = INFINITY;
+    for (int i = tid; i < V; i += ST) {
+        const float x = row[i];
+        mx = fmaxf(mx, x);
+        mn = fminf(mn, x);
+    }
+    const float maxv = block_max(mx, scratch);
+    const float minv = -block_max(-mn, scratch);
+    const float inv_t = 1.0f / T;
+    const int k = a.top_k[r];
+    const int k_eff = (k > 0 && k < V) ? k : 0;
+
+    float topk_thr = -INFINITY;
+    if (k_eff > 0) {
+        float lo = minv, hi = maxv;
+        for (int it = 0; it < 30; ++it) {
+            const float mid = (lo + hi) * 0.5f;
+            float cnt = 0.f;
+            for (int i = tid; i < V; i += ST) cnt += row[i] > mid ? 1.f : 0.f;
+            cnt = block_sum<ST>(cnt, scratch);
+            if (cnt >= (float)k_eff) lo = mid; else hi = mid;
+        }
+        topk_thr = hi;
+    }
+
+    // total mass, summed segment by segment in index order
+    float part = 0.f;
+    for (int i = i0; i < i1; ++i) part += expf((row[i] - maxv) * inv_t);
+    const float s_tot = block_sum<ST>(part, scratch);
+
+    const float top_p = a.top_p[r];
+    const bool use_topp = top_p < 1.0f;
+    float cut = 0.f;
+    if (use_topp) {
+        float lo = 0.f, hi = 1.f;
+        for (int it = 0; it < 30; ++it) {
+            const float mid = (lo + hi) * 0.5f;
+            float acc = 0.f;
+            for (int i = i0; i < i1; ++i) {
+                const float pr = expf((row[i] - maxv) * inv_t);
+                if (pr >= mid) acc += pr;
+            }
+            acc = block_sum<ST>(acc, scratch);
+            if (acc >= top_p * s_tot) lo = mid; else hi = mid;
+        }
+        cut = lo;
+    }
+
+    auto allowed = [&](float x, float pr) { return (k_eff == 0 || x >= topk_thr) && (!use_topp || pr >= cut); };
+
+    float mass = 0.f;
+    for (int i = i0; i < i1; ++i) {
+        const float pr = expf((row[i] - maxv) * inv_t);
+        if (allowed(row[i], pr)) mass += pr;
+    }
+    seg[tid] = mass;
+    __syncthreads();
+    if (tid == 0) {
+        float acc = 0.f;
+        for (int j = 0; j < ST; ++j) { seg_pref[j] = acc; acc += seg[j]; }
+        scratch[0] = acc;
+    }
+    __syncthreads();
+    const float tot = scratch[0];
+    const float target = s_u * tot;
+    if (seg_pref[tid] <= target && target < seg_pref[tid] + seg[tid]) {
+        float acc = seg_pref[tid];
+        for (int i = i0; i < i1; ++i) {
+            const float pr = expf((row[i] - maxv) * inv_t);
+            if (allowed(row[i], pr)) {
+                acc += pr;
+                if (acc > target) { s_found = i; break; }  // segments are disjoint: one owner
+            }
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int found = s_found;
+        if (found < 0) {
+            // rounding at the top of the mass: the last allowed token, as a walk that never
+            // exceeds the target ends there
+            for (int i = V - 1; i >= 0 && found < 0; --i) {
+                const float pr = expf((row[i] - maxv) * inv_t);
+                if (allowed(row[i], pr)) found = i;
+            }
+            if (found < 0) found = 0;
+        }
+        a.out_token[r] = found;
+        a.out_logprob[r] = (row[found] - maxv) * inv_t - logf(tot);
+    }
+}
+
+// logits[row_of[e], token[e]] += delta[e]: penalties and biases, merged per (row, token) on the host
+__global__ void logit_edit_kernel(float* logits, int vocab, const int* row_of, const int* token, const float* delta,
+                                  int n) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < n && token[e] >= 0 && token[e] < vocab) logits[(size_t)row_of[e] * vocab + token[e]] += delta[e];
+}
+
+}  // namespace ms
+
+using namespace ms;
+
+extern "C" int ms_sample(const float* logits, const float* temperature, const int* top_k, const float* top_p,
+                         unsigned long long* state, int* out_token, float* out_logprob, int rows, int vocab,
+                         hipStream_t stream) {
+    MS_REQUIRE(rows > 0 && vocab > 0, "sample: empty problem rows=%d vocab=%d", rows, vocab);
+    SampleArgs a{logits, temperature, top_k, top_p, state, out_token, out_logprob, vocab};
+    hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(ST), 0, stream, a);
+    return check_launch("sample");
+}
+
+extern "C" int ms_logit_edit(float* logits, int vocab, const int* row_of, const int* token, const float* delta, int n,
+                             hipStream_t stream) {
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(logit_edit_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, stream, logits, vocab, row_of, token,
+                       delta, n);
+    return check_launch("logit_edit");
+}

@@ -1,0 +1,230 @@
+"""The one boundary between Python and the HIP libraries (role of ``mach-kernel-sys`` in the
+reference, ``crates/mach-kernel-sys/src/hip.rs``): torch tensors own the memory, every
+operand is checked on the host against what the kernel and its grid assume, and the raw
+pointers go to the ``extern "C"`` entry points on torch's current stream.
+
+There is no fallback: without a GPU or without the libraries, construction raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build
+
+_c_int, _c_float, _c_void = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return _c_void(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return _c_void(torch.cuda.current_stream().cuda_stream)
+
+
+class HipOps:
+    """Kernels of one element type: ``torch.bfloat16`` (serving) or ``torch.float32`` (true 32-bit)."""
+
+    def __init__(self, dtype: torch.dtype, device: str = "cuda:0"):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise KernelError(f"no kernels for element type {dtype}; bfloat16 and float32 are built")
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible: the HIP kernels have no CPU fallback")
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.elem = "bf16" if dtype == torch.bfloat16 else "f32"
+        self._core = self._load(build.ensure_library("core", self.elem))
+        self._attn = {}
+
+    def _load(self, path: str):
+        try:
+            lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelError(f"cannot load {path}: {e}") from None
+        lib.ms_last_error.restype = ctypes.c_char_p
+        return lib
+
+    def _check(self, lib, rc: int):
+        if rc != 0:
+            raise KernelError(lib.ms_last_error().decode())
+
+    def _want(self, t: torch.Tensor, dtype, name: str, *shape):
+        if t.device.type != "cuda" or t.dtype != dtype or not t.is_contiguous():
+            raise KernelError(f"{name}: expected a contiguous {dtype} GPU tensor, got {t.dtype} on {t.device}"
+                              f"{'' if t.is_contiguous() else ' (not contiguous)'}")
+        if shape and tuple(t.shape) != tuple(shape):
+            raise KernelError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
+
+    # ------------------------------------------------------------------ elementwise
+    def embed(self, tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+        T, (V, d) = tokens.numel(), table.shape
+        self._want(tokens, torch.int32, "embed tokens", T)
+        self._want(table, self.dtype, "embed table")
+        x = torch.empty((T, d), dtype=torch.float32, device=table.device)
+        self._check(self._core, self._core.ms_embed(_ptr(tokens), _ptr(table), _ptr(x), _c_int(T), _c_int(d), _stream()))
+        return x
+
+    def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, rows: Optional[torch.Tensor] = None,
+                out_f32: bool = False) -> torch.Tensor:
+        T, d = x.shape
+        self._want(x, torch.float32, "rmsnorm input")
+        self._want(weight, torch.float32, "rmsnorm weight", d)
+        n = T
+        if rows is not None:
+            self._want(rows, torch.int32, "rmsnorm rows")
+            n = rows.numel()
+        out = torch.empty((n, d), dtype=torch.float32 if out_f32 else self.dtype, device=x.device)
+        self._check(self._core, self._core.ms_rmsnorm(_ptr(x), _ptr(rows), _ptr(weight), _ptr(out), _c_int(int(out_f32)),
+                                                      _c_int(n), _c_int(d), _c_float(eps), _stream()))
+        return out
+
+    def rope_kv_write(self, qkv: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[torch.Tensor],
+                      slot_map: Optional[torch.Tensor], kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor],
+                      H: int, KV: int, hd: int, page_size: int) -> torch.Tensor:
+        T, stride = qkv.shape
+        self._want(qkv, torch.float32, "rope qkv")
+        self._want(positions, torch.int32, "rope positions", T)
+        if inv_freq is not None:
+            self._want(inv_freq, torch.float32, "rope inv_freq", hd // 2)
+        if slot_map is not None:
+            self._want(slot_map, torch.int32, "rope slot_map", T)
+            pages = kpool.shape[0]
+            self._want(kpool, self.dtype, "key pool", pages, KV, page_size, hd)
+            self._want(vpool, self.dtype, "value pool", pages, KV, hd, page_size)
+        q = torch.empty((T, H * hd), dtype=self.dtype, device=qkv.device)
+        self._check(self._core, self._core.ms_rope_kv_write(
+            _ptr(qkv), _c_int(stride), _ptr(positions), _ptr(inv_freq), _ptr(slot_map), _ptr(q), _ptr(kpool), _ptr(vpool),
+            _c_int(T), _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), _stream()))
+        return q
+
+    # ------------------------------------------------------------------ matrix products
+    def _mm_operands(self, a: torch.Tensor, w: torch.Tensor, what: str):
+        self._want(a, self.dtype, f"{what} input")
+        self._want(w, self.dtype, f"{what} weight")
+        M, K = a.shape
+        if w.shape[1] != K:
+            raise KernelError(f"{what}: input has {K} columns, weight has {w.shape[1]}")
+        return M, w.shape[0], K
+
+    def linear(self, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+               out_f32: bool = False) -> torch.Tensor:
+        """``a @ w.T (+ bias)``; 32-bit output on request (projections that feed the rotation, logits)."""
+        M, N, K = self._mm_operands(a, w, "linear")
+        if bias is not None:
+            self._want(bias, torch.float32, "linear bias", N)
+        out = torch.empty((M, N), dtype=torch.float32 if out_f32 else self.dtype, device=a.device)
+        self._check(self._core, self._core.ms_linear(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), _c_int(int(out_f32)),
+                                                     _c_int(M), _c_int(N), _c_int(K), _stream()))
+        return out
+
+    def linear_residual(self, a: torch.Tensor, w: torch.Tensor, x: torch.Tensor) -> None:
+        """``x += a @ w.T`` in the 32-bit residual stream."""
+        M, N, K = self._mm_operands(a, w, "linear_residual")
+        self._want(x, torch.float32, "residual stream", M, N)
+        self._check(self._core, self._core.ms_linear_residual(_ptr(a), _ptr(w), _ptr(x), _c_int(M), _c_int(N), _c_int(K),
+                                                              _stream()))
+
+    def linear_swiglu(self, a: torch.Tensor, w_gate_up: torch.Tensor, intermediate: int) -> torch.Tensor:
+        """``silu(a @ gate.T) * (a @ up.T)`` with gate and up rows interleaved in blocks of 16
+        (see :func:`interleave_gate_up`)."""
+        M, N, K = self._mm_operands(a, w_gate_up, "linear_swiglu")
+        if N != 2 * ((intermediate + 15) // 16) * 16:
+            raise KernelError(f"linear_swiglu: interleaved weight has {N} rows for intermediate size {intermediate}")
+        out = torch.empty((M, intermediate), dtype=self.dtype, device=a.device)
+        self._check(self._core, self._core.ms_linear_swiglu(_ptr(a), _ptr(w_gate_up), _ptr(out), _c_int(M),
+                                                            _c_int(intermediate), _c_int(K), _stream()))
+        return out
+
+    # ------------------------------------------------------------------ attention
+    def _attention_lib(self, hd: int):
+        nd = build.attention_tile_for(hd)
+        if nd not in self._attn:
+            lib = self._load(build.ensure_library("attention", self.elem, nd))
+            self._attn[nd] = (lib, getattr(lib, f"ms_paged_attention_nd{nd}"),
+                              getattr(lib, f"ms_attention_rows_per_block_nd{nd}")())
+        return self._attn[nd]
+
+    def attention_rows_per_block(self, hd: int) -> int:
+        return self._attention_lib(hd)[2]
+
+    def paged_attention(self, q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
+                        seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_pos0: torch.Tensor,
+                        work: torch.Tensor, H: int, KV: int, hd: int, page_size: int, window: Optional[int],
+                        scale: float) -> torch.Tensor:
+        lib, fn, _ = self._attention_lib(hd)
+        T = q.shape[0]
+        self._want(q, self.dtype, "attention q", T, H * hd)
+        pages = kpool.shape[0]
+        self._want(kpool, self.dtype, "key pool", pages, KV, page_size, hd)
+        self._want(vpool, self.dtype, "value pool", pages, KV, hd, page_size)
+        S = seq_q_start.numel()
+        self._want(block_table, torch.int32, "block table")
+        if block_table.dim() != 2 or block_table.shape[0] != S:
+            raise KernelError(f"attention: block table {tuple(block_table.shape)} for {S} requests")
+        for t, n in ((seq_q_start, "seq_q_start"), (seq_q_len, "seq_q_len"), (seq_pos0, "seq_pos0")):
+            self._want(t, torch.int32, n, S)
+        self._want(work, torch.int32, "attention work")
+        if work.dim() != 2 or work.shape[1] != 2 or work.shape[0] == 0:
+            raise KernelError(f"attention: work list of shape {tuple(work.shape)}")
+        out = torch.empty((T, H * hd), dtype=self.dtype, device=q.device)
+        self._check(lib, fn(_ptr(q), _ptr(kpool), _ptr(vpool), _ptr(out), _ptr(block_table), _c_int(block_table.shape[1]),
+                            _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_pos0), _ptr(work), _c_int(work.shape[0]),
+                            _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), _c_int(window or 0), _c_float(scale),
+                            _stream()))
+        return out
+
+    # ------------------------------------------------------------------ sampling
+    def sample(self, logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+               state: torch.Tensor):
+        """One token per row; ``state`` (int64 SplitMix64 states) advances in place.
+        Returns ``(tokens int32, logprobs float32)``."""
+        W, V = logits.shape
+        self._want(logits, torch.float32, "sample logits")
+        self._want(temperature, torch.float32, "sample temperature", W)
+        self._want(top_k, torch.int32, "sample top_k", W)
+        self._want(top_p, torch.float32, "sample top_p", W)
+        self._want(state, torch.int64, "sample state", W)
+        tok = torch.empty(W, dtype=torch.int32, device=logits.device)
+        lp = torch.empty(W, dtype=torch.float32, device=logits.device)
+        self._check(self._core, self._core.ms_sample(_ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p),
+                                                     _ptr(state), _ptr(tok), _ptr(lp), _c_int(W), _c_int(V), _stream()))
+        return tok, lp
+
+    def logit_edit(self, logits: torch.Tensor, row_of: torch.Tensor, token: torch.Tensor, delta: torch.Tensor) -> None:
+        """``logits[row_of[e], token[e]] += delta[e]`` (penalties and biases merged on the host)."""
+        n = row_of.numel()
+        self._want(logits, torch.float32, "logit_edit logits")
+        self._want(row_of, torch.int32, "logit_edit rows", n)
+        self._want(token, torch.int32, "logit_edit tokens", n)
+        self._want(delta, torch.float32, "logit_edit deltas", n)
+        self._check(self._core, self._core.ms_logit_edit(_ptr(logits), _c_int(logits.shape[1]), _ptr(row_of), _ptr(token),
+                                                         _ptr(delta), _c_int(n), _stream()))
+
+
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """``[2 * ceil16(I), d]``: blocks of 16 gate rows and the same 16 up rows alternate, zero
+    rows pad the last block; the layout :meth:`HipOps.linear_swiglu` multiplies by."""
+    I, d = gate.shape
+    Ip = (I + 15) // 16 * 16
+    g = torch.zeros((Ip, d), dtype=gate.dtype, device=gate.device)
+    u = torch.zeros((Ip, d), dtype=gate.dtype, device=gate.device)
+    g[:I] = gate
+    u[:I] = up
+    return torch.stack([g.view(Ip // 16, 16, d), u.view(Ip // 16, 16, d)], dim=1).reshape(2 * Ip, d).contiguous()
+
+
+_OPS = {}
+
+
+def get_ops(dtype: torch.dtype, device: str = "cuda:0") -> HipOps:
+    key = (dtype, device)
+    if key not in _OPS:
+        _OPS[key] = HipOps(dtype, device)
+    return _OPS[key]

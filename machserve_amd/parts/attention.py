@@ -1,0 +1,84 @@
+"""Grouped-query attention over the paged cache.
+
+Per step (``crates/mach-model/src/batched.rs:3566-3679, 3819-3878, 4022-4031``):
+q/k/v projection in one product with the biases in its epilogue, rotation of q and k fused
+with the write of k and v into their pages, attention of every row over its request's
+cache, output projection accumulated into the 32-bit stream.  Bias tensors are optional
+and their presence decides (``crates/mach-model/src/weights.rs:30-31``).
+"""
+from __future__ import annotations
+
+import torch
+
+from .base import Mixer, PagedKVRequest, SharedKVRequest, TensorDecl
+from .registry import POSITION_ENCODINGS, register_mixer
+
+
+@register_mixer("attention")
+class Attention(Mixer):
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        s = spec
+        if s.heads % s.kv_heads:
+            raise ValueError(f"attention: {s.heads} heads are not a multiple of {s.kv_heads} key/value heads")
+        self.nq, self.nkv = s.heads * s.head_dim, s.kv_heads * s.head_dim
+        self.scale = float(s.head_dim) ** -0.5
+        self.position = POSITION_ENCODINGS.build(s.position, rt) if s.position is not None else None
+        self.writes_cache = s.kv_source is None
+        self.group = None
+        self.kpool = self.vpool = None
+
+    def sub_parts(self):
+        return [self.position] if self.position is not None else []
+
+    def tensor_decls(self):
+        s = self.spec
+        decls = [TensorDecl("q.weight", (self.nq, s.hidden)), TensorDecl("o.weight", (s.hidden, self.nq)),
+                 TensorDecl("q.bias", (self.nq,), "vector", optional=True)]
+        if self.writes_cache:
+            decls += [TensorDecl("k.weight", (self.nkv, s.hidden)), TensorDecl("v.weight", (self.nkv, s.hidden)),
+                      TensorDecl("k.bias", (self.nkv,), "vector", optional=True),
+                      TensorDecl("v.bias", (self.nkv,), "vector", optional=True)]
+        return decls
+
+    def load(self, t):
+        names = ["q", "k", "v"] if self.writes_cache else ["q"]
+        self.w_qkv = torch.cat([t[n + ".weight"] for n in names], dim=0).contiguous()
+        if any(t.get(n + ".bias") is not None for n in names):
+            dev = self.w_qkv.device
+            self.b_qkv = torch.cat([t[n + ".bias"] if t.get(n + ".bias") is not None
+                                    else torch.zeros(t[n + ".weight"].shape[0], dtype=torch.float32, device=dev)
+                                    for n in names]).contiguous()
+        else:
+            self.b_qkv = None
+        self.w_o = t["o.weight"]
+
+    def cache_request(self):
+        s = self.spec
+        if not self.writes_cache:
+            return SharedKVRequest(s.kv_source)
+        return PagedKVRequest(s.kv_heads, s.head_dim, s.window)
+
+    def bind_cache(self, binding):
+        self.group, self.kpool, self.vpool = binding.group, binding.kpool, binding.vpool
+
+    def attention_rows_per_token(self):
+        return self.spec.heads // self.spec.kv_heads
+
+    def forward(self, h, x, ctx):
+        s, ops = self.spec, self.rt.ops
+        view = ctx.groups[self.group]
+        qkv = ops.linear(h, self.w_qkv, self.b_qkv, out_f32=True)
+        inv_freq = self.position.rotary_inv_freq() if self.position is not None else None
+        if self.position is not None and inv_freq is None:
+            T = qkv.shape[0]
+            q = qkv[:, :self.nq].unflatten(1, (s.heads, s.head_dim))
+            k = qkv[:, self.nq:self.nq + self.nkv].unflatten(1, (s.kv_heads, s.head_dim)) if self.writes_cache else None
+            self.position.apply(q, k, ctx)
+        q = ops.rope_kv_write(qkv, ctx.positions, inv_freq, view.slot_map if self.writes_cache else None,
+                              self.kpool if self.writes_cache else None, self.vpool if self.writes_cache else None,
+                              s.heads, s.kv_heads, s.head_dim, view.page_size)
+        o = ops.paged_attention(q, self.kpool, self.vpool, view.block_table, ctx.seq_q_start, ctx.seq_q_len,
+                                ctx.seq_pos0, ctx.attention_work[self.attention_rows_per_token()], s.heads, s.kv_heads,
+                                s.head_dim, view.page_size, s.window, self.scale)
+        ops.linear_residual(o, self.w_o, x)

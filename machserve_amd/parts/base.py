@@ -1,0 +1,157 @@
+"""Interfaces of the parts a decoder is put together from.
+
+A part is built from its spec (``config.specs``) and a :class:`Runtime`; it declares the
+tensors it needs by its *own* names, receives them from the loader, and runs on a
+:class:`StepContext`.  A part never looks at the model around it: sizes and constants
+come from its spec, positions and cache addresses from the context.
+
+Adding a part: subclass the matching base class, give it the methods below, and register
+it under a ``kind`` in ``parts.registry``; a spec whose ``kind`` names it is all a model
+needs to use it.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Mapping, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class TensorDecl:
+    """A tensor a part wants.  ``role`` decides how it is kept on the device: a 'matrix'
+    (operand of a matrix product, or the embedding table) in the element type of the
+    run, a 'vector' (norm weight, bias) in float32, a 'table' of integers in int32."""
+    name: str
+    shape: Tuple[int, ...]
+    role: str = "matrix"
+    optional: bool = False
+
+
+@dataclass
+class Runtime:
+    """What a part gets from its surroundings: the device, the element type and the kernels."""
+    device: torch.device
+    dtype: torch.dtype
+    ops: object
+
+
+@dataclass(frozen=True)
+class PagedKVRequest:
+    """A mixer's need of a paged cache: K and V per token, all keys or a window of them."""
+    kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class SharedKVRequest:
+    """A mixer that reads the cache another layer writes."""
+    source_layer: int
+
+
+@dataclass(frozen=True)
+class StateRequest:
+    """A mixer's need of per-request state of fixed size: one tensor ``[slots, *shape]``
+    per entry, zeroed when a request takes the slot."""
+    shapes: Mapping[str, Tuple[int, ...]]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class GroupView:
+    """Addresses of one cache group for the rows and requests of a step."""
+    page_size: int
+    slot_map: torch.Tensor     # int32 [T]: page * page_size + offset where each row's key goes
+    block_table: torch.Tensor  # int32 [S, P]: pages of each request of the step, -1 = none
+
+
+@dataclass
+class StepContext:
+    """Everything about one step that parts may read.  Device tensors are int32.
+
+    Rows are the tokens of the step; requests are listed in the order of their rows, and a
+    request's rows are contiguous and in position order.
+    """
+    n_rows: int
+    n_seqs: int
+    tokens: torch.Tensor        # [T]
+    positions: torch.Tensor     # [T]
+    seq_q_start: torch.Tensor   # [S] first row of each request
+    seq_q_len: torch.Tensor     # [S] number of its rows
+    seq_pos0: torch.Tensor      # [S] position of its first row
+    seq_slot: torch.Tensor      # [S] state slot of each request
+    want_rows: torch.Tensor     # [W] rows whose logits are wanted
+    groups: Dict[str, GroupView] = field(default_factory=dict)
+    attention_work: Dict[int, torch.Tensor] = field(default_factory=dict)  # rows per token -> [n, 2]
+    host: Dict[str, object] = field(default_factory=dict)  # the same lists on the host
+    decode_only: bool = False
+
+
+class Part:
+    def __init__(self, spec, rt: Runtime):
+        self.spec = spec
+        self.rt = rt
+
+    def tensor_decls(self) -> List[TensorDecl]:
+        return []
+
+    def load(self, tensors: Dict[str, Optional[torch.Tensor]]) -> None:
+        """Receive the declared tensors (absent optional ones are None), already on the
+        device in the dtype of their role."""
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None, out_f32: bool = False) -> torch.Tensor:
+        """Normalised copy of the 32-bit stream ``x`` (of its ``rows`` if given), in the element type."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def rotary_inv_freq(self) -> Optional[torch.Tensor]:
+        """``[head_dim / 2]`` inverse frequencies if this is a plain rotation that the fused
+        kernel can apply; None otherwise (then :meth:`apply` is called)."""
+        return None
+
+    def apply(self, q: torch.Tensor, k: Optional[torch.Tensor], ctx: StepContext) -> None:
+        """Encode positions in place into ``q [T, H, hd]`` and ``k [T, KV, hd]`` (float32 views)."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    """Mixes information between positions of one request (attention, or a recurrence)."""
+
+    def cache_request(self):
+        """PagedKVRequest, SharedKVRequest, StateRequest or None."""
+        return None
+
+    def bind_cache(self, binding) -> None:
+        """Receive what the cache manager made for :meth:`cache_request`."""
+
+    def attention_rows_per_token(self) -> Optional[int]:
+        """Query heads per KV head if the mixer needs attention work lists, else None."""
+        return None
+
+    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
+        """Add the mixer's output for the normalised input ``h`` into the stream ``x``."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
+        """Add the feed-forward's output for the normalised input ``h`` into the stream ``x``."""
+        raise NotImplementedError
+
+
+class Block:
+    """An arrangement of a mixer, a feed-forward and their norms around the stream."""
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+
+    def parts(self):
+        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> None:
+        raise NotImplementedError

@@ -1,0 +1,31 @@
+"""Dense gated feed-forward ``down(silu(gate(x)) * up(x))``, activation on the gate branch
+(``crates/mach-model/src/batched.rs:4424-4453``, ``crates/mach-model/src/kernels.rs:131-140``).
+Gate and up are one product whose epilogue applies the activation; down accumulates into
+the 32-bit stream."""
+from __future__ import annotations
+
+from ..kernels.ops import interleave_gate_up
+from .base import FeedForward, TensorDecl
+from .registry import register_feed_forward
+
+
+@register_feed_forward("gated_mlp")
+class GatedMlp(FeedForward):
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        if spec.activation != "silu":
+            raise ValueError(f"gated_mlp: activation {spec.activation!r} is not built (silu only)")
+
+    def tensor_decls(self):
+        s = self.spec
+        return [TensorDecl("gate.weight", (s.intermediate, s.hidden)), TensorDecl("up.weight", (s.intermediate, s.hidden)),
+                TensorDecl("down.weight", (s.hidden, s.intermediate))]
+
+    def load(self, t):
+        self.w_gate_up = interleave_gate_up(t["gate.weight"], t["up.weight"])
+        self.w_down = t["down.weight"]
+
+    def forward(self, h, x, ctx):
+        ops = self.rt.ops
+        a = ops.linear_swiglu(h, self.w_gate_up, self.spec.intermediate)
+        ops.linear_residual(a, self.w_down, x)

@@ -1,0 +1,104 @@
+"""A decoder built from a :class:`ModelSpec`: embedding, blocks chosen layer by layer from
+the registries, final norm, output head.  ``order`` is the list of layers a step runs; it
+may name a layer twice.  Only the rows whose logits are wanted reach the head
+(the reference computes the head for every row, ``crates/mach-model/src/batched.rs:4594-4626``).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..config.specs import ModelSpec
+from .base import Block, Part, Runtime, StepContext, TensorDecl
+from .registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
+
+
+class Embedding(Part):
+    def tensor_decls(self):
+        return [TensorDecl("weight", (self.spec.vocab, self.spec.width), "matrix")]
+
+    def load(self, t):
+        self.weight = t["weight"]
+
+    def forward(self, tokens: torch.Tensor) -> torch.Tensor:
+        return self.rt.ops.embed(tokens, self.weight)
+
+
+class Head(Part):
+    """Output projection; tied to the embedding table when the spec says so, or when it
+    leaves it open and the checkpoint has no head tensor
+    (``crates/mach-model/src/loader.rs:1025-1033``)."""
+
+    def __init__(self, spec, rt, embedding: Embedding):
+        super().__init__(spec, rt)
+        self.embedding = embedding
+        self.weight = None
+
+    def tensor_decls(self):
+        if self.spec.tied is True:
+            return []
+        return [TensorDecl("weight", (self.spec.vocab, self.spec.width), "matrix", optional=self.spec.tied is None)]
+
+    def ignored_tensors(self):
+        """Checkpoint names that may be present without being used."""
+        return [self.spec.tensors.get("weight", "weight")] if self.spec.tied is True else []
+
+    def load(self, t):
+        self.weight = t.get("weight")
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        w = self.weight if self.weight is not None else self.embedding.weight
+        return self.rt.ops.linear(h, w, None, out_f32=True)
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, rt: Runtime):
+        spec.validate()
+        self.spec, self.rt = spec, rt
+        self.embedding = Embedding(spec.embedding, rt)
+        self.blocks: List[Block] = []
+        for layer in spec.layers:
+            block_cls = BLOCKS.get(layer.block)
+            self.blocks.append(block_cls(MIXERS.build(layer.mixer, rt), FEED_FORWARDS.build(layer.feed_forward, rt),
+                                         NORMS.build(layer.mixer_norm, rt), NORMS.build(layer.feed_forward_norm, rt)))
+        self.order = list(spec.order)
+        self.final_norm = NORMS.build(spec.final_norm, rt)
+        self.head = Head(spec.head, rt, self.embedding)
+
+    # ------------------------------------------------------------------ structure
+    def parts(self) -> List[Part]:
+        out: List[Part] = [self.embedding]
+        for b in self.blocks:
+            for p in b.parts():
+                out.append(p)
+                out.extend(getattr(p, "sub_parts", lambda: [])())
+        out += [self.final_norm, self.head]
+        return out
+
+    def cache_requests(self):
+        return [b.mixer.cache_request() for b in self.blocks]
+
+    def bind_cache(self, device_cache) -> None:
+        for i, b in enumerate(self.blocks):
+            binding = device_cache.binding(i)
+            if binding is not None:
+                b.mixer.bind_cache(binding)
+
+    def attention_rows_per_token(self) -> List[int]:
+        return sorted({g for g in (b.mixer.attention_rows_per_token() for b in self.blocks) if g})
+
+    @property
+    def vocab(self) -> int:
+        return self.spec.head.vocab
+
+    # ------------------------------------------------------------------ the forward pass
+    def forward(self, ctx: StepContext) -> Optional[torch.Tensor]:
+        """Run the step's rows through the layers in ``order``; float32 logits ``[W, vocab]`` of
+        the wanted rows, or None when none is wanted."""
+        x = self.embedding.forward(ctx.tokens)
+        for i in self.order:
+            self.blocks[i].forward(x, ctx)
+        if ctx.want_rows.numel() == 0:
+            return None
+        return self.head.forward(self.final_norm.forward(x, rows=ctx.want_rows))

@@ -1,0 +1,18 @@
+"""RMS norm: ``y = x / sqrt(mean(x^2) + eps) * w`` with 32-bit statistics
+(``crates/mach-model/src/kernels.rs:63-80``)."""
+from __future__ import annotations
+
+from .base import Norm, TensorDecl
+from .registry import register_norm
+
+
+@register_norm("rmsnorm")
+class RMSNorm(Norm):
+    def tensor_decls(self):
+        return [TensorDecl("weight", (self.spec.width,), "vector")]
+
+    def load(self, tensors):
+        self.weight = tensors["weight"]
+
+    def forward(self, x, rows=None, out_f32=False):
+        return self.rt.ops.rmsnorm(x, self.weight, self.spec.eps, rows, out_f32)

@@ -1,0 +1,118 @@
+"""CPU stand-ins for the HIP entry points, with the same signatures and memory layouts.
+
+Used only by tests: they let the host logic of the engine (step building, cache manager,
+scheduler, replay) run where there is no GPU, and they are the per-kernel references of
+the GPU tests.  Nothing in the package imports this file.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+
+MASK64 = (1 << 64) - 1
+
+
+class EmulatedOps:
+    attention_rows_per_block_default = 64
+
+    def __init__(self, dtype=torch.float32, device="cpu"):
+        self.dtype = dtype
+        self.device = torch.device(device)
+
+    def _r(self, t):  # round to the element type, as a kernel's store does
+        return t.to(self.dtype)
+
+    def embed(self, tokens, table):
+        return table[tokens.long()].float()
+
+    def rmsnorm(self, x, weight, eps, rows=None, out_f32=False):
+        src = x if rows is None else x[rows.long()]
+        y = src * (1.0 / torch.sqrt((src * src).sum(-1, keepdim=True) / src.shape[-1] + eps)) * weight
+        return y if out_f32 else self._r(y)
+
+    def linear(self, a, w, bias=None, out_f32=False):
+        y = a.float() @ w.float().t()
+        if bias is not None:
+            y = y + bias
+        return y if out_f32 else self._r(y)
+
+    def linear_residual(self, a, w, x):
+        x += a.float() @ w.float().t()
+
+    def linear_swiglu(self, a, w_gate_up, intermediate):
+        Ip = w_gate_up.shape[0] // 2
+        w = w_gate_up.float().view(Ip // 16, 2, 16, -1)
+        gate = a.float() @ w[:, 0].reshape(Ip, -1).t()
+        up = a.float() @ w[:, 1].reshape(Ip, -1).t()
+        return self._r((gate / (1.0 + torch.exp(-gate)) * up)[:, :intermediate])
+
+    def rope_kv_write(self, qkv, positions, inv_freq, slot_map, kpool, vpool, H, KV, hd, page_size):
+        T = qkv.shape[0]
+        half = hd // 2
+        if inv_freq is not None:
+            ang = positions.float()[:, None] * inv_freq[None, :]
+            c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        else:
+            c = torch.ones(T, 1, half)
+            s = torch.zeros(T, 1, half)
+
+        def rot(x):
+            a, b = x[..., :half], x[..., half:]
+            return torch.cat([a * c - b * s, a * s + b * c], -1)
+
+        q = self._r(rot(qkv[:, :H * hd].reshape(T, H, hd))).reshape(T, H * hd)
+        if slot_map is not None:
+            k = self._r(rot(qkv[:, H * hd:(H + KV) * hd].reshape(T, KV, hd)))
+            v = self._r(qkv[:, (H + KV) * hd:(H + 2 * KV) * hd].reshape(T, KV, hd))
+            page, off = (slot_map // page_size).long(), (slot_map % page_size).long()
+            for t in range(T):
+                kpool[page[t], :, off[t], :] = k[t]
+                vpool[page[t], :, :, off[t]] = v[t]
+        return q
+
+    def attention_rows_per_block(self, hd):
+        return 64
+
+    def paged_attention(self, q, kpool, vpool, block_table, seq_q_start, seq_q_len, seq_pos0, work, H, KV, hd,
+                        page_size, window, scale):
+        T = q.shape[0]
+        g = H // KV
+        out = torch.zeros(T, H * hd)
+        done = set()
+        for s, r0 in work.tolist():
+            qs, ql, p0 = int(seq_q_start[s]), int(seq_q_len[s]), int(seq_pos0[s])
+            for r in range(r0, min(r0 + 64, ql * g)):
+                tok, j = divmod(r, g)
+                pos = p0 + tok
+                lo = 0 if not window else max(0, pos - window + 1)
+                keys = torch.arange(lo, pos + 1)
+                pages = block_table[s].long()[keys // page_size]
+                assert (pages >= 0).all(), "attention reads a page that was given back"
+                offs = keys % page_size
+                for kvh in range(KV):
+                    h = kvh * g + j
+                    kk = kpool[pages, kvh, offs, :].float()
+                    vv = vpool[pages, kvh, :, offs].float()
+                    sc = (kk @ q[qs + tok, h * hd:(h + 1) * hd].float()) * scale
+                    p = torch.softmax(sc, 0)
+                    out[qs + tok, h * hd:(h + 1) * hd] = p @ vv
+                    done.add((qs + tok, h))
+        assert len(done) == T * H, "the work list does not cover every row and head"
+        return self._r(out)
+
+    def sample(self, logits, temperature, top_k, top_p, state):
+        from plain.qwen2_plain import sample as plain_sample
+        toks, lps = [], []
+        for r in range(logits.shape[0]):
+            st = int(state[r].item()) & MASK64
+            tok, st = plain_sample(logits[r].numpy(), float(temperature[r]), int(top_k[r]), float(top_p[r]), st)
+            state[r] = st - (1 << 64) if st >= (1 << 63) else st
+            toks.append(tok)
+            lps.append(0.0)
+        return torch.tensor(toks, dtype=torch.int32), torch.tensor(lps)
+
+    def logit_edit(self, logits, row_of, token, delta):
+        for r, t, d in zip(row_of.tolist(), token.tolist(), delta.tolist()):
+            logits[r, t] += d

@@ -1,0 +1,290 @@
+"""Plain, slow Qwen2 decoder: whole sequences, no cache, one function per part.
+
+Written from the formulas of gqf2008/machserve (paths below are relative to the
+reference checkout).  It shares no code with the engine: it takes a dict of
+tensors by checkpoint name and a dict of sizes, and computes everything with
+ordinary torch ops on the CPU in the dtype of ``compute`` (float32 or float64).
+
+Every function cites the reference lines it was written from.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+
+def rms_norm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
+    """``y_i = x_i * (1 / sqrt(mean(x^2) + eps)) * w_i``: eps inside the root, added
+    to the mean, weight multiplied last and not offset by one.
+
+    crates/mach-model/src/ref_model.rs:1180-1188, crates/mach-model/src/kernels.rs:63-80.
+    """
+    ss = (x * x).sum(dim=-1, keepdim=True)
+    inv = 1.0 / torch.sqrt(ss / x.shape[-1] + eps)
+    return x * inv * w
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None = None) -> torch.Tensor:
+    """``y[n] = sum_k W[n, k] x[k] (+ b[n])``; weight is row-major ``[out, in]`` and
+    an absent bias tensor means no add.
+
+    crates/mach-model/src/ref_model.rs:1167-1178 (matvec_t), tools/ref_llama.py:104-115 (bias).
+    """
+    y = x @ w.t()
+    if b is not None:
+        y = y + b
+    return y
+
+
+def rope_angles(positions: torch.Tensor, head_dim: int, theta: float, dtype=torch.float32) -> torch.Tensor:
+    """``ang[p, j] = float(pos_p) * (1 / theta^(2j / head_dim))`` for ``j < head_dim/2``,
+    every step in ``dtype`` as the reference does it in f32.
+
+    crates/mach-model/src/ref_model.rs:636-643 (rope_freq, yarn off) and 679-681.
+    """
+    j = torch.arange(head_dim // 2, dtype=dtype)
+    freq = 1.0 / torch.pow(torch.tensor(float(theta), dtype=dtype), 2.0 * j / head_dim)
+    return positions.to(dtype)[:, None] * freq[None, :]
+
+
+def rope(x: torch.Tensor, positions: torch.Tensor, theta: float) -> torch.Tensor:
+    """Rotate pairs ``(j, j + head_dim/2)`` (rotate_half pairing, whole head rotated):
+    ``a' = a cos - b sin``, ``b' = a sin + b cos``.  ``x`` is ``[T, heads, head_dim]``.
+
+    crates/mach-model/src/ref_model.rs:669-704 (apply_rope, interleave=false), tools/ref_llama.py:56-67.
+    """
+    hd = x.shape[-1]
+    half = hd // 2
+    ang = rope_angles(positions, hd, theta, x.dtype)
+    c = torch.cos(ang)[:, None, :]
+    s = torch.sin(ang)[:, None, :]
+    a = x[..., :half]
+    b = x[..., half:]
+    return torch.cat([a * c - b * s, a * s + b * c], dim=-1)
+
+
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int | None = None) -> torch.Tensor:
+    """Causal grouped-query attention over a whole sequence.
+
+    ``q`` is ``[T, H, hd]``, ``k``/``v`` are ``[T, KV, hd]``.  Query head ``h`` reads
+    key/value head ``h // (H // KV)``; the row at position ``p`` sees keys ``0..=p``
+    (with ``window``: only the last ``window`` of them, ``p - window < t <= p``);
+    ``scale = head_dim^-0.5``; softmax with the maximum subtracted.
+
+    crates/mach-model/src/ref_model.rs:1130-1165 (attention_decode),
+    crates/mach-model/src/config.rs:231-234 (scale).  The window is not in the reference.
+    """
+    T, H, hd = q.shape
+    KV = k.shape[1]
+    g = H // KV
+    scale = hd ** -0.5
+    out = torch.zeros_like(q)
+    for h in range(H):
+        kv = h // g
+        for p in range(T):
+            lo = 0 if window is None else max(0, p - window + 1)
+            scores = (k[lo:p + 1, kv, :] @ q[p, h, :]) * scale
+            e = torch.exp(scores - scores.max())
+            out[p, h, :] = (e[:, None] * v[lo:p + 1, kv, :]).sum(dim=0) / e.sum()
+    return out
+
+
+def silu(x: torch.Tensor) -> torch.Tensor:
+    """``x / (1 + exp(-x))``.  crates/mach-model/src/ref_model.rs:1190-1192."""
+    return x / (1.0 + torch.exp(-x))
+
+
+def swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
+    """``down( silu(gate(x)) * up(x) )``: the activation is on the gate branch.
+
+    crates/mach-model/src/ref_model.rs:299-309, crates/mach-model/src/kernels.rs:131-140,
+    tools/ref_llama.py:120-123.
+    """
+    return linear(silu(linear(x, w_gate)) * linear(x, w_up), w_down)
+
+
+def attention_block(x, w, prefix, positions, sizes, window=None):
+    """q/k/v projections with optional bias, rotation of q and k, attention, output
+    projection without bias.  crates/mach-model/src/batched.rs:3566-3679, 4022-4031;
+    tools/ref_llama.py:100-119.
+    """
+    H, KV, hd = sizes["heads"], sizes["kv_heads"], sizes["head_dim"]
+    T = x.shape[0]
+    q = linear(x, w[prefix + "q_proj.weight"], w.get(prefix + "q_proj.bias"))
+    k = linear(x, w[prefix + "k_proj.weight"], w.get(prefix + "k_proj.bias"))
+    v = linear(x, w[prefix + "v_proj.weight"], w.get(prefix + "v_proj.bias"))
+    q = rope(q.view(T, H, hd), positions, sizes["theta"])
+    k = rope(k.view(T, KV, hd), positions, sizes["theta"])
+    o = attention(q, k, v.view(T, KV, hd), window)
+    return linear(o.reshape(T, H * hd), w[prefix + "o_proj.weight"])
+
+
+def layer_windows(sizes) -> list:
+    """Window of each layer: none unless ``use_sliding_window``; then layers with index
+    ``>= max_window_layers`` attend to the last ``sliding_window`` keys.  (Keys the
+    reference does not read; meaning taken from the keys' own names and documentation.)
+    """
+    L = sizes["layers"]
+    if not sizes.get("use_sliding_window", False):
+        return [None] * L
+    return [sizes["sliding_window"] if i >= sizes["max_window_layers"] else None for i in range(L)]
+
+
+def forward(weights: dict, sizes: dict, tokens, compute=torch.float32, start_pos: int = 0) -> torch.Tensor:
+    """Logits ``[T, vocab]`` at every position of one whole sequence.
+
+    Pre-norm blocks ``x += attn(norm(x)); x += mlp(norm(x))``, final norm, head =
+    ``lm_head.weight`` when the tensor exists, else the embedding table.
+    crates/mach-model/src/batched.rs:3150-3200, 4031-4050, 4424-4453, 4580-4626;
+    crates/mach-model/src/loader.rs:1025-1033 (head rule); tools/ref_llama.py:89-125.
+    """
+    w = {n: t.to(compute) for n, t in weights.items()}
+    toks = torch.as_tensor(tokens, dtype=torch.long)
+    positions = torch.arange(start_pos, start_pos + len(toks))
+    x = w["model.embed_tokens.weight"][toks]
+    windows = layer_windows(sizes)
+    for i in range(sizes["layers"]):
+        p = f"model.layers.{i}."
+        xn = rms_norm(x, w[p + "input_layernorm.weight"], sizes["eps"])
+        x = x + attention_block(xn, w, p + "self_attn.", positions, sizes, windows[i])
+        xn = rms_norm(x, w[p + "post_attention_layernorm.weight"], sizes["eps"])
+        x = x + swiglu(xn, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    xf = rms_norm(x, w["model.norm.weight"], sizes["eps"])
+    head = w["lm_head.weight"] if "lm_head.weight" in w and not sizes.get("tied", False) else w["model.embed_tokens.weight"]
+    return linear(xf, head)
+
+
+def sizes_from_config(cfg: dict) -> dict:
+    """Sizes the plain model needs, read from config.json's own keys.
+    crates/mach-server/src/startup.rs:63-98."""
+    heads = cfg["num_attention_heads"]
+    return {
+        "layers": cfg["num_hidden_layers"],
+        "hidden": cfg["hidden_size"],
+        "heads": heads,
+        "kv_heads": cfg.get("num_key_value_heads", heads),
+        "head_dim": cfg.get("head_dim", cfg["hidden_size"] // heads),
+        "intermediate": cfg["intermediate_size"],
+        "vocab": cfg["vocab_size"],
+        "eps": cfg.get("rms_norm_eps", 1e-6),
+        "theta": cfg.get("rope_theta", 10000.0),
+        "tied": cfg.get("tie_word_embeddings", False),
+        "use_sliding_window": cfg.get("use_sliding_window", False),
+        "sliding_window": cfg.get("sliding_window"),
+        "max_window_layers": cfg.get("max_window_layers", cfg["num_hidden_layers"]),
+    }
+
+
+def greedy_generate(weights, sizes, prompt, max_new, eos=None, compute=torch.float32):
+    """Greedy continuation by recomputing the whole sequence for every new token."""
+    seq = list(prompt)
+    out = []
+    for _ in range(max_new):
+        logits = forward(weights, sizes, seq, compute)[-1]
+        tok = argmax_first(logits)
+        out.append(tok)
+        seq.append(tok)
+        if eos is not None and tok == eos:
+            break
+    return out
+
+
+# ---------------------------------------------------------------- sampling
+
+MASK64 = (1 << 64) - 1
+RNG_GOLDEN = 0x9E3779B97F4A7C15
+
+
+def mix64(z: int) -> int:
+    """SplitMix64 finalizer.  crates/mach-model/src/sampling.rs:27-31."""
+    z &= MASK64
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & MASK64
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & MASK64
+    return z ^ (z >> 31)
+
+
+def next_uniform(state: int):
+    """One draw in [0, 1): finalizer of the state *before* the increment, top 24 bits.
+    Returns ``(u, new_state)``.  crates/mach-model/src/sampling.rs:34-44."""
+    z = mix64(state)
+    return (z >> 40) / 16777216.0, (state + RNG_GOLDEN) & MASK64
+
+
+def argmax_first(logits) -> int:
+    """Smallest index among the maxima.  crates/mach-model/src/sampling.rs:1153-1161."""
+    best = 0
+    vals = logits.tolist()
+    for i, v in enumerate(vals):
+        if v > vals[best]:
+            best = i
+    return best
+
+
+def sample(logits, temperature, top_k, top_p, state, presence=0.0, frequency=0.0, counts=(), bias=()):
+    """CPU mirror of the sampler; returns ``(token, new_state)``.  One draw and one
+    state advance per call, also when greedy.
+    crates/mach-model/src/sampling.rs:1169-1274 (sample_cpu).
+    """
+    import numpy as np
+    x = np.asarray(logits, dtype=np.float32).copy()
+    u, state = next_uniform(state)
+    for t, c in counts:
+        if t < len(x) and c > 0:
+            x[t] -= np.float32(presence + frequency * c)
+    for t, b in bias:
+        if t < len(x):
+            x[t] += np.float32(b)
+    if temperature <= 0.0:
+        return argmax_first(torch.from_numpy(x)), state
+    maxv, minv = x.max(), x.min()
+    inv_t = np.float32(1.0 / temperature)
+    prob = np.exp((x - maxv) * inv_t).astype(np.float32)
+    k_eff = top_k if 0 < top_k < len(x) else 0
+    thr = -np.inf
+    if k_eff:
+        lo, hi = np.float32(minv), np.float32(maxv)
+        for _ in range(30):
+            mid = np.float32((lo + hi) * np.float32(0.5))
+            if int((x > mid).sum()) >= k_eff:
+                lo = mid
+            else:
+                hi = mid
+        thr = hi
+    s_tot = np.float32(prob.sum(dtype=np.float32))
+    cut = np.float32(0.0)
+    use_topp = top_p < 1.0
+    if use_topp:
+        lo, hi = np.float32(0.0), np.float32(1.0)
+        for _ in range(30):
+            mid = np.float32((lo + hi) * np.float32(0.5))
+            acc = prob[prob >= mid].sum(dtype=np.float32)
+            if acc >= np.float32(top_p) * s_tot:
+                lo = mid
+            else:
+                hi = mid
+        cut = lo
+    allowed = np.ones(len(x), dtype=bool)
+    if k_eff:
+        allowed &= x >= thr
+    if use_topp:
+        allowed &= prob >= cut
+    target = np.float32(u) * prob[allowed].sum(dtype=np.float32)
+    acc = np.float32(0.0)
+    for i in range(len(x)):
+        if allowed[i]:
+            acc = np.float32(acc + prob[i])
+            if acc > target:
+                return i, state
+    return argmax_first(torch.from_numpy(x)), state
+
+
+def f32_to_bf16_bits(x: float) -> int:
+    """Round-to-nearest-even on the high 16 bits.  crates/mach-model/src/fp16.rs:84-94."""
+    import struct
+    b = struct.unpack("<I", struct.pack("<f", x))[0]
+    h = b >> 16
+    rem = b & 0xFFFF
+    if rem > 0x8000 or (rem == 0x8000 and (h & 1) == 1):
+        h = (h + 1) & 0xFFFF
+    return h

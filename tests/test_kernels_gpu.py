@@ -1,0 +1,241 @@
+"""Each HIP kernel alone against its plain reference, at sizes other than the engine's:
+head sizes in steps of 16, odd numbers of heads and groups, widths and vocabularies that
+are no power of two, page sizes 16 to 128, single rows beside long portions."""
+import math
+
+import pytest
+import torch
+
+from emulated_ops import EmulatedOps
+from gpu_util import DEV, assert_close
+from plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def ops_for(dtype):
+    from machserve_amd.kernels import get_ops
+    return get_ops(dtype, DEV)
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,V,d", [(1, 50, 24), (37, 1000, 200), (300, 777, 896)])
+def test_embed(dtype, T, V, d):
+    ops = ops_for(dtype)
+    table = rnd((V, d), dtype, 1)
+    toks = torch.randint(0, V, (T,), generator=torch.Generator().manual_seed(2), dtype=torch.int32)
+    got = ops.embed(toks.to(DEV), table.to(DEV))
+    assert torch.equal(got.cpu(), table[toks.long()].float())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,d,eps", [(1, 8, 1e-6), (5, 200, 1e-5), (130, 896, 1e-6), (3, 5000, 1e-2)])
+def test_rmsnorm(dtype, T, d, eps):
+    ops = ops_for(dtype)
+    x = rnd((T, d), torch.float32, 3, 3.0)
+    w = 1 + rnd((d,), torch.float32, 4, 0.1)
+    ref = P.rms_norm(x, w, eps)
+    assert_close(ops.rmsnorm(x.to(DEV), w.to(DEV), eps), ref, dtype, "rmsnorm")
+    rows = torch.tensor([T - 1, 0, T // 2], dtype=torch.int32)
+    got = ops.rmsnorm(x.to(DEV), w.to(DEV), eps, rows.to(DEV), out_f32=True)
+    assert_close(got, ref[rows.long()], torch.float32, "rmsnorm of gathered rows")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 16, 8), (7, 1000, 200), (64, 130, 896), (65, 257, 72), (300, 896, 4864),
+                                   (129, 9728 + 16, 64)])
+def test_linear(dtype, M, N, K):
+    ops = ops_for(dtype)
+    a, w = rnd((M, K), dtype, 5), rnd((N, K), dtype, 6, K ** -0.5)
+    b = rnd((N,), torch.float32, 7)
+    ref = P.linear(a.double(), w.double(), b.double())
+    assert_close(ops.linear(a.to(DEV), w.to(DEV), b.to(DEV), out_f32=True), ref, torch.float32 if dtype == torch.float32 else dtype, "linear f32 out")
+    assert_close(ops.linear(a.to(DEV), w.to(DEV), None), P.linear(a.double(), w.double()), dtype, "linear")
+    x = rnd((M, N), torch.float32, 8)
+    xd = x.to(DEV).clone()
+    ops.linear_residual(a.to(DEV), w.to(DEV), xd)
+    assert_close(xd, x.double() + P.linear(a.double(), w.double()), torch.float32 if dtype == torch.float32 else dtype, "linear_residual")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,I,K", [(1, 16, 8), (9, 160, 64), (70, 328, 192), (200, 4864, 896)])
+def test_linear_swiglu(dtype, M, I, K):
+    from machserve_amd.kernels import interleave_gate_up
+    ops = ops_for(dtype)
+    a, g, u = rnd((M, K), dtype, 9), rnd((I, K), dtype, 10, K ** -0.5 * 3), rnd((I, K), dtype, 11, K ** -0.5)
+    ref = P.silu(P.linear(a.double(), g.double())) * P.linear(a.double(), u.double())
+    got = ops.linear_swiglu(a.to(DEV), interleave_gate_up(g, u).to(DEV), I)
+    assert_close(got, ref, dtype, "swiglu")
+    swapped = P.silu(P.linear(a.double(), u.double())) * P.linear(a.double(), g.double())
+    assert (ref - swapped).abs().max() > 0.05 * ref.abs().max(), "the test must tell gate from up"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,KV,hd,ps,theta", [(4, 2, 16, 16, 1e4), (6, 1, 32, 32, 1e6), (5, 5, 48, 64, 5e4),
+                                              (14, 2, 64, 64, 1e6), (3, 3, 128, 128, 1e6)])
+def test_rope_kv_write(dtype, H, KV, hd, ps, theta):
+    ops, emu = ops_for(dtype), EmulatedOps(dtype)
+    T, pages = 45, 12
+    qkv = rnd((T, (H + 2 * KV) * hd), torch.float32, 12)
+    pos = torch.randint(0, 3000, (T,), generator=torch.Generator().manual_seed(13), dtype=torch.int32)
+    perm = torch.randperm(pages * ps, generator=torch.Generator().manual_seed(14))[:T].to(torch.int32)
+    j = torch.arange(hd // 2, dtype=torch.float32)
+    inv = 1.0 / torch.pow(torch.tensor(theta, dtype=torch.float32), 2.0 * j / hd)
+    kp, vp = torch.zeros(pages, KV, ps, hd, dtype=dtype), torch.zeros(pages, KV, hd, ps, dtype=dtype)
+    q_ref = emu.rope_kv_write(qkv, pos, inv, perm, kp, vp, H, KV, hd, ps)
+    # the emulation's rotation against the plain model's
+    q_plain = P.rope(qkv[:, :H * hd].view(T, H, hd), pos, theta).reshape(T, H * hd)
+    assert_close(q_ref, q_plain, dtype, "emulated rotation")
+    kd, vd = torch.zeros_like(kp).to(DEV), torch.zeros_like(vp).to(DEV)
+    q = ops.rope_kv_write(qkv.to(DEV), pos.to(DEV), inv.to(DEV), perm.to(DEV), kd, vd, H, KV, hd, ps)
+    assert_close(q, q_plain, dtype, "q rotation")
+    assert_close(kd, kp, dtype, "key pages")
+    assert_close(vd, vp, dtype, "value pages")
+    # without a table of frequencies nothing rotates
+    q0 = ops.rope_kv_write(qkv.to(DEV), pos.to(DEV), None, None, None, None, H, KV, hd, ps)
+    assert_close(q0, qkv[:, :H * hd], dtype, "no rotation")
+
+
+def _attention_case(dtype, H, KV, hd, ps, window, seqs, seed, peak=False):
+    """seqs: list of (cached length, rows in this step).  Builds scattered pages holding random
+    keys and values for positions < cached + rows and queries for the step's rows."""
+    ops, emu = ops_for(dtype), EmulatedOps(dtype)
+    g = H // KV
+    gen = torch.Generator().manual_seed(seed)
+    n_pages = sum(-(-(c + n) // ps) for c, n in seqs) + 3
+    order = torch.randperm(n_pages, generator=gen).tolist()
+    kp = rnd((n_pages, KV, ps, hd), dtype, seed + 1)
+    vp = rnd((n_pages, KV, hd, ps), dtype, seed + 2)
+    width = max(-(-(c + n) // ps) for c, n in seqs)
+    table = torch.full((len(seqs), width), -1, dtype=torch.int32)
+    q_start, q_len, pos0, work = [], [], [], []
+    T = 0
+    for i, (c, n) in enumerate(seqs):
+        for p in range(-(-(c + n) // ps)):
+            table[i, p] = order.pop()
+        q_start.append(T), q_len.append(n), pos0.append(c)
+        work += [(i, r0) for r0 in range(0, n * g, 64)]
+        T += n
+    q = rnd((T, H * hd), dtype, seed + 3)
+    if peak:
+        # one far key stands out for one query row: scale that key and query so that the score
+        # towers over the rest and a missed key shows in the output
+        i, (c, n) = max(enumerate(seqs), key=lambda t: t[1][0])
+        row, head, far = q_start[i] + n - 1, H - 1, (1 if not window else c + n - window)
+        kvh = head // g
+        page, off = int(table[i, far // ps]), far % ps
+        qv = q[row, head * hd:(head + 1) * hd].float()
+        kp[page, kvh, off, :] = (qv / qv.norm() * 8.0).to(dtype)
+        q[row, head * hd:(head + 1) * hd] = (qv / qv.norm() * 8.0 * math.sqrt(hd) / 4).to(dtype)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32)
+    args = (i32(q_start), i32(q_len), i32(pos0), i32(work).view(-1, 2))
+    ref = emu.paged_attention(q, kp, vp, table, *args, H, KV, hd, ps, window, hd ** -0.5)
+    got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV), table.to(DEV), *[a.to(DEV) for a in args], H, KV, hd,
+                              ps, window, hd ** -0.5)
+    return got, ref
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,KV,hd,ps", [(4, 2, 16, 16), (6, 1, 32, 32), (5, 5, 48, 16), (14, 2, 64, 64), (7, 7, 80, 32),
+                                        (12, 2, 128, 64), (20, 1, 64, 128), (2, 1, 256, 16)])
+def test_attention_mixed_batch(dtype, H, KV, hd, ps):
+    seqs = [(0, 1), (0, 70), (130, 1), (37, 45), (ps - 1, 2), (ps, 1), (2 * ps - 1, 1)]
+    got, ref = _attention_case(dtype, H, KV, hd, ps, None, seqs, 100 + hd)
+    assert_close(got, ref, dtype, "attention")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 17, 64, 100])
+def test_attention_window(dtype, window):
+    seqs = [(0, 150), (200, 1), (63, 3), (0, 1)]
+    got, ref = _attention_case(dtype, 6, 2, 32, 16, window, seqs, 200 + window)
+    assert_close(got, ref, dtype, f"attention with window {window}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [None, 300])
+def test_attention_far_key_stands_out(dtype, window):
+    seqs = [(700, 1), (0, 5), (400, 40)]
+    got, ref = _attention_case(dtype, 8, 2, 64, 64, window, seqs, 300, peak=True)
+    assert_close(got, ref, dtype, "attention with a far key that dominates")
+
+
+def test_attention_equals_library_attention_without_rotation_or_paging():
+    """One request, whole prompt, pages in order: the kernel is plain causal attention."""
+    dtype = torch.float32
+    H, KV, hd, ps, T = 4, 4, 32, 16, 50
+    got, ref = _attention_case(dtype, H, KV, hd, ps, None, [(0, T)], 400)
+    assert_close(got, ref, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_refusals(dtype):
+    from machserve_amd.kernels import KernelError
+    ops = ops_for(dtype)
+    a, w = torch.zeros(4, 12, dtype=dtype, device=DEV), torch.zeros(16, 12, dtype=dtype, device=DEV)
+    with pytest.raises(KernelError, match="multiple of 8"):
+        ops.linear(a, w)
+    with pytest.raises(Exception, match="multiple of 16"):
+        ops.attention_rows_per_block(40)
+    with pytest.raises(KernelError, match="GPU tensor"):
+        ops.linear(a.cpu(), w)
+
+
+def test_sampler_matches_cpu_mirror():
+    """Peaked logits as in crates/mach-model/src/sampling.rs:1711-1752: the boundary tiers and
+    the draw land far from any edge, so the orders of summation cannot change the outcome."""
+    ops = ops_for(torch.float32)
+    V, n = 2048, 12
+    logits = torch.zeros(n, V)
+    for s in range(n):
+        logits[s] = 0.5 - 1.2 * torch.arange(V) * 0.25
+        logits[s, ::37] += 0.05
+        logits[s] = logits[s].roll(s * 97)
+    temps = torch.tensor([[0.8, 1.0, 1.2, 0.0][i % 4] for i in range(n)])
+    ks = torch.tensor([[0, 0, 40, 10][i % 4] for i in range(n)], dtype=torch.int32)
+    ps_ = torch.tensor([[0.95, 1.0, 0.9, 0.8][i % 4] for i in range(n)])
+    seeds = torch.tensor([7000 + i for i in range(n)], dtype=torch.int64)
+    state = seeds.clone().to(DEV)
+    for rep in range(3):
+        got, _ = ops.sample(logits.to(DEV), temps.to(DEV), ks.to(DEV), ps_.to(DEV), state)
+        for i in range(n):
+            st = int(seeds[i]) + rep * P.RNG_GOLDEN
+            want, new = P.sample(logits[i].numpy(), float(temps[i]), int(ks[i]), float(ps_[i]), st & P.MASK64)
+            assert int(got[i]) == want, f"row {i} rep {rep}"
+    want_state = [(int(s) + 3 * P.RNG_GOLDEN) & P.MASK64 for s in seeds]
+    assert [int(v) & P.MASK64 for v in state.cpu().tolist()] == want_state
+
+
+def test_sampler_greedy_ties_and_spread():
+    ops = ops_for(torch.float32)
+    V = 1000
+    logits = torch.zeros(3, V)
+    logits[0, [5, 700, 999]] = 2.0           # ties: the smallest index wins
+    logits[1, 999] = 1.0
+    logits[2] = torch.randn(V, generator=torch.Generator().manual_seed(1))
+    z = torch.zeros(3)
+    tok, lp = ops.sample(logits.to(DEV), z.to(DEV), torch.zeros(3, dtype=torch.int32, device=DEV), torch.ones(3).to(DEV),
+                         torch.zeros(3, dtype=torch.int64, device=DEV))
+    assert tok.cpu().tolist() == [5, 999, int(logits[2].argmax())]
+    # a flat distribution is covered by different seeds
+    flat = torch.zeros(64, V)
+    st = torch.arange(1, 65, dtype=torch.int64).to(DEV)
+    tok, _ = ops.sample(flat.to(DEV), torch.ones(64).to(DEV), torch.zeros(64, dtype=torch.int32, device=DEV),
+                        torch.ones(64).to(DEV), st)
+    assert len(set(tok.cpu().tolist())) > 40
+
+
+def test_logit_edit():
+    ops = ops_for(torch.float32)
+    x = torch.zeros(2, 10, device=DEV)
+    ops.logit_edit(x, torch.tensor([0, 1, 1], dtype=torch.int32, device=DEV),
+                   torch.tensor([3, 0, 9], dtype=torch.int32, device=DEV), torch.tensor([1.5, -2.0, 4.0], device=DEV))
+    ref = torch.zeros(2, 10)
+    ref[0, 3], ref[1, 0], ref[1, 9] = 1.5, -2.0, 4.0
+    assert torch.equal(x.cpu(), ref)

@@ -1,0 +1,173 @@
+"""The engine against the plain model through the step function, cache and kernels that
+generation uses: each request alone and whole; most of it in one step and the last 32
+tokens one by one; portions of changing size down to two tokens; and mixed, up to four
+live requests with portions of some beside decoded tokens of others and so few pages
+that they are handed out again.  In 32-bit and in bfloat16."""
+import pytest
+import torch
+
+from gpu_util import DEV
+from plain import qwen2_plain as P
+from tiny_configs import CONFIGS, make_model_dir, random_prompt, read_for_plain
+
+pytestmark = pytest.mark.gpu
+
+PAGE = {"A": 16, "B": 32, "C": 16}
+LENGTHS = {"A": [5, 17, 33, 90], "B": [1, 9, 40, 100], "C": [3, 64, 130, 47]}
+
+
+def logit_tol(dtype, ref):
+    """float32: the reference's own bound for a 32-bit GPU against a CPU forward is
+    2e-3 + 2e-3 * scale (crates/mach-model/tests/decode_slice.rs:79-85); ours is a hundred
+    times tighter.  bfloat16 (weights rounded once, activations rounded at every matrix
+    input, cache in bfloat16): 8 bits of mantissa, ~2^-8 per rounding, a few dozen roundings
+    adding up like a random walk."""
+    scale = ref.abs().max().item()
+    return (2e-5 + 2e-5 * scale) if dtype == torch.float32 else (3e-2 * scale)
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    tmp = tmp_path_factory.mktemp("models")
+    out = {}
+    for which in CONFIGS:
+        d = make_model_dir(tmp, which)
+        w, sizes = read_for_plain(d)
+        prompts = [random_prompt(n, sizes["vocab"], 10 * i + len(which)) for i, n in enumerate(LENGTHS[which])]
+        out[which] = (d, w, sizes, prompts, {})
+    return out
+
+
+def plain_logits(models, which, dtype, i):
+    d, w, sizes, prompts, memo = models[which]
+    key = (dtype, i)
+    if key not in memo:
+        ww = w if dtype == torch.float32 else {k: v.to(torch.bfloat16).float() if v.dim() == 2 else v for k, v in w.items()}
+        memo[key] = P.forward(ww, sizes, prompts[i])
+    return memo[key]
+
+
+def engine(models, which, dtype, num_pages):
+    from machserve_amd.engine import load_model
+    return load_model(models[which][0], dtype=dtype, device=DEV, page_size=PAGE[which], num_pages=num_pages)
+
+
+def check(got, ref, dtype, what):
+    got = got.float().cpu()
+    err = (got - ref).abs().max().item()
+    assert err <= logit_tol(dtype, ref), f"{what}: max error {err:.3e}, allowed {logit_tol(dtype, ref):.3e}"
+    if dtype == torch.float32:
+        assert torch.equal(got.argmax(-1), ref.argmax(-1)), f"{what}: argmax differs"
+
+
+def run_cuts(lm, prompt, cuts):
+    from machserve_amd.engine import StepEntry
+    slot = lm.cache.admit()
+    out, i = [], 0
+    for c in cuts:
+        out.append(lm.step([StepEntry(slot, prompt[i:i + c], list(range(c)))]))
+        i += c
+    assert i == len(prompt)
+    lm.cache.release(slot)
+    lm.cache.check()
+    return torch.cat(out)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_whole_prompts(models, which, dtype):
+    lm = engine(models, which, dtype, 16)
+    for i, prompt in enumerate(models[which][3]):
+        check(run_cuts(lm, prompt, [len(prompt)]), plain_logits(models, which, dtype, i), dtype, f"{which} prompt {i} whole")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_last_32_one_by_one(models, which, dtype):
+    lm = engine(models, which, dtype, 16)
+    for i, prompt in enumerate(models[which][3]):
+        n = len(prompt)
+        head = max(0, n - 32)
+        cuts = ([head] if head else []) + [1] * (n - head)
+        check(run_cuts(lm, prompt, cuts), plain_logits(models, which, dtype, i), dtype, f"{which} prompt {i} decoded")
+
+
+def changing_cuts(n):
+    sizes, out, i = [7, 2, 5, 3, 11, 2, 24, 2, 1, 31, 4], [], 0
+    while n > 0:
+        c = min(sizes[i % len(sizes)], n)
+        if n - c == 1:  # no portion of one token at the end of a prompt unless it is the whole rest
+            c = n
+        out.append(c)
+        n -= c
+        i += 1
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_portions_of_changing_size(models, which, dtype):
+    lm = engine(models, which, dtype, 16)
+    for i, prompt in enumerate(models[which][3]):
+        check(run_cuts(lm, prompt, changing_cuts(len(prompt))), plain_logits(models, which, dtype, i), dtype,
+              f"{which} prompt {i} in portions")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_mixed_with_page_reuse(models, which, dtype):
+    """Requests arrive one after another; every step carries a portion of the newest beside
+    one token of each older one.  The pool holds the live requests and no more, so a
+    finished request's pages go to the next."""
+    from machserve_amd.engine import StepEntry
+    d, w, sizes, prompts, _ = models[which]
+    ps = PAGE[which]
+    seqs = [prompts[i % len(prompts)] for i in range(7)]
+    refs = [plain_logits(models, which, dtype, i % len(prompts)) for i in range(7)]
+    live_cap = 3
+    pages = sum(sorted(-(-len(s) // ps) for s in seqs)[-live_cap:])
+    lm = engine(models, which, dtype, pages)
+    got = [[] for _ in seqs]
+    state = {}  # request -> [slot, fed]
+    waiting = list(range(len(seqs)))
+    portion = [9, 2, 17, 5]
+    step, reused = 0, set()
+    first_pages = None
+    while waiting or state:
+        while waiting and len(state) < live_cap:
+            r = waiting[0]
+            need = -(-len(seqs[r]) // ps)
+            held = sum(-(-len(seqs[q]) // ps) for q in state)
+            if held + need > pages:
+                break
+            waiting.pop(0)
+            state[r] = [lm.cache.admit(), 0]
+        entries, order = [], []
+        newest = max(state)
+        for r, (slot, fed) in sorted(state.items()):
+            left = len(seqs[r]) - fed
+            if r == newest:
+                n = min(portion[step % len(portion)], left)
+                if left - n == 1:
+                    n = left
+            else:
+                n = 1
+            entries.append(StepEntry(slot, seqs[r][fed:fed + n], list(range(n))))
+            order.append((r, n))
+        logits = lm.step(entries)
+        lm.cache.check()
+        k = 0
+        for r, n in order:
+            got[r].append(logits[k:k + n])
+            k += n
+            state[r][1] += n
+            reused.update(lm.cache.table(next(iter(lm.cache.groups)), state[r][0]))
+            if state[r][1] == len(seqs[r]):
+                lm.cache.release(state.pop(r)[0])
+        step += 1
+    lm.cache.check()
+    assert all(g.pool.available() == g.pool.num_pages for g in lm.cache.groups.values())
+    total_pages = sum(-(-len(s) // ps) for s in seqs)
+    assert total_pages > pages, "the trace must need more pages than the pool has"
+    for r in range(len(seqs)):
+        check(torch.cat(got[r]), refs[r], dtype, f"{which} request {r} mixed")
