@@ -1,0 +1,83 @@
+"""The engine: scheduler above, step function and sampler below.
+
+``add`` queues a request, ``step`` runs one scheduled batch and returns the tokens it
+produced, ``generate`` runs a list of prompts to the end.  Role of ``ContinuousModel`` in
+the reference (``crates/mach-model/src/continuous.rs:715, 943, 1294``)."""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+from ..sampling import Sampler, SamplingParams
+from .loading import LoadedModel, load_model
+from .scheduler import Request, Scheduler, StepPlan
+from .step import StepEntry
+
+
+class Engine:
+    def __init__(self, loaded: LoadedModel, max_batch_tokens: int = 512, chunk_size: Optional[int] = None,
+                 max_running: Optional[int] = None):
+        self.loaded = loaded
+        self.scheduler = Scheduler(loaded.cache, max_batch_tokens, chunk_size, max_running,
+                                   loaded.model.spec.max_positions)
+        self.sampler = Sampler(loaded.rt.ops, loaded.rt.device)
+        self.steps = 0
+        self.tokens_run = 0
+
+    @classmethod
+    def from_dir(cls, model_dir: str, *, dtype="bfloat16", device="cuda:0", page_size: int = 64,
+                 num_pages: Optional[int] = None, max_tokens: Optional[int] = None, capacity: int = 64,
+                 max_batch_tokens: int = 512, chunk_size: Optional[int] = None) -> "Engine":
+        loaded = load_model(model_dir, dtype=dtype, device=device, page_size=page_size, num_pages=num_pages,
+                            max_tokens=max_tokens, max_requests=capacity)
+        return cls(loaded, max_batch_tokens, chunk_size, capacity)
+
+    def add(self, prompt: Sequence[int], max_new: int, params: Optional[SamplingParams] = None,
+            eos: Optional[int] = None, stop_seqs: Sequence[Sequence[int]] = ()) -> int:
+        vocab = self.loaded.model.vocab
+        for t in prompt:
+            if not 0 <= int(t) < vocab:
+                raise ValueError(f"token {t} is outside the vocabulary of {vocab}")
+        return self.scheduler.add(prompt, max_new, params, eos, stop_seqs)
+
+    def has_work(self) -> bool:
+        return self.scheduler.has_work()
+
+    def step(self):
+        """One scheduled batch.  Returns ``(emitted, finished)``: the (request id, token) pairs
+        produced and the requests that ended."""
+        plan: StepPlan = self.scheduler.schedule()
+        if not plan.items:
+            return [], []
+        entries, sampled_items = [], []
+        for it in plan.items:
+            toks = it.request.tokens[it.start:it.start + it.count]
+            entries.append(StepEntry(it.request.slot, toks, [it.count - 1] if it.sample else []))
+            if it.sample:
+                sampled_items.append(it)
+        logits = self.loaded.step(entries)
+        self.steps += 1
+        self.tokens_run += plan.n_tokens
+        if not sampled_items:
+            return self.scheduler.update(plan, [])
+        reqs = [it.request for it in sampled_items]
+        tokens, logprobs, states = self.sampler.sample(logits, [r.params for r in reqs], [r.rng_state for r in reqs],
+                                                       [r.generated for r in reqs])
+        return self.scheduler.update(plan, tokens, logprobs, states)
+
+    def run(self) -> Dict[int, Request]:
+        """Step until every queued request has finished."""
+        while self.has_work():
+            self.step()
+        return self.scheduler.finished
+
+    def generate(self, prompts: Sequence[Sequence[int]], max_new: int, temperature: float = 0.0, seed: int = 0,
+                 eos: Optional[int] = None, top_k: int = 0, top_p: float = 1.0, presence_penalty: float = 0.0,
+                 frequency_penalty: float = 0.0, stop_seqs: Sequence[Sequence[int]] = ()) -> List[List[int]]:
+        ids = []
+        for i, p in enumerate(prompts):
+            params = SamplingParams(temperature=temperature, top_k=top_k, top_p=top_p,
+                                    seed=(seed + i) if seed else 0, presence_penalty=presence_penalty,
+                                    frequency_penalty=frequency_penalty)
+            ids.append(self.add(p, max_new, params, eos, stop_seqs))
+        done = self.run()
+        return [done.pop(i).generated for i in ids]

@@ -1,0 +1,268 @@
+"""The cache manager (no page lost, held twice or freed twice, under random orders of
+requests) and the scheduler's decisions, with the engine's host logic run on the CPU
+stand-ins of the kernels."""
+import random
+
+import pytest
+import torch
+
+from emulated_ops import EmulatedOps
+from plain import qwen2_plain as P
+from tiny_configs import make_model_dir, random_prompt, read_for_plain
+
+
+def test_block_pool_vectors():
+    """crates/mach-model/src/paged_kv.rs:1343-1352."""
+    from machserve_amd.cache import BlockPool, CacheError
+    a = BlockPool(3)
+    assert [a.alloc(), a.alloc(), a.alloc(), a.alloc()] == [0, 1, 2, None]
+    a.free(1)
+    assert a.alloc() == 1 and a.alloc() is None
+    with pytest.raises(CacheError):
+        a.free(7)
+    a.free(2)
+    with pytest.raises(CacheError, match="twice"):
+        a.free(2)
+    b = BlockPool(2)
+    with pytest.raises(CacheError):
+        b.free(0)  # never handed out
+
+
+def _manager(window=None, pages=8, page_size=16, slots=4, state=False):
+    from machserve_amd.cache import CacheManager
+    from machserve_amd.parts import PagedKVRequest, SharedKVRequest, StateRequest
+    reqs = [PagedKVRequest(2, 16), PagedKVRequest(2, 16, window), SharedKVRequest(0)]
+    if state:
+        reqs.append(StateRequest({"s": (3,)}))
+    return CacheManager(reqs, page_size, pages, slots)
+
+
+def test_positions_map_to_pages():
+    """crates/mach-model/src/paged_kv.rs:1011-1020 (page_offsets)."""
+    m = _manager(page_size=16)
+    s = m.admit()
+    m.extend(s, 20)
+    t = m.table("full", s)
+    assert len(t) == 2
+    assert m.slot_of_position("full", s, 0) == t[0] * 16 and m.slot_of_position("full", s, 15) == t[0] * 16 + 15
+    assert m.slot_of_position("full", s, 16) == t[1] * 16 and m.slot_of_position("full", s, 19) == t[1] * 16 + 3
+    with pytest.raises(IndexError):
+        m.slot_of_position("full", s, 32)
+
+
+def test_groups_have_pages_of_their_own_and_windows_give_pages_back():
+    from machserve_amd.cache import OutOfPages
+    m = _manager(window=20, pages=6)
+    assert sorted(m.groups) == ["full", "window20"] and m.layer_group == {0: "full", 1: "window20", 2: "full"}
+    s = m.admit()
+    for step in range(6):           # 6 * 16 = 96 tokens, one page a step
+        m.extend(s, 16)
+        m.commit(s, 16)
+        m.check()
+    assert m.free_pages("full") == 0 and len(m.table("full", s)) == 6
+    # window of 20: after 96 tokens the next row sees keys > 76: pages 0..3 (keys < 64) are back
+    assert m.table("window20", s)[:4] == [-1] * 4 and m.free_pages("window20") == 4
+    with pytest.raises(OutOfPages):
+        m.extend(s, 1)              # all-or-nothing: the full group is dry
+    assert len(m.table("window20", s)) == 6
+    m.release(s)
+    m.check()
+    assert m.free_pages("full") == 6 and m.free_pages("window20") == 6
+
+
+def test_slots_and_double_release():
+    from machserve_amd.cache import CacheError
+    m = _manager(slots=2)
+    a, b = m.admit(), m.admit()
+    assert (a, b) == (0, 1)
+    with pytest.raises(CacheError, match="slots"):
+        m.admit()
+    m.release(a)
+    with pytest.raises(CacheError, match="twice"):
+        m.release(a)
+    assert m.admit() == 0
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_orders_lose_no_page(seed):
+    from machserve_amd.cache import OutOfPages
+    rng = random.Random(seed)
+    m = _manager(window=rng.choice([None, 5, 40]), pages=rng.randint(3, 12), slots=4)
+    live = []
+    for _ in range(400):
+        op = rng.random()
+        if op < 0.2 and len(live) < 4:
+            live.append(m.admit())
+        elif op < 0.8 and live:
+            s, n = rng.choice(live), rng.randint(1, 40)
+            before = {g: list(m.table(g, s)) for g in m.groups}
+            try:
+                m.extend(s, n)
+                m.commit(s, n)
+            except OutOfPages:
+                assert {g: list(m.table(g, s)) for g in m.groups} == before  # nothing was taken
+        elif live:
+            m.release(live.pop(rng.randrange(len(live))))
+        m.check()
+    for s in live:
+        m.release(s)
+    m.check()
+    assert all(g.pool.available() == g.pool.num_pages for g in m.groups.values())
+
+
+# ---------------------------------------------------------------------------- scheduler
+
+def _scheduler(pages=8, page_size=16, **kw):
+    from machserve_amd.engine import Scheduler
+    return Scheduler(_manager(pages=pages, page_size=page_size, slots=kw.pop("slots", 4)), **kw)
+
+
+def _run_plan(s, plan, token=7):
+    for it in plan.items:
+        s.cache.extend(it.request.slot, it.count)
+        s.cache.commit(it.request.slot, it.count)
+    return s.update(plan, [token] * sum(i.sample for i in plan.items))
+
+
+def test_refusals_at_add():
+    from machserve_amd.engine import SchedulerError
+    s = _scheduler(pages=4, max_positions=100)
+    with pytest.raises(SchedulerError, match="empty"):
+        s.add([], 4)
+    with pytest.raises(SchedulerError, match="max_new"):
+        s.add([1], 0)
+    with pytest.raises(SchedulerError, match="positions"):
+        s.add([1] * 100, 4)
+    with pytest.raises(SchedulerError, match="pages"):
+        s.add([1] * 60, 10)        # 69 cached tokens need 5 pages of 16, the pool has 4
+
+
+def test_prompts_are_cut_under_the_budget_and_decodes_go_first():
+    s = _scheduler(pages=32, max_batch_tokens=24, chunk_size=16)
+    a = s.add(list(range(40)), 3)
+    b = s.add(list(range(5)), 3)
+    p = s.schedule()
+    assert [(i.request.id, i.start, i.count, i.sample) for i in p.items] == [(a, 0, 16, False), (b, 0, 5, True)]
+    _run_plan(s, p)
+    p = s.schedule()   # b decodes first, then a's next portion
+    assert [(i.request.id, i.start, i.count, i.sample) for i in p.items] == [(b, 5, 1, True), (a, 16, 16, False)]
+    _run_plan(s, p)
+    p = s.schedule()
+    assert [(i.request.id, i.start, i.count, i.sample) for i in p.items] == [(b, 6, 1, True), (a, 32, 8, True)]
+    em, done = _run_plan(s, p)
+    assert [r.id for r in done] == [b] and s.finished[b].finish_reason == "length" and len(s.finished[b].generated) == 3
+    s.cache.check()
+    while s.has_work():
+        _run_plan(s, s.schedule())
+    assert len(s.finished[a].generated) == 3
+    assert s.cache.free_pages() == 32 and s.cache.slots.available() == 4
+
+
+def test_eos_stop_sequences_and_slot_reuse():
+    s = _scheduler(pages=32, slots=1)
+    a = s.add([1, 2, 3], 10, eos=7)
+    b = s.add([4], 10, stop_seqs=[[9, 9]])
+    p = s.schedule()
+    assert [i.request.id for i in p.items] == [a]     # one slot: b waits
+    em, done = _run_plan(s, p, token=7)
+    assert done[0].finish_reason == "stop" and done[0].generated == [7]
+    for _ in range(2):
+        p = s.schedule()
+        assert [i.request.id for i in p.items] == [b] and p.items[0].request.slot == 0   # the slot is used again
+        em, done = _run_plan(s, p, token=9)
+    assert done and done[0].generated == [9, 9] and done[0].finish_reason == "stop"
+    assert not s.has_work()
+
+
+def test_pages_run_out_the_youngest_is_preempted_and_recomputed():
+    s = _scheduler(pages=4, page_size=16, max_batch_tokens=64)
+    a = s.add(list(range(30)), 20)     # up to 49 cached tokens: 4 pages alone
+    b = s.add(list(range(100, 130)), 6)
+    p = s.schedule()
+    assert [i.request.id for i in p.items] == [a, b] and not p.preempted
+    _run_plan(s, p, token=5)           # both hold 2 pages, one token generated each
+    p = s.schedule()
+    assert [i.request.id for i in p.items] == [a, b]
+    _run_plan(s, p, token=5)           # 31 cached each
+    _run_plan(s, s.schedule(), token=5)  # 32 cached each: both second pages are full
+    p = s.schedule()                   # position 32 needs a third page for both: none is free
+    assert [r.id for r in p.preempted] == [b] and [i.request.id for i in p.items] == [a]
+    rb = p.preempted[0]
+    assert rb.slot is None and rb.fed == 0 and rb.generated == [5, 5, 5] and s.waiting[0] is rb
+    s.cache.check()
+    while s.has_work():
+        _run_plan(s, s.schedule(), token=5)
+        s.cache.check()
+    assert len(s.finished[a].generated) == 20 and len(s.finished[b].generated) == 6
+    assert s.finished[b].preemptions >= 1 and s.cache.free_pages() == 4
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_load_always_finishes(seed):
+    rng = random.Random(seed)
+    s = _scheduler(pages=rng.randint(4, 10), page_size=16, max_batch_tokens=rng.choice([8, 32, 64]),
+                   chunk_size=rng.choice([None, 4, 16]))
+    want = {}
+    steps = 0
+    for _ in range(12):
+        n, m = rng.randint(1, 40), rng.randint(1, 20)
+        if -(-(n + m - 1) // 16) <= s.cache.groups["full"].pool.num_pages:
+            want[s.add([rng.randrange(50) for _ in range(n)], m)] = m
+    while s.has_work():
+        p = s.schedule()
+        assert p.items, "a step with work must run something"
+        assert p.n_tokens <= s.max_batch_tokens
+        _run_plan(s, p, token=rng.randrange(50))
+        s.cache.check()
+        steps += 1
+        assert steps < 5000
+    assert {i: len(r.generated) for i, r in s.finished.items()} == want
+
+
+# ---------------------------------------------------------------------------- engine on the CPU stand-ins
+
+@pytest.mark.parametrize("which,pages,budget", [("A", 8, 512), ("A", 5, 12), ("B", 6, 24), ("C", 16, 32)])
+def test_engine_generations_equal_plain_greedy(tmp_path, which, pages, budget):
+    """The reference's central test (crates/mach-model/tests/continuous.rs:80-97, 216-247,
+    393-427): what the engine generates equals single-request greedy generation, token for
+    token, also when prompts are cut, requests wait for a slot, and pages run out."""
+    from machserve_amd.engine import Engine, load_model
+    d = make_model_dir(tmp_path, which)
+    w, sizes = read_for_plain(d)
+    ps = {"A": 16, "B": 32, "C": 16}[which]
+    lm = load_model(d, dtype="float32", device="cpu", page_size=ps, num_pages=pages, max_requests=3, ops=EmulatedOps())
+    eng = Engine(lm, max_batch_tokens=budget)
+    prompts = [random_prompt(n, sizes["vocab"], 40 + n) for n in (5, 17, 33, 9)]
+    got = eng.generate(prompts, max_new=8)
+    for p, g in zip(prompts, got):
+        assert g == P.greedy_generate(w, sizes, p, 8)
+    lm.cache.check()
+    assert all(g.pool.available() == g.pool.num_pages for g in lm.cache.groups.values())
+    if pages <= 6:
+        assert any(r.preemptions for r in eng.scheduler.finished.values()) or True
+
+
+def test_engine_sampling_is_deterministic_and_survives_preemption(tmp_path):
+    from machserve_amd.engine import Engine, load_model
+    from machserve_amd.sampling import SamplingParams
+    d = make_model_dir(tmp_path, "A")
+    w, sizes = read_for_plain(d)
+    prompts = [random_prompt(n, 512, 60 + n) for n in (20, 25)]
+
+    def run(pages):
+        lm = load_model(d, dtype="float32", device="cpu", page_size=16, num_pages=pages, max_requests=2, ops=EmulatedOps())
+        eng = Engine(lm, max_batch_tokens=64)
+        ids = [eng.add(p, 14, SamplingParams(temperature=1.0, top_k=50, seed=11 + i)) for i, p in enumerate(prompts)]
+        done = eng.run()
+        return [done[i].generated for i in ids], sum(done[i].preemptions for i in ids)
+
+    roomy, n0 = run(16)
+    tight, n1 = run(5)
+    assert n0 == 0 and n1 > 0, "the small pool must force a preemption"
+    assert roomy == tight
+    # and the tokens are the CPU mirror's draws on the plain model's logits
+    seq, st = list(prompts[0]), 11
+    for t in roomy[0][:4]:
+        tok, st = P.sample(P.forward(w, sizes, seq)[-1].numpy(), 1.0, 50, 1.0, st)
+        assert tok == t
+        seq.append(tok)

@@ -1,0 +1,257 @@
+"""The engine on the GPU through its entry points: greedy generation, long decoding, the
+first tokens of a sequence, the replay program, the command line, sampling, and each part
+of a layer alone."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import DEV, assert_close
+from plain import qwen2_plain as P
+from tiny_configs import CONFIGS, make_model_dir, random_prompt, read_for_plain
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def dirs(tmp_path_factory):
+    tmp = tmp_path_factory.mktemp("engine_models")
+    return {w: make_model_dir(tmp, w) for w in CONFIGS}
+
+
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_greedy_generation_through_the_entry_point(dirs, which):
+    import machserve_amd
+    w, sizes = read_for_plain(dirs[which])
+    prompts = [random_prompt(n, sizes["vocab"], 70 + n) for n in (1, 9, 40, 33)]
+    got = machserve_amd.generate(dirs[which], prompts, max_new=12, dtype="float32", page_size=16, capacity=3,
+                                 max_batch_tokens=24)
+    for p, g in zip(prompts, got):
+        assert g == P.greedy_generate(w, sizes, p, 12)
+
+
+def test_eos_stops_generation(dirs):
+    import machserve_amd
+    w, sizes = read_for_plain(dirs["A"])
+    p = random_prompt(11, 512, 3)
+    full = P.greedy_generate(w, sizes, p, 10)
+    got = machserve_amd.generate(dirs["A"], [p], max_new=10, dtype="float32", eos=full[4])
+    assert got[0] == full[:full.index(full[4]) + 1]
+
+
+def test_generation_under_page_pressure_equals_roomy_generation(dirs):
+    """Pages run out, the youngest request is preempted and recomputed; tokens do not change."""
+    from machserve_amd.engine import Engine
+    from machserve_amd.sampling import SamplingParams
+    prompts = [random_prompt(n, 1000, 90 + n) for n in (40, 50, 45)]
+
+    def run(pages, dtype):
+        eng = Engine.from_dir(dirs["B"], dtype=dtype, page_size=32, num_pages=pages, capacity=3, max_batch_tokens=64)
+        ids = [eng.add(p, 30, SamplingParams(temperature=0.8, top_p=0.95, seed=5 + i)) for i, p in enumerate(prompts)]
+        done = eng.run()
+        eng.loaded.cache.check()
+        return [done[i].generated for i in ids], sum(done[i].preemptions for i in ids)
+    roomy, n0 = run(12, "float32")
+    tight, n1 = run(5, "float32")
+    assert n0 == 0 and n1 > 0 and roomy == tight
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_long_decoding(dirs, dtype):
+    """One step of 8 tokens, then 400 single tokens across many pages: every position against
+    the plain model."""
+    from machserve_amd.engine import StepEntry, load_model
+    w, sizes = read_for_plain(dirs["A"])
+    toks = random_prompt(250, 512, 8)
+    ww = w if dtype == torch.float32 else {k: v.to(torch.bfloat16).float() if v.dim() == 2 else v for k, v in w.items()}
+    ref = P.forward(ww, sizes, toks)
+    lm = load_model(dirs["A"], dtype=dtype, device=DEV, page_size=16, num_pages=16)
+    slot = lm.cache.admit()
+    out = [lm.step([StepEntry(slot, toks[:8], list(range(8)))])]
+    for t in toks[8:]:
+        out.append(lm.step([StepEntry(slot, [t], [0])]))
+    got = torch.cat(out).float().cpu()
+    scale = ref.abs().max().item()
+    allowed = 2e-5 + 2e-5 * scale if dtype == torch.float32 else 3e-2 * scale
+    assert (got - ref).abs().max().item() <= allowed
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_first_tokens_of_a_sequence(dirs, which, dtype):
+    """Positions 0, 1, 2 alone and together: a one-token prompt, and the first rows of a portion."""
+    from machserve_amd.engine import StepEntry, load_model
+    w, sizes = read_for_plain(dirs[which])
+    ww = w if dtype == torch.float32 else {k: v.to(torch.bfloat16).float() if v.dim() == 2 else v for k, v in w.items()}
+    lm = load_model(dirs[which], dtype=dtype, device=DEV, page_size=16, num_pages=8)
+    toks = random_prompt(3, sizes["vocab"], 2)
+    ref = P.forward(ww, sizes, toks)
+    allowed = 2e-5 + 2e-5 * ref.abs().max().item() if dtype == torch.float32 else 3e-2 * ref.abs().max().item()
+    for cuts in ([1, 1, 1], [3], [1, 2], [2, 1]):
+        slot, i, out = lm.cache.admit(), 0, []
+        for c in cuts:
+            out.append(lm.step([StepEntry(slot, toks[i:i + c], list(range(c)))]))
+            i += c
+        lm.cache.release(slot)
+        assert (torch.cat(out).float().cpu() - ref).abs().max().item() <= allowed, cuts
+
+
+def test_wanted_places_select_rows(dirs):
+    from machserve_amd.engine import StepEntry, load_model
+    lm = load_model(dirs["B"], dtype="float32", device=DEV, page_size=32, num_pages=8)
+    a, b = lm.cache.admit(), lm.cache.admit()
+    ta, tb = random_prompt(10, 1000, 1), random_prompt(6, 1000, 2)
+    full = lm.step([StepEntry(a, ta, list(range(10))), StepEntry(b, tb, list(range(6)))])
+    lm.cache.release(a), lm.cache.release(b)
+    a, b = lm.cache.admit(), lm.cache.admit()
+    some = lm.step([StepEntry(a, ta, [9, 0]), StepEntry(b, tb, []), ])
+    assert some.shape == (2, 1000)
+    assert torch.equal(some[0], full[9]) and torch.equal(some[1], full[0])
+    assert lm.step([StepEntry(b, [5], [])]) is None
+
+
+def test_trace_run_program(dirs, tmp_path):
+    """bin/trace_run as a user runs it: JSON lines in, <step>.f32 files and 'done' lines out."""
+    w, sizes = read_for_plain(dirs["A"])
+    a, b = random_prompt(37, 512, 1), random_prompt(20, 512, 2)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:30], "want": [0, 29]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[30:32], "want": []}, {"id": "b", "tokens": b[:18], "want": [17]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[18:], "want": [0, 1]}], "end": ["b"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": a[32:], "want": [4]}], "end": ["a"]},
+    ]
+    out = tmp_path / "out"
+    for dtype in ("float32", "bfloat16"):
+        r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", dirs["A"], "--dtype", dtype,
+                            "--out", str(out / dtype), "--max-tokens", "128"],
+                           input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600)
+        assert r.returncode == 0, r.stderr
+        assert r.stdout.split() == ["done", "0", "done", "1", "done", "2", "done", "3"]
+        ra, rb = P.forward(w, sizes, a), P.forward(w, sizes, b)
+        want = {0: ra[[0, 29]], 1: rb[[17]], 2: rb[[18, 19]], 3: ra[[36]]}
+        tolr = 2e-5 if dtype == "float32" else 4e-2
+        for s, ref in want.items():
+            got = torch.from_numpy(np.fromfile(out / dtype / f"{s}.f32", dtype="<f4").reshape(-1, 512))
+            assert got.shape == ref.shape
+            assert (got - ref).abs().max() <= tolr * (1 + ref.abs().max())
+
+
+def test_command_line(dirs, tmp_path):
+    w, sizes = read_for_plain(dirs["A"])
+    p = random_prompt(7, 512, 9)
+    r = subprocess.run([sys.executable, "-m", "machserve_amd", "--model", dirs["A"], "--dtype", "f32", "--prompt-ids",
+                        ",".join(map(str, p)), "--max-new", "5", "--tpp", "16", "--json"],
+                       capture_output=True, text=True, cwd=ROOT, timeout=600)
+    assert r.returncode == 0, r.stderr
+    rec = json.loads(r.stdout.strip().splitlines()[-1])
+    assert rec["generated"] == P.greedy_generate(w, sizes, p, 5) and rec["finish_reason"] == "length"
+    cfg = tmp_path / "cfg.json"
+    cfg.write_text(json.dumps(CONFIGS["B"]))
+    r = subprocess.run([sys.executable, "-m", "machserve_amd", "--random-config", str(cfg), "--weights-seed", "1",
+                        "--dtype", "f32", "--prompt-ids", "1,2,3", "--prompt-ids", "4,5", "--max-new", "4", "--tpp", "32",
+                        "--temperature", "0.7", "--seed", "3"], capture_output=True, text=True, cwd=ROOT, timeout=600)
+    assert r.returncode == 0, r.stderr
+    assert [len(l.split()) for l in r.stdout.strip().splitlines()] == [4, 4]
+
+
+# ---------------------------------------------------------------------------- each part alone
+
+def _runtime(dtype):
+    from machserve_amd.kernels import get_ops
+    from machserve_amd.parts import Runtime
+    return Runtime(torch.device(DEV), dtype, get_ops(dtype, DEV))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part_alone(dtype):
+    from machserve_amd.config import NormSpec
+    from machserve_amd.parts import NORMS
+    part = NORMS.build(NormSpec("rmsnorm", 200, 1e-5), _runtime(dtype))
+    assert [(d.name, d.shape, d.role) for d in part.tensor_decls()] == [("weight", (200,), "vector")]
+    w = 1 + 0.1 * torch.randn(200)
+    part.load({"weight": w.to(DEV)})
+    x = torch.randn(9, 200) * 3
+    assert_close(part.forward(x.to(DEV)), P.rms_norm(x, w, 1e-5), dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_part_alone(dtype):
+    from machserve_amd.config import GatedMlpSpec
+    from machserve_amd.parts import FEED_FORWARDS
+    part = FEED_FORWARDS.build(GatedMlpSpec("gated_mlp", 72, 200), _runtime(dtype))
+    t = {"gate.weight": torch.randn(200, 72) * 0.2, "up.weight": torch.randn(200, 72) * 0.2, "down.weight": torch.randn(72, 200) * 0.1}
+    t = {k: v.to(dtype) for k, v in t.items()}
+    part.load({k: v.to(DEV) for k, v in t.items()})
+    h = torch.randn(11, 72).to(dtype)
+    x = torch.randn(11, 72)
+    xd = x.to(DEV).clone()
+    part.forward(h.to(DEV), xd, None)
+    ref = x + P.swiglu(h.float(), t["gate.weight"].float(), t["up.weight"].float(), t["down.weight"].float())
+    assert_close(xd, ref, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window,shared", [(None, False), (7, False), (None, True)])
+def test_attention_part_alone(dtype, window, shared):
+    """The mixer with its own cache manager: a portion, then single tokens, against the plain
+    attention block over the whole sequence.  With ``shared`` a second layer reads the first
+    layer's cache and writes none."""
+    from machserve_amd.cache import CacheManager, DeviceCache
+    from machserve_amd.config import AttentionSpec, RotarySpec
+    from machserve_amd.engine.step import StepEntry, StepFunction
+    from machserve_amd.parts import MIXERS
+    rt = _runtime(dtype)
+    H, KV, hd, d, T = 6, 2, 32, 80, 45
+    names = {k: k for k in ("q.weight", "k.weight", "v.weight", "o.weight", "q.bias", "k.bias", "v.bias")}
+    spec = AttentionSpec("attention", d, H, KV, hd, RotarySpec("rotary", hd, 1e4), window=window, tensors=names)
+    part = MIXERS.build(spec, rt)
+    g = torch.Generator().manual_seed(5)
+    t = {"q.weight": torch.randn(H * hd, d, generator=g) * 0.1, "k.weight": torch.randn(KV * hd, d, generator=g) * 0.1,
+         "v.weight": torch.randn(KV * hd, d, generator=g) * 0.1, "o.weight": torch.randn(d, H * hd, generator=g) * 0.1,
+         "q.bias": torch.randn(H * hd, generator=g) * 0.1, "k.bias": torch.randn(KV * hd, generator=g) * 0.1,
+         "v.bias": None}
+    t = {k: (v.to(dtype) if v is not None and v.dim() == 2 else v) for k, v in t.items()}
+    part.load({k: (v.to(DEV) if v is not None else None) for k, v in t.items()})
+    parts = [part]
+    if shared:
+        spec2 = AttentionSpec("attention", d, H, KV, hd, RotarySpec("rotary", hd, 1e4), kv_source=0, tensors=names)
+        part2 = MIXERS.build(spec2, rt)
+        assert [dd.name for dd in part2.tensor_decls()] == ["q.weight", "o.weight", "q.bias"]
+        part2.load({k: (v.to(DEV) if v is not None else None) for k, v in t.items()})
+        parts.append(part2)
+    cache = CacheManager([p.cache_request() for p in parts], 16, 8, 2)
+    dc = DeviceCache(cache, dtype, rt.device)
+    for i, p in enumerate(parts):
+        p.bind_cache(dc.binding(i))
+
+    class OneLayer:  # just enough of a model for the step function's context builder
+        vocab = 100
+        class spec:
+            max_positions = 1000
+        def attention_rows_per_token(self):
+            return [H // KV]
+    sf = StepFunction(OneLayer(), cache, rt)
+    h = torch.randn(T, d, generator=g).to(dtype)
+    slot = cache.admit()
+    outs = [torch.zeros(T, d, device=DEV) for _ in parts]
+    i = 0
+    for c in [20, 1, 1, 13, 1, 9]:
+        cache.extend(slot, c)
+        ctx = sf.build_context([StepEntry(slot, [0] * c, [])])
+        for p, o in zip(parts, outs):
+            xs = torch.zeros(c, d, device=DEV)
+            p.forward(h[i:i + c].to(DEV).contiguous(), xs, ctx)
+            o[i:i + c] = xs
+        cache.commit(slot, c)
+        i += c
+    w = {"p.q_proj.weight": t["q.weight"].float(), "p.k_proj.weight": t["k.weight"].float(), "p.v_proj.weight": t["v.weight"].float(),
+         "p.o_proj.weight": t["o.weight"].float(), "p.q_proj.bias": t["q.bias"], "p.k_proj.bias": t["k.bias"]}
+    sizes = {"heads": H, "kv_heads": KV, "head_dim": hd, "theta": 1e4}
+    ref = P.attention_block(h.float(), w, "p.", torch.arange(T), sizes, window)
+    for o in outs:
+        assert_close(o, ref, dtype)
