@@ -226,6 +226,218 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
     }
 }
 
+
+// ---------------------------------------------------------------------------------------
+// Decode attention: every request of the step has one row.  The g query heads of one KV
+// head are the rows of one MFMA tile (g <= 16), so each key and value is read once per KV
+// head.  The keys of a request are cut into `nsplit` contiguous ranges (grid z), and inside
+// a block each of the four waves takes every fourth key tile, reading K and V^T straight
+// from the pages into fragments (nothing is shared between waves, so nothing is staged in
+// LDS).  Waves combine through LDS; blocks write (max, sum, unnormalised output) per split,
+// and a second kernel merges the splits.
+// Role in the reference: attn_decode_batched_f16_gqa (crates/mach-model/src/kernels.rs:2905-3036).
+
+struct DecodeArgs {
+    const elem_t* q;         // [S, H, hd]
+    const elem_t* kpool;
+    const elem_t* vpool;
+    elem_t* out;             // [S, H * hd] (written when nsplit == 1)
+    float* part_o;           // [S, H, nsplit, hd]
+    float* part_ml;          // [S, H, nsplit, 2]
+    const int* block_table;  // [S, table_stride]
+    const int* seq_pos0;     // [S] position of the row = number of keys before it
+    int table_stride, H, KV, hd, ps, window, nsplit;
+    float scale;
+};
+
+__global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
+    __shared__ float sm_o[3][HDT][16];
+    __shared__ float sm_m[3][16], sm_l[3][16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, grp = lane >> 4;
+    const int s = blockIdx.x, kvh = blockIdx.y, sp = blockIdx.z;
+    const int g = a.H / a.KV, hd = a.hd, ps = a.ps;
+    const int pos = a.seq_pos0[s], kv_len = pos + 1;
+    const int lo_key = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+    const int* table = a.block_table + (size_t)s * a.table_stride;
+    const bool valid = r16 < g;
+    const int head = kvh * g + (valid ? r16 : 0);
+
+    const int t_lo = lo_key / BKV, t_hi = ceil_div(kv_len, BKV);
+    const int tps = ceil_div(t_hi - t_lo, a.nsplit);
+    const int t0 = t_lo + sp * tps, t1 = min(t_hi, t0 + tps);
+
+    Frag qf[NKS];
+    {
+        const elem_t* qrow = a.q + ((size_t)s * a.H + head) * hd;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            const int d0 = ks * 32 + grp * 8;
+            qf[ks] = (valid && d0 < hd) ? frag_load(qrow + d0) : frag_zero();
+        }
+    }
+    f32x4 acc_o[ND];
+#pragma unroll
+    for (int i = 0; i < ND; ++i) acc_o[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m_run = NEG_BIG, l_run = 0.f;
+
+    for (int t = t0 + wave; t < t1; t += 4) {
+        const int kt0 = t * BKV;
+        f32x4 sc[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            sc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            const int key = kt0 + nt * 16 + r16;
+            const int page = key < kv_len ? table[key / ps] : -1;
+            const elem_t* krow = a.kpool + (((size_t)max(page, 0) * a.KV + kvh) * ps + key % ps) * hd;
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+                const int d0 = ks * 32 + grp * 8;
+                Frag kf = (page >= 0 && d0 < hd) ? frag_load(krow + d0) : frag_zero();
+                mma_16x16x32(sc[nt], kf, qf[ks]);
+            }
+        }
+        float tmax = NEG_BIG;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = kt0 + nt * 16 + grp * 4 + i;
+                const bool ok = valid && key <= pos && key >= lo_key;
+                const float v = ok ? sc[nt][i] * a.scale : -INFINITY;
+                sc[nt][i] = v;
+                tmax = fmaxf(tmax, v);
+            }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+        const float m_new = fmaxf(m_run, tmax);
+        const float alpha = exp_f(m_run - m_new);
+        float psum = 0.f;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float p = exp_f(sc[nt][i] - m_new);
+                sc[nt][i] = p;
+                psum += p;
+            }
+        psum += __shfl_xor(psum, 16, WAVE);
+        psum += __shfl_xor(psum, 32, WAVE);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc_o[dt][i] *= alpha;
+#pragma unroll
+        for (int pp = 0; pp < NTP; ++pp) {
+            Frag pf;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                pf.v[i] = from_f32<elem_t>(sc[2 * pp][i]);
+                pf.v[4 + i] = from_f32<elem_t>((2 * pp + 1 < NT) ? sc[(2 * pp + 1) % NT][i] : 0.f);
+            }
+            // the two 4-key groups this lane multiplies: same 16-key tile -> same page
+            const int ka = kt0 + (2 * pp) * 16 + grp * 4, kb = ka + 16;
+            const int pa = ka < kv_len ? table[ka / ps] : -1;
+            const int pb = (2 * pp + 1 < NT && kb < kv_len) ? table[kb / ps] : -1;
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt) {
+                const int d = dt * 16 + r16;
+                Frag vf;
+                if (pa >= 0 && d < hd) {
+                    const elem_t* v0 = a.vpool + (((size_t)pa * a.KV + kvh) * hd + d) * ps + ka % ps;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) vf.v[i] = v0[i];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) vf.v[i] = from_f32<elem_t>(0.f);
+                }
+                if (pb >= 0 && d < hd) {
+                    const elem_t* v1 = a.vpool + (((size_t)pb * a.KV + kvh) * hd + d) * ps + kb % ps;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) vf.v[4 + i] = v1[i];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) vf.v[4 + i] = from_f32<elem_t>(0.f);
+                }
+                mma_16x16x32(acc_o[dt], vf, pf);
+            }
+        }
+    }
+
+    // waves 1..3 hand their state to wave 0
+    if (wave > 0) {
+        if (grp == 0) { sm_m[wave - 1][r16] = m_run; sm_l[wave - 1][r16] = l_run; }
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sm_o[wave - 1][dt * 16 + grp * 4 + i][r16] = acc_o[dt][i];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    float m_all = m_run;
+#pragma unroll
+    for (int w = 0; w < 3; ++w) m_all = fmaxf(m_all, sm_m[w][r16]);
+    const float c0 = exp_f(m_run - m_all);
+    float l_all = l_run * c0;
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc_o[dt][i] *= c0;
+#pragma unroll
+    for (int w = 0; w < 3; ++w) {
+        const float c = exp_f(sm_m[w][r16] - m_all);
+        l_all += sm_l[w][r16] * c;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc_o[dt][i] += sm_o[w][dt * 16 + grp * 4 + i][r16] * c;
+    }
+    if (!valid) return;
+    if (a.nsplit == 1) {
+        const float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
+        elem_t* orow = a.out + ((size_t)s * a.H + head) * hd;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) {
+            const int d0 = dt * 16 + grp * 4;
+            if (d0 < hd) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) orow[d0 + i] = from_f32<elem_t>(acc_o[dt][i] * inv);
+            }
+        }
+    } else {
+        const size_t base = ((size_t)s * a.H + head) * a.nsplit + sp;
+        float* po = a.part_o + base * hd;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) {
+            const int d0 = dt * 16 + grp * 4;
+            if (d0 < hd) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) po[d0 + i] = acc_o[dt][i];
+            }
+        }
+        if (grp == 0) { a.part_ml[base * 2] = m_all; a.part_ml[base * 2 + 1] = l_all; }
+    }
+}
+
+// out[row, :] = sum_sp o_sp exp(m_sp - m) / sum_sp l_sp exp(m_sp - m), splits in order
+__global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                          elem_t* __restrict__ out, int hd, int nsplit) {
+    const size_t row = blockIdx.x;  // (request, head)
+    const float* ml = part_ml + row * nsplit * 2;
+    float m = NEG_BIG;
+    for (int sp = 0; sp < nsplit; ++sp) m = fmaxf(m, ml[sp * 2]);
+    float l = 0.f;
+    for (int sp = 0; sp < nsplit; ++sp) l += ml[sp * 2 + 1] * exp_f(ml[sp * 2] - m);
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    for (int d = threadIdx.x; d < hd; d += 64) {
+        float o = 0.f;
+        for (int sp = 0; sp < nsplit; ++sp) o += part_o[(row * nsplit + sp) * hd + d] * exp_f(ml[sp * 2] - m);
+        out[row * hd + d] = from_f32<elem_t>(o * inv);
+    }
+}
+
 }  // namespace ms
 
 using namespace ms;
@@ -251,3 +463,26 @@ extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
 }
 
 extern "C" int MS_CAT(ms_attention_rows_per_block_nd, MS_ATTN_ND)() { return ROWS_PER_BLOCK; }
+
+// Attention of a step in which every request has exactly one row (row s = request s).
+// part_o [S, H, nsplit, hd] and part_ml [S, H, nsplit, 2] are float workspaces (unused when
+// nsplit == 1).  Needs H / KV <= 16.
+extern "C" int MS_CAT(ms_decode_attention_nd, MS_ATTN_ND)(
+    const void* q, const void* kpool, const void* vpool, void* out, float* part_o, float* part_ml, const int* block_table,
+    int table_stride, const int* seq_pos0, int S, int H, int KV, int hd, int ps, int window, int nsplit, float scale,
+    hipStream_t stream) {
+    MS_REQUIRE(S > 0, "decode attention: no rows");
+    MS_REQUIRE(hd % 16 == 0 && hd > 0 && hd <= HDT, "decode attention: head size %d does not fit this tile of %d", hd, HDT);
+    MS_REQUIRE(KV > 0 && H % KV == 0 && H / KV <= 16, "decode attention: %d heads over %d key/value heads (at most 16 each)", H, KV);
+    MS_REQUIRE(ps % 16 == 0 && ps > 0, "decode attention: page size %d must be a multiple of 16", ps);
+    MS_REQUIRE(nsplit >= 1 && nsplit <= 65535 && (nsplit == 1 || (part_o && part_ml)), "decode attention: %d splits", nsplit);
+    DecodeArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, (elem_t*)out, part_o, part_ml, block_table,
+                 seq_pos0, table_stride, H, KV, hd, ps, window, nsplit, scale};
+    hipLaunchKernelGGL(decode_attention_kernel, dim3((unsigned)S, (unsigned)KV, (unsigned)nsplit), dim3(256), 0, stream, a);
+    int rc = check_launch("decode_attention");
+    if (rc || nsplit == 1) return rc;
+    hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)(S * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit);
+    return check_launch("decode_merge");
+}
+
+extern "C" int MS_CAT(ms_attention_key_tile_nd, MS_ATTN_ND)() { return BKV; }

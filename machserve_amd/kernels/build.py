@@ -24,7 +24,7 @@ ARCH = "gfx950"
 FLAGS = ["-O3", f"--offload-arch={ARCH}", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
          "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 ELEM_DEFINE = {"bf16": "MS_ELEM_BF16", "f32": "MS_ELEM_F32"}
-CORE_SOURCES = ["runtime.hip", "gemm.hip", "elementwise.hip", "sampling.hip", "decode.hip"]
+CORE_SOURCES = ["runtime.hip", "gemm.hip", "skinny.hip", "elementwise.hip", "sampling.hip"]
 ATTENTION_TILES = (1, 2, 3, 4, 6, 8, 12, 16)  # head-size tiles in units of 16
 
 _lock = threading.Lock()
@@ -66,7 +66,7 @@ def _hipcc() -> str:
 
 def _sources_of(kind: str):
     if kind == "core":
-        return [s for s in CORE_SOURCES if os.path.exists(os.path.join(CSRC, s))]
+        return list(CORE_SOURCES)
     return ["runtime.hip", "attention.hip"]
 
 

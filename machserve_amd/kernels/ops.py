@@ -72,25 +72,46 @@ class HipOps:
         return x
 
     def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, rows: Optional[torch.Tensor] = None,
-                out_f32: bool = False) -> torch.Tensor:
+                out_f32: bool = False, partials: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Norm of ``x + sum(partials)`` (of its ``rows`` if given).  With ``partials [P, T, d]`` and
+        no ``rows`` the sum is also written back into ``x``."""
         T, d = x.shape
         self._want(x, torch.float32, "rmsnorm input")
         self._want(weight, torch.float32, "rmsnorm weight", d)
-        n = T
+        n, P = T, 0
         if rows is not None:
             self._want(rows, torch.int32, "rmsnorm rows")
             n = rows.numel()
+        if partials is not None:
+            P = partials.shape[0]
+            self._want(partials, torch.float32, "rmsnorm partial sums", P, T, d)
         out = torch.empty((n, d), dtype=torch.float32 if out_f32 else self.dtype, device=x.device)
-        self._check(self._core, self._core.ms_rmsnorm(_ptr(x), _ptr(rows), _ptr(weight), _ptr(out), _c_int(int(out_f32)),
-                                                      _c_int(n), _c_int(d), _c_float(eps), _stream()))
+        self._check(self._core, self._core.ms_rmsnorm(_ptr(x), _ptr(partials), _c_int(P), _c_int(T), _ptr(rows),
+                                                      _ptr(weight), _ptr(out), _c_int(int(out_f32)), _c_int(n), _c_int(d),
+                                                      _c_float(eps), _stream()))
         return out
 
-    def rope_kv_write(self, qkv: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[torch.Tensor],
-                      slot_map: Optional[torch.Tensor], kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor],
-                      H: int, KV: int, hd: int, page_size: int) -> torch.Tensor:
-        T, stride = qkv.shape
+    def add_partials(self, x: torch.Tensor, partials: torch.Tensor) -> None:
+        """``x += sum(partials)`` in order."""
+        T, d = x.shape
+        self._want(x, torch.float32, "stream")
+        self._want(partials, torch.float32, "partial sums", partials.shape[0], T, d)
+        self._check(self._core, self._core.ms_add_partials(_ptr(x), _ptr(partials), _c_int(partials.shape[0]), _c_int(T),
+                                                           _c_int(d), _stream()))
+
+    def rope_kv_write(self, qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
+                      inv_freq: Optional[torch.Tensor], slot_map: Optional[torch.Tensor], kpool: Optional[torch.Tensor],
+                      vpool: Optional[torch.Tensor], H: int, KV: int, hd: int, page_size: int) -> torch.Tensor:
+        """``qkv [P, T, stride]`` are partial sums of the q/k/v projection (see :meth:`linear_split`);
+        their sum plus ``bias`` is rotated (q and k) and written (k and v) into the pages.  Returns
+        q ``[T, H * hd]`` in the element type."""
+        if qkv.dim() == 2:
+            qkv = qkv.unsqueeze(0)
+        P, T, stride = qkv.shape
         self._want(qkv, torch.float32, "rope qkv")
         self._want(positions, torch.int32, "rope positions", T)
+        if bias is not None:
+            self._want(bias, torch.float32, "rope bias", stride)
         if inv_freq is not None:
             self._want(inv_freq, torch.float32, "rope inv_freq", hd // 2)
         if slot_map is not None:
@@ -100,8 +121,8 @@ class HipOps:
             self._want(vpool, self.dtype, "value pool", pages, KV, hd, page_size)
         q = torch.empty((T, H * hd), dtype=self.dtype, device=qkv.device)
         self._check(self._core, self._core.ms_rope_kv_write(
-            _ptr(qkv), _c_int(stride), _ptr(positions), _ptr(inv_freq), _ptr(slot_map), _ptr(q), _ptr(kpool), _ptr(vpool),
-            _c_int(T), _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), _stream()))
+            _ptr(qkv), _c_int(P), _ptr(bias), _c_int(stride), _ptr(positions), _ptr(inv_freq), _ptr(slot_map), _ptr(q),
+            _ptr(kpool), _ptr(vpool), _c_int(T), _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), _stream()))
         return q
 
     # ------------------------------------------------------------------ matrix products
@@ -113,10 +134,27 @@ class HipOps:
             raise KernelError(f"{what}: input has {K} columns, weight has {w.shape[1]}")
         return M, w.shape[0], K
 
+    SKINNY_ROWS = 64  # at most this many rows: the weight-streaming kernels
+
+    def linear_split(self, a: torch.Tensor, w: torch.Tensor, allow_partials: bool = True) -> torch.Tensor:
+        """Float32 ``[P, M, N]`` whose sum over P is ``a @ w.T``.  P depends on N and K only (1 for
+        more than 64 rows), so the consumer that adds the parts sees the same sums for a row
+        whatever else is in the batch."""
+        M, N, K = self._mm_operands(a, w, "linear_split")
+        if M > self.SKINNY_ROWS:
+            return self.linear(a, w, None, out_f32=True).unsqueeze(0)
+        P = self._core.ms_skinny_partials(_c_int(N), _c_int(K), _c_int(int(allow_partials)))
+        out = torch.empty((P, M, N), dtype=torch.float32, device=a.device)
+        self._check(self._core, self._core.ms_linear_skinny(_ptr(a), _ptr(w), _ptr(out), _c_int(M), _c_int(N), _c_int(K),
+                                                            _c_int(int(allow_partials)), _stream()))
+        return out
+
     def linear(self, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
                out_f32: bool = False) -> torch.Tensor:
-        """``a @ w.T (+ bias)``; 32-bit output on request (projections that feed the rotation, logits)."""
+        """``a @ w.T (+ bias)``; 32-bit output on request (logits)."""
         M, N, K = self._mm_operands(a, w, "linear")
+        if M <= self.SKINNY_ROWS and out_f32 and bias is None:
+            return self.linear_split(a, w, allow_partials=False)[0]
         if bias is not None:
             self._want(bias, torch.float32, "linear bias", N)
         out = torch.empty((M, N), dtype=torch.float32 if out_f32 else self.dtype, device=a.device)
@@ -124,12 +162,17 @@ class HipOps:
                                                      _c_int(M), _c_int(N), _c_int(K), _stream()))
         return out
 
-    def linear_residual(self, a: torch.Tensor, w: torch.Tensor, x: torch.Tensor) -> None:
-        """``x += a @ w.T`` in the 32-bit residual stream."""
+    def linear_residual(self, a: torch.Tensor, w: torch.Tensor, x: torch.Tensor) -> Optional[torch.Tensor]:
+        """``x += a @ w.T`` in the 32-bit residual stream.  With few rows the sum is not added here:
+        the float32 partial sums ``[P, M, N]`` are returned for the consumer (the next norm) to
+        fold in; otherwise None."""
         M, N, K = self._mm_operands(a, w, "linear_residual")
         self._want(x, torch.float32, "residual stream", M, N)
+        if M <= self.SKINNY_ROWS:
+            return self.linear_split(a, w)
         self._check(self._core, self._core.ms_linear_residual(_ptr(a), _ptr(w), _ptr(x), _c_int(M), _c_int(N), _c_int(K),
                                                               _stream()))
+        return None
 
     def linear_swiglu(self, a: torch.Tensor, w_gate_up: torch.Tensor, intermediate: int) -> torch.Tensor:
         """``silu(a @ gate.T) * (a @ up.T)`` with gate and up rows interleaved in blocks of 16
@@ -138,8 +181,9 @@ class HipOps:
         if N != 2 * ((intermediate + 15) // 16) * 16:
             raise KernelError(f"linear_swiglu: interleaved weight has {N} rows for intermediate size {intermediate}")
         out = torch.empty((M, intermediate), dtype=self.dtype, device=a.device)
-        self._check(self._core, self._core.ms_linear_swiglu(_ptr(a), _ptr(w_gate_up), _ptr(out), _c_int(M),
-                                                            _c_int(intermediate), _c_int(K), _stream()))
+        fn = self._core.ms_linear_swiglu_skinny if M <= self.SKINNY_ROWS else self._core.ms_linear_swiglu
+        self._check(self._core, fn(_ptr(a), _ptr(w_gate_up), _ptr(out), _c_int(M), _c_int(intermediate), _c_int(K),
+                                   _stream()))
         return out
 
     # ------------------------------------------------------------------ attention
@@ -148,7 +192,8 @@ class HipOps:
         if nd not in self._attn:
             lib = self._load(build.ensure_library("attention", self.elem, nd))
             self._attn[nd] = (lib, getattr(lib, f"ms_paged_attention_nd{nd}"),
-                              getattr(lib, f"ms_attention_rows_per_block_nd{nd}")())
+                              getattr(lib, f"ms_attention_rows_per_block_nd{nd}")(),
+                              getattr(lib, f"ms_decode_attention_nd{nd}"), getattr(lib, f"ms_attention_key_tile_nd{nd}")())
         return self._attn[nd]
 
     def attention_rows_per_block(self, hd: int) -> int:
@@ -158,7 +203,7 @@ class HipOps:
                         seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_pos0: torch.Tensor,
                         work: torch.Tensor, H: int, KV: int, hd: int, page_size: int, window: Optional[int],
                         scale: float) -> torch.Tensor:
-        lib, fn, _ = self._attention_lib(hd)
+        lib, fn = self._attention_lib(hd)[:2]
         T = q.shape[0]
         self._want(q, self.dtype, "attention q", T, H * hd)
         pages = kpool.shape[0]
@@ -178,6 +223,39 @@ class HipOps:
                             _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_pos0), _ptr(work), _c_int(work.shape[0]),
                             _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), _c_int(window or 0), _c_float(scale),
                             _stream()))
+        return out
+
+    DECODE_MAX_GROUP = 16  # query heads per key/value head the decode kernel takes
+
+    def decode_attention(self, q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
+                         seq_pos0: torch.Tensor, H: int, KV: int, hd: int, page_size: int, window: Optional[int],
+                         scale: float) -> torch.Tensor:
+        """Attention of a step in which request ``s`` has the single row ``s``.  The keys are cut
+        into splits so that the grid fills the chip; how many follows from the number of
+        requests and the width of the block table only."""
+        lib, _, _, fn, key_tile = self._attention_lib(hd)
+        S = q.shape[0]
+        self._want(q, self.dtype, "attention q", S, H * hd)
+        pages = kpool.shape[0]
+        self._want(kpool, self.dtype, "key pool", pages, KV, page_size, hd)
+        self._want(vpool, self.dtype, "value pool", pages, KV, hd, page_size)
+        self._want(block_table, torch.int32, "block table")
+        if block_table.dim() != 2 or block_table.shape[0] != S:
+            raise KernelError(f"attention: block table {tuple(block_table.shape)} for {S} requests")
+        self._want(seq_pos0, torch.int32, "seq_pos0", S)
+        if H // KV > self.DECODE_MAX_GROUP:
+            raise KernelError(f"decode attention: {H // KV} heads per key/value head, at most {self.DECODE_MAX_GROUP}")
+        span = block_table.shape[1] * page_size if not window else min(block_table.shape[1] * page_size, window + key_tile)
+        tiles = max(1, -(-span // key_tile))
+        nsplit = max(1, min(-(-1024 // (S * KV)), -(-tiles // 4)))
+        out = torch.empty((S, H * hd), dtype=self.dtype, device=q.device)
+        part_o = part_ml = None
+        if nsplit > 1:
+            part_o = torch.empty((S, H, nsplit, hd), dtype=torch.float32, device=q.device)
+            part_ml = torch.empty((S, H, nsplit, 2), dtype=torch.float32, device=q.device)
+        self._check(lib, fn(_ptr(q), _ptr(kpool), _ptr(vpool), _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(block_table),
+                            _c_int(block_table.shape[1]), _ptr(seq_pos0), _c_int(S), _c_int(H), _c_int(KV), _c_int(hd),
+                            _c_int(page_size), _c_int(window or 0), _c_int(nsplit), _c_float(scale), _stream()))
         return out
 
     # ------------------------------------------------------------------ sampling

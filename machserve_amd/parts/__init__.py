@@ -1,4 +1,4 @@
-from .base import (Block, FeedForward, GroupView, Mixer, Norm, PagedKVRequest, Part, PositionEncoding, Runtime,
+from .base import (Block, FeedForward, GroupView, Mixer, Norm, PagedKVRequest, Part, PositionEncoding, ResidualStream, Runtime,
                    SharedKVRequest, StateRequest, StepContext, TensorDecl)
 from .registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, register_block, register_feed_forward,
                        register_mixer, register_norm, register_position_encoding)
@@ -6,6 +6,6 @@ from . import norm, rotary, attention, feed_forward, block  # noqa: F401  (regis
 from .model import DecoderModel, Embedding, Head
 
 __all__ = ["Block", "FeedForward", "GroupView", "Mixer", "Norm", "PagedKVRequest", "Part", "PositionEncoding",
-           "Runtime", "SharedKVRequest", "StateRequest", "StepContext", "TensorDecl", "BLOCKS", "FEED_FORWARDS",
+           "ResidualStream", "Runtime", "SharedKVRequest", "StateRequest", "StepContext", "TensorDecl", "BLOCKS", "FEED_FORWARDS",
            "MIXERS", "NORMS", "POSITION_ENCODINGS", "register_block", "register_feed_forward", "register_mixer",
            "register_norm", "register_position_encoding", "DecoderModel", "Embedding", "Head"]

@@ -65,20 +65,31 @@ class Attention(Mixer):
     def attention_rows_per_token(self):
         return self.spec.heads // self.spec.kv_heads
 
-    def forward(self, h, x, ctx):
+    def forward(self, h, stream, ctx):
         s, ops = self.spec, self.rt.ops
         view = ctx.groups[self.group]
-        qkv = ops.linear(h, self.w_qkv, self.b_qkv, out_f32=True)
+        qkv = ops.linear_split(h, self.w_qkv)  # [P, T, nq (+ 2 nkv)] partial sums, bias not yet added
         inv_freq = self.position.rotary_inv_freq() if self.position is not None else None
+        bias = self.b_qkv
         if self.position is not None and inv_freq is None:
-            T = qkv.shape[0]
-            q = qkv[:, :self.nq].unflatten(1, (s.heads, s.head_dim))
-            k = qkv[:, self.nq:self.nq + self.nkv].unflatten(1, (s.kv_heads, s.head_dim)) if self.writes_cache else None
+            # a position encoding the fused kernel does not know: finish the sums, let the part
+            # encode in place, then write without rotation
+            qkv = qkv.sum(0, keepdim=True)
+            if bias is not None:
+                qkv += bias
+                bias = None
+            q = qkv[0, :, :self.nq].unflatten(1, (s.heads, s.head_dim))
+            k = qkv[0, :, self.nq:self.nq + self.nkv].unflatten(1, (s.kv_heads, s.head_dim)) if self.writes_cache else None
             self.position.apply(q, k, ctx)
-        q = ops.rope_kv_write(qkv, ctx.positions, inv_freq, view.slot_map if self.writes_cache else None,
+        q = ops.rope_kv_write(qkv, bias, ctx.positions, inv_freq, view.slot_map if self.writes_cache else None,
                               self.kpool if self.writes_cache else None, self.vpool if self.writes_cache else None,
                               s.heads, s.kv_heads, s.head_dim, view.page_size)
-        o = ops.paged_attention(q, self.kpool, self.vpool, view.block_table, ctx.seq_q_start, ctx.seq_q_len,
-                                ctx.seq_pos0, ctx.attention_work[self.attention_rows_per_token()], s.heads, s.kv_heads,
-                                s.head_dim, view.page_size, s.window, self.scale)
-        ops.linear_residual(o, self.w_o, x)
+        g = self.attention_rows_per_token()
+        if ctx.decode_only and g <= ops.DECODE_MAX_GROUP:
+            o = ops.decode_attention(q, self.kpool, self.vpool, view.block_table, ctx.seq_pos0, s.heads, s.kv_heads,
+                                     s.head_dim, view.page_size, s.window, self.scale)
+        else:
+            o = ops.paged_attention(q, self.kpool, self.vpool, view.block_table, ctx.seq_q_start, ctx.seq_q_len,
+                                    ctx.seq_pos0, ctx.attention_work[g], s.heads, s.kv_heads, s.head_dim, view.page_size,
+                                    s.window, self.scale)
+        stream.add_linear(o, self.w_o)

@@ -88,6 +88,36 @@ class StepContext:
     decode_only: bool = False
 
 
+class ResidualStream:
+    """The 32-bit residual stream ``x [T, width]`` and, possibly, sums that are still to be added
+    to it.  A product with few rows leaves its result as partial sums; the norm that reads
+    the stream next adds them in the same kernel, which saves a pass over the stream."""
+
+    def __init__(self, x: torch.Tensor, ops):
+        self.x = x
+        self.ops = ops
+        self.pending: Optional[torch.Tensor] = None  # float32 [P, T, width]
+
+    def add_linear(self, a: torch.Tensor, w: torch.Tensor) -> None:
+        """``x += a @ w.T``."""
+        self.flush()
+        self.pending = self.ops.linear_residual(a, w, self.x)
+
+    def add(self, y: torch.Tensor) -> None:
+        """``x += y`` for a part that computes its output by other means."""
+        self.flush()
+        self.x += y.to(self.x.dtype)
+
+    def flush(self) -> None:
+        if self.pending is not None:
+            self.ops.add_partials(self.x, self.pending)
+            self.pending = None
+
+    def value(self) -> torch.Tensor:
+        self.flush()
+        return self.x
+
+
 class Part:
     def __init__(self, spec, rt: Runtime):
         self.spec = spec
@@ -102,8 +132,9 @@ class Part:
 
 
 class Norm(Part):
-    def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None, out_f32: bool = False) -> torch.Tensor:
-        """Normalised copy of the 32-bit stream ``x`` (of its ``rows`` if given), in the element type."""
+    def forward(self, stream: ResidualStream, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Normalised copy of the stream (of its ``rows`` if given), in the element type.  Pending
+        sums of the stream are folded in."""
         raise NotImplementedError
 
 
@@ -132,14 +163,15 @@ class Mixer(Part):
         """Query heads per KV head if the mixer needs attention work lists, else None."""
         return None
 
-    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
-        """Add the mixer's output for the normalised input ``h`` into the stream ``x``."""
+    def forward(self, h: torch.Tensor, stream: ResidualStream, ctx: StepContext) -> None:
+        """Add the mixer's output for the normalised input ``h`` into the stream
+        (``stream.add_linear`` for a final projection, ``stream.add`` for a finished tensor)."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
-    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
-        """Add the feed-forward's output for the normalised input ``h`` into the stream ``x``."""
+    def forward(self, h: torch.Tensor, stream: ResidualStream, ctx: StepContext) -> None:
+        """Add the feed-forward's output for the normalised input ``h`` into the stream."""
         raise NotImplementedError
 
 
@@ -153,5 +185,5 @@ class Block:
     def parts(self):
         return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
 
-    def forward(self, x: torch.Tensor, ctx: StepContext) -> None:
+    def forward(self, stream: ResidualStream, ctx: StepContext) -> None:
         raise NotImplementedError

@@ -8,6 +8,6 @@ from .registry import register_block
 
 @register_block("prenorm")
 class PreNormBlock(Block):
-    def forward(self, x, ctx):
-        self.mixer.forward(self.mixer_norm.forward(x), x, ctx)
-        self.feed_forward.forward(self.feed_forward_norm.forward(x), x, ctx)
+    def forward(self, stream, ctx):
+        self.mixer.forward(self.mixer_norm.forward(stream), stream, ctx)
+        self.feed_forward.forward(self.feed_forward_norm.forward(stream), stream, ctx)

@@ -25,7 +25,6 @@ class GatedMlp(FeedForward):
         self.w_gate_up = interleave_gate_up(t["gate.weight"], t["up.weight"])
         self.w_down = t["down.weight"]
 
-    def forward(self, h, x, ctx):
-        ops = self.rt.ops
-        a = ops.linear_swiglu(h, self.w_gate_up, self.spec.intermediate)
-        ops.linear_residual(a, self.w_down, x)
+    def forward(self, h, stream, ctx):
+        a = self.rt.ops.linear_swiglu(h, self.w_gate_up, self.spec.intermediate)
+        stream.add_linear(a, self.w_down)

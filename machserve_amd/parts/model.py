@@ -10,7 +10,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..config.specs import ModelSpec
-from .base import Block, Part, Runtime, StepContext, TensorDecl
+from .base import Block, Part, ResidualStream, Runtime, StepContext, TensorDecl
 from .registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
 
 
@@ -96,9 +96,9 @@ class DecoderModel:
     def forward(self, ctx: StepContext) -> Optional[torch.Tensor]:
         """Run the step's rows through the layers in ``order``; float32 logits ``[W, vocab]`` of
         the wanted rows, or None when none is wanted."""
-        x = self.embedding.forward(ctx.tokens)
+        stream = ResidualStream(self.embedding.forward(ctx.tokens), self.rt.ops)
         for i in self.order:
-            self.blocks[i].forward(x, ctx)
+            self.blocks[i].forward(stream, ctx)
         if ctx.want_rows.numel() == 0:
             return None
-        return self.head.forward(self.final_norm.forward(x, rows=ctx.want_rows))
+        return self.head.forward(self.final_norm.forward(stream, rows=ctx.want_rows))

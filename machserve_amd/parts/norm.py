@@ -14,5 +14,8 @@ class RMSNorm(Norm):
     def load(self, tensors):
         self.weight = tensors["weight"]
 
-    def forward(self, x, rows=None, out_f32=False):
-        return self.rt.ops.rmsnorm(x, self.weight, self.spec.eps, rows, out_f32)
+    def forward(self, stream, rows=None):
+        h = self.rt.ops.rmsnorm(stream.x, self.weight, self.spec.eps, rows, False, stream.pending)
+        if rows is None:
+            stream.pending = None  # the kernel wrote the sum back
+        return h

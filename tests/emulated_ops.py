@@ -27,8 +27,14 @@ class EmulatedOps:
     def embed(self, tokens, table):
         return table[tokens.long()].float()
 
-    def rmsnorm(self, x, weight, eps, rows=None, out_f32=False):
-        src = x if rows is None else x[rows.long()]
+    SKINNY_ROWS = 64
+    DECODE_MAX_GROUP = 16
+
+    def rmsnorm(self, x, weight, eps, rows=None, out_f32=False, partials=None):
+        full = x if partials is None else x + partials.sum(0)
+        if partials is not None and rows is None:
+            x.copy_(full)
+        src = full if rows is None else full[rows.long()]
         y = src * (1.0 / torch.sqrt((src * src).sum(-1, keepdim=True) / src.shape[-1] + eps)) * weight
         return y if out_f32 else self._r(y)
 
@@ -38,8 +44,21 @@ class EmulatedOps:
             y = y + bias
         return y if out_f32 else self._r(y)
 
+    def add_partials(self, x, partials):
+        x += partials.sum(0)
+
+    def linear_split(self, a, w, allow_partials=True):
+        y = a.float() @ w.float().t()
+        if a.shape[0] <= self.SKINNY_ROWS and allow_partials:  # two parts, to exercise the consumers
+            r = torch.randn(y.shape, generator=torch.Generator().manual_seed(0))
+            return torch.stack([y - r, r])
+        return y.unsqueeze(0)
+
     def linear_residual(self, a, w, x):
+        if a.shape[0] <= self.SKINNY_ROWS:
+            return self.linear_split(a, w)
         x += a.float() @ w.float().t()
+        return None
 
     def linear_swiglu(self, a, w_gate_up, intermediate):
         Ip = w_gate_up.shape[0] // 2
@@ -48,7 +67,10 @@ class EmulatedOps:
         up = a.float() @ w[:, 1].reshape(Ip, -1).t()
         return self._r((gate / (1.0 + torch.exp(-gate)) * up)[:, :intermediate])
 
-    def rope_kv_write(self, qkv, positions, inv_freq, slot_map, kpool, vpool, H, KV, hd, page_size):
+    def rope_kv_write(self, qkv, bias, positions, inv_freq, slot_map, kpool, vpool, H, KV, hd, page_size):
+        qkv = qkv if qkv.dim() == 2 else qkv.sum(0)
+        if bias is not None:
+            qkv = qkv + bias
         T = qkv.shape[0]
         half = hd // 2
         if inv_freq is not None:
@@ -101,6 +123,13 @@ class EmulatedOps:
                     done.add((qs + tok, h))
         assert len(done) == T * H, "the work list does not cover every row and head"
         return self._r(out)
+
+    def decode_attention(self, q, kpool, vpool, block_table, seq_pos0, H, KV, hd, page_size, window, scale):
+        S = q.shape[0]
+        ar = torch.arange(S, dtype=torch.int32)
+        work = torch.stack([ar, torch.zeros_like(ar)], 1)
+        return self.paged_attention(q, kpool, vpool, block_table, ar, torch.ones_like(ar), seq_pos0, work, H, KV, hd,
+                                    page_size, window, scale)
 
     def sample(self, logits, temperature, top_k, top_p, state):
         from plain.qwen2_plain import sample as plain_sample

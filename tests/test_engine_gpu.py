@@ -175,8 +175,9 @@ def test_norm_part_alone(dtype):
     assert [(d.name, d.shape, d.role) for d in part.tensor_decls()] == [("weight", (200,), "vector")]
     w = 1 + 0.1 * torch.randn(200)
     part.load({"weight": w.to(DEV)})
+    from machserve_amd.parts import ResidualStream
     x = torch.randn(9, 200) * 3
-    assert_close(part.forward(x.to(DEV)), P.rms_norm(x, w, 1e-5), dtype)
+    assert_close(part.forward(ResidualStream(x.to(DEV), part.rt.ops)), P.rms_norm(x, w, 1e-5), dtype)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -187,12 +188,15 @@ def test_feed_forward_part_alone(dtype):
     t = {"gate.weight": torch.randn(200, 72) * 0.2, "up.weight": torch.randn(200, 72) * 0.2, "down.weight": torch.randn(72, 200) * 0.1}
     t = {k: v.to(dtype) for k, v in t.items()}
     part.load({k: v.to(DEV) for k, v in t.items()})
-    h = torch.randn(11, 72).to(dtype)
-    x = torch.randn(11, 72)
-    xd = x.to(DEV).clone()
-    part.forward(h.to(DEV), xd, None)
-    ref = x + P.swiglu(h.float(), t["gate.weight"].float(), t["up.weight"].float(), t["down.weight"].float())
-    assert_close(xd, ref, dtype)
+    from machserve_amd.parts import ResidualStream
+    for rows in (11, 100):  # few rows: pending partial sums; many: added in the product's epilogue
+        h = torch.randn(rows, 72).to(dtype)
+        x = torch.randn(rows, 72)
+        stream = ResidualStream(x.to(DEV).clone(), part.rt.ops)
+        part.forward(h.to(DEV), stream, None)
+        assert (stream.pending is not None) == (rows <= 64)
+        ref = x + P.swiglu(h.float(), t["gate.weight"].float(), t["up.weight"].float(), t["down.weight"].float())
+        assert_close(stream.value(), ref, dtype)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -204,7 +208,7 @@ def test_attention_part_alone(dtype, window, shared):
     from machserve_amd.cache import CacheManager, DeviceCache
     from machserve_amd.config import AttentionSpec, RotarySpec
     from machserve_amd.engine.step import StepEntry, StepFunction
-    from machserve_amd.parts import MIXERS
+    from machserve_amd.parts import MIXERS, ResidualStream
     rt = _runtime(dtype)
     H, KV, hd, d, T = 6, 2, 32, 80, 45
     names = {k: k for k in ("q.weight", "k.weight", "v.weight", "o.weight", "q.bias", "k.bias", "v.bias")}
@@ -244,9 +248,9 @@ def test_attention_part_alone(dtype, window, shared):
         cache.extend(slot, c)
         ctx = sf.build_context([StepEntry(slot, [0] * c, [])])
         for p, o in zip(parts, outs):
-            xs = torch.zeros(c, d, device=DEV)
-            p.forward(h[i:i + c].to(DEV).contiguous(), xs, ctx)
-            o[i:i + c] = xs
+            stream = ResidualStream(torch.zeros(c, d, device=DEV), rt.ops)
+            p.forward(h[i:i + c].to(DEV).contiguous(), stream, ctx)
+            o[i:i + c] = stream.value()
         cache.commit(slot, c)
         i += c
     w = {"p.q_proj.weight": t["q.weight"].float(), "p.k_proj.weight": t["k.weight"].float(), "p.v_proj.weight": t["v.weight"].float(),

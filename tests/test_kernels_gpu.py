@@ -45,6 +45,18 @@ def test_rmsnorm(dtype, T, d, eps):
     rows = torch.tensor([T - 1, 0, T // 2], dtype=torch.int32)
     got = ops.rmsnorm(x.to(DEV), w.to(DEV), eps, rows.to(DEV), out_f32=True)
     assert_close(got, ref[rows.long()], torch.float32, "rmsnorm of gathered rows")
+    # pending sums are folded in, and written back when no rows are gathered
+    parts = rnd((3, T, d), torch.float32, 5)
+    total = x + parts.sum(0)
+    xd = x.to(DEV).clone()
+    assert_close(ops.rmsnorm(xd, w.to(DEV), eps, partials=parts.to(DEV)), P.rms_norm(total, w, eps), dtype, "norm of sums")
+    assert_close(xd, total, torch.float32, "sums written back")
+    xd = x.to(DEV).clone()
+    got = ops.rmsnorm(xd, w.to(DEV), eps, rows.to(DEV), True, parts.to(DEV))
+    assert_close(got, P.rms_norm(total, w, eps)[rows.long()], torch.float32, "gathered norm of sums")
+    assert torch.equal(xd.cpu(), x), "gathered rows leave the stream alone"
+    ops.add_partials(xd, parts.to(DEV))
+    assert_close(xd, total, torch.float32, "add_partials")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -59,12 +71,38 @@ def test_linear(dtype, M, N, K):
     assert_close(ops.linear(a.to(DEV), w.to(DEV), None), P.linear(a.double(), w.double()), dtype, "linear")
     x = rnd((M, N), torch.float32, 8)
     xd = x.to(DEV).clone()
-    ops.linear_residual(a.to(DEV), w.to(DEV), xd)
+    pending = ops.linear_residual(a.to(DEV), w.to(DEV), xd)
+    assert (pending is not None) == (M <= 64)
+    if pending is not None:
+        ops.add_partials(xd, pending)
     assert_close(xd, x.double() + P.linear(a.double(), w.double()), torch.float32 if dtype == torch.float32 else dtype, "linear_residual")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,I,K", [(1, 16, 8), (9, 160, 64), (70, 328, 192), (200, 4864, 896)])
+@pytest.mark.parametrize("M,N,K", [(1, 16, 8), (3, 1000, 200), (8, 896, 4864), (17, 1152, 896), (33, 130, 72),
+                                   (64, 9728, 896), (5, 40000, 136), (48, 896, 896)])
+def test_linear_few_rows(dtype, M, N, K):
+    """The weight-streaming kernels: partial sums that add up to the product, cut the same way
+    for every number of rows, and a row's sums do not depend on the other rows."""
+    ops = ops_for(dtype)
+    a, w = rnd((M, K), dtype, 21), rnd((N, K), dtype, 22, K ** -0.5)
+    ref = P.linear(a.double(), w.double())
+    parts = ops.linear_split(a.to(DEV), w.to(DEV))
+    assert parts.shape[1:] == (M, N)
+    assert_close(parts.sum(0), ref, torch.float32 if dtype == torch.float32 else dtype, "sum of partial sums")
+    whole = ops.linear_split(a.to(DEV), w.to(DEV), allow_partials=False)
+    assert whole.shape == (1, M, N)
+    assert_close(whole[0], ref, torch.float32 if dtype == torch.float32 else dtype, "one sum")
+    assert_close(ops.linear(a.to(DEV), w.to(DEV), None, out_f32=True), ref, torch.float32 if dtype == torch.float32 else dtype)
+    alone = ops.linear_split(a[M - 1:].to(DEV).contiguous(), w.to(DEV))
+    assert alone.shape[0] == parts.shape[0] and torch.equal(alone[:, 0], parts[:, M - 1]), "a row alone gives the same bits"
+    x = rnd((M, N), torch.float32, 23).to(DEV)
+    pend = ops.linear_residual(a.to(DEV), w.to(DEV), x)
+    assert pend is not None and torch.equal(pend, parts)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,I,K", [(1, 16, 8), (9, 160, 64), (70, 328, 192), (200, 4864, 896), (64, 4864, 896), (33, 264, 136)])
 def test_linear_swiglu(dtype, M, I, K):
     from machserve_amd.kernels import interleave_gate_up
     ops = ops_for(dtype)
@@ -88,18 +126,28 @@ def test_rope_kv_write(dtype, H, KV, hd, ps, theta):
     j = torch.arange(hd // 2, dtype=torch.float32)
     inv = 1.0 / torch.pow(torch.tensor(theta, dtype=torch.float32), 2.0 * j / hd)
     kp, vp = torch.zeros(pages, KV, ps, hd, dtype=dtype), torch.zeros(pages, KV, hd, ps, dtype=dtype)
-    q_ref = emu.rope_kv_write(qkv, pos, inv, perm, kp, vp, H, KV, hd, ps)
+    q_ref = emu.rope_kv_write(qkv, None, pos, inv, perm, kp, vp, H, KV, hd, ps)
     # the emulation's rotation against the plain model's
     q_plain = P.rope(qkv[:, :H * hd].view(T, H, hd), pos, theta).reshape(T, H * hd)
     assert_close(q_ref, q_plain, dtype, "emulated rotation")
     kd, vd = torch.zeros_like(kp).to(DEV), torch.zeros_like(vp).to(DEV)
-    q = ops.rope_kv_write(qkv.to(DEV), pos.to(DEV), inv.to(DEV), perm.to(DEV), kd, vd, H, KV, hd, ps)
+    q = ops.rope_kv_write(qkv.to(DEV), None, pos.to(DEV), inv.to(DEV), perm.to(DEV), kd, vd, H, KV, hd, ps)
     assert_close(q, q_plain, dtype, "q rotation")
     assert_close(kd, kp, dtype, "key pages")
     assert_close(vd, vp, dtype, "value pages")
     # without a table of frequencies nothing rotates
-    q0 = ops.rope_kv_write(qkv.to(DEV), pos.to(DEV), None, None, None, None, H, KV, hd, ps)
+    q0 = ops.rope_kv_write(qkv.to(DEV), None, pos.to(DEV), None, None, None, None, H, KV, hd, ps)
     assert_close(q0, qkv[:, :H * hd], dtype, "no rotation")
+    # three partial sums and a bias: the kernel adds them before it rotates
+    parts = torch.stack([qkv * 0.5, qkv * 0.25 - 1.0, qkv * 0.25 + 1.0])
+    bias = rnd(((H + 2 * KV) * hd,), torch.float32, 15)
+    kp2, vp2 = torch.zeros_like(kp), torch.zeros_like(vp)
+    q_ref2 = emu.rope_kv_write(qkv + bias, None, pos, inv, perm, kp2, vp2, H, KV, hd, ps)
+    kd.zero_(), vd.zero_()
+    q2 = ops.rope_kv_write(parts.to(DEV), bias.to(DEV), pos.to(DEV), inv.to(DEV), perm.to(DEV), kd, vd, H, KV, hd, ps)
+    assert_close(q2, q_ref2, dtype, "q from partial sums")
+    assert_close(kd, kp2, dtype, "key pages from partial sums")
+    assert_close(vd, vp2, dtype, "value pages from partial sums")
 
 
 def _attention_case(dtype, H, KV, hd, ps, window, seqs, seed, peak=False):
@@ -164,6 +212,47 @@ def test_attention_far_key_stands_out(dtype, window):
     seqs = [(700, 1), (0, 5), (400, 40)]
     got, ref = _attention_case(dtype, 8, 2, 64, 64, window, seqs, 300, peak=True)
     assert_close(got, ref, dtype, "attention with a far key that dominates")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,KV,hd,ps,window", [(4, 2, 16, 16, None), (6, 1, 32, 32, None), (5, 5, 48, 16, 40),
+                                               (14, 2, 64, 64, None), (16, 1, 80, 32, 100), (12, 2, 128, 64, None),
+                                               (2, 1, 256, 16, None), (14, 2, 64, 64, 1)])
+def test_decode_attention(dtype, H, KV, hd, ps, window):
+    """One row per request, contexts from 0 to a few thousand keys, scattered pages; against the
+    plain attention of the same rows, and against the general kernel."""
+    ops, emu = ops_for(dtype), EmulatedOps(dtype)
+    lens = [0, 1, ps - 1, ps, 130, 700, 2049] if hd < 256 else [0, 5, 300]
+    gen = torch.Generator().manual_seed(500 + hd)
+    n_pages = sum(-(-(c + 1) // ps) for c in lens) + 2
+    order = torch.randperm(n_pages, generator=gen).tolist()
+    kp, vp = rnd((n_pages, KV, ps, hd), dtype, 501), rnd((n_pages, KV, hd, ps), dtype, 502)
+    width = max(-(-(c + 1) // ps) for c in lens)
+    table = torch.full((len(lens), width), -1, dtype=torch.int32)
+    for i, c in enumerate(lens):
+        for p in range(-(-(c + 1) // ps)):
+            table[i, p] = order.pop()
+    S = len(lens)
+    q = rnd((S, H * hd), dtype, 503)
+    # one far key towers over the rest for the longest request's last head
+    c = lens[-1]
+    far = 3 if not window else max(0, c - window + 1)
+    qv = q[S - 1, (H - 1) * hd:].float()
+    kp[int(table[S - 1, far // ps]), KV - 1, far % ps, :] = (qv / qv.norm() * 8.0).to(dtype)
+    q[S - 1, (H - 1) * hd:] = (qv / qv.norm() * 8.0 * math.sqrt(hd) / 4).to(dtype)
+    pos0 = torch.tensor(lens, dtype=torch.int32)
+    ref = emu.decode_attention(q, kp, vp, table, pos0, H, KV, hd, ps, window, hd ** -0.5)
+    got = ops.decode_attention(q.to(DEV), kp.to(DEV), vp.to(DEV), table.to(DEV), pos0.to(DEV), H, KV, hd, ps, window, hd ** -0.5)
+    assert_close(got, ref, dtype, "decode attention")
+    ar = torch.arange(S, dtype=torch.int32)
+    work = torch.stack([ar, torch.zeros_like(ar)], 1).contiguous()
+    gen_out = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV), table.to(DEV), ar.to(DEV), torch.ones_like(ar).to(DEV),
+                                  pos0.to(DEV), work.to(DEV), H, KV, hd, ps, window, hd ** -0.5)
+    assert_close(got, gen_out.float().cpu(), dtype, "decode kernel against the general kernel")
+    # a request alone (other split count) agrees within rounding
+    one = ops.decode_attention(q[S - 1:].to(DEV).contiguous(), kp.to(DEV), vp.to(DEV), table[S - 1:].to(DEV).contiguous(),
+                               pos0[S - 1:].to(DEV), H, KV, hd, ps, window, hd ** -0.5)
+    assert_close(one, ref[S - 1:], dtype, "decode attention of one request")
 
 
 def test_attention_equals_library_attention_without_rotation_or_paging():
