@@ -63,7 +63,8 @@ class _Group:
 
 class CacheManager:
     def __init__(self, layer_requests, page_size: int, num_pages: int, max_requests: int):
-        """``layer_requests[i]`` is the cache request of layer ``i`` (see ``parts.base``)."""
+        """``layer_requests[p]`` is the cache request of the p-th layer run of a step (see
+        ``parts.base`` and ``DecoderModel.cache_requests``); "layer" below means such a run."""
         from ..parts.base import PagedKVRequest, SharedKVRequest, StateRequest
         if page_size < 16 or page_size % 16:
             raise CacheError(f"page size {page_size} must be a positive multiple of 16")

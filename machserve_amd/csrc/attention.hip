@@ -248,10 +248,20 @@ struct DecodeArgs {
     const int* seq_pos0;     // [S] position of the row = number of keys before it
     int table_stride, H, KV, hd, ps, window, nsplit;
     float scale;
+    // fused form: q, k, v of the step come as partial sums of the projection; the kernel adds
+    // them and the bias, rotates q and k, writes k and v into their page and merges the splits
+    const float* qkv;        // [n_partials, S, stride]: q heads, k heads, v heads
+    const float* bias;       // [stride] or null
+    const float* inv_freq;   // [hd / 2] or null: no rotation
+    const int* slot_map;     // [S] page * ps + offset of the row's key
+    int n_partials, stride;
 };
 
+constexpr int MAX_SPLITS = 64;
+
+template <bool FUSED>
 __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
-    __shared__ float sm_o[3][HDT][16];
+    __shared__ float sm_o[3][HDT][16];  // also the staging area of the fused prologue: (g + 2) * hd floats
     __shared__ float sm_m[3][16], sm_l[3][16];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, grp = lane >> 4;
@@ -268,7 +278,59 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
     const int t0 = t_lo + sp * tps, t1 = min(t_hi, t0 + tps);
 
     Frag qf[NKS];
-    {
+    if constexpr (FUSED) {
+        __shared__ float cs[HDT / 2], sn[HDT / 2];
+        const int half = hd / 2;
+        const size_t pstride = (size_t)gridDim.x * a.stride;
+        const float* row0 = a.qkv + (size_t)s * a.stride;
+        // stage this KV head's share of the row: its g query heads, its key, its value
+        float* rowv = &sm_o[0][0][0];
+        const int qcol = kvh * g * hd, kcol = a.H * hd + kvh * hd, vcol = (a.H + a.KV) * hd + kvh * hd;
+        for (int c = tid; c < (g + 2) * hd; c += 256) {
+            const int col = c < g * hd ? qcol + c : (c < (g + 1) * hd ? kcol + c - g * hd : vcol + c - (g + 1) * hd);
+            float v = a.bias ? a.bias[col] : 0.f;
+            for (int p = 0; p < a.n_partials; ++p) v += row0[p * pstride + col];
+            rowv[c] = v;
+        }
+        if (tid < half) {
+            float c = 1.f, sv = 0.f;
+            if (a.inv_freq) sincosf((float)pos * a.inv_freq[tid], &sv, &c);
+            cs[tid] = c;
+            sn[tid] = sv;
+        }
+        __syncthreads();
+        // the block whose keys include this row's own position writes the row's k and v
+        const int sp_own = (pos / BKV - t_lo) / tps;
+        if (sp == sp_own) {
+            const int slot = a.slot_map[s];
+            const int page = slot / ps, off = slot % ps;
+            const float* kv_ = rowv + g * hd;
+            const float* vv_ = rowv + (g + 1) * hd;
+            for (int d = tid; d < hd; d += 256) {
+                const int j = d < half ? d : d - half;
+                const float x0 = kv_[j], x1 = kv_[j + half];
+                const float kv = d < half ? x0 * cs[j] - x1 * sn[j] : x0 * sn[j] + x1 * cs[j];
+                const_cast<elem_t*>(a.kpool)[(((size_t)page * a.KV + kvh) * ps + off) * hd + d] = from_f32<elem_t>(kv);
+                const_cast<elem_t*>(a.vpool)[(((size_t)page * a.KV + kvh) * hd + d) * ps + off] = from_f32<elem_t>(vv_[d]);
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            const int d0 = ks * 32 + grp * 8;
+            if (valid && d0 < hd) {
+                const float* qh = rowv + r16 * hd;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int d = d0 + e, j = d < half ? d : d - half;
+                    const float x0 = qh[j], x1 = qh[j + half];
+                    qf[ks].v[e] = from_f32<elem_t>(d < half ? x0 * cs[j] - x1 * sn[j] : x0 * sn[j] + x1 * cs[j]);
+                }
+            } else {
+                qf[ks] = frag_zero();
+            }
+        }
+        __syncthreads();  // the row's own key and value are in the page before any wave reads it
+    } else {
         const elem_t* qrow = a.q + ((size_t)s * a.H + head) * hd;
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
@@ -276,6 +338,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
             qf[ks] = (valid && d0 < hd) ? frag_load(qrow + d0) : frag_zero();
         }
     }
+
     f32x4 acc_o[ND];
 #pragma unroll
     for (int i = 0; i < ND; ++i) acc_o[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -375,49 +438,49 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
             for (int i = 0; i < 4; ++i) sm_o[wave - 1][dt * 16 + grp * 4 + i][r16] = acc_o[dt][i];
     }
     __syncthreads();
-    if (wave > 0) return;
-    float m_all = m_run;
+    if (wave == 0) {
+        float m_all = m_run;
 #pragma unroll
-    for (int w = 0; w < 3; ++w) m_all = fmaxf(m_all, sm_m[w][r16]);
-    const float c0 = exp_f(m_run - m_all);
-    float l_all = l_run * c0;
-#pragma unroll
-    for (int dt = 0; dt < ND; ++dt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc_o[dt][i] *= c0;
-#pragma unroll
-    for (int w = 0; w < 3; ++w) {
-        const float c = exp_f(sm_m[w][r16] - m_all);
-        l_all += sm_l[w][r16] * c;
+        for (int w = 0; w < 3; ++w) m_all = fmaxf(m_all, sm_m[w][r16]);
+        const float c0 = exp_f(m_run - m_all);
+        float l_all = l_run * c0;
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc_o[dt][i] += sm_o[w][dt * 16 + grp * 4 + i][r16] * c;
-    }
-    if (!valid) return;
-    if (a.nsplit == 1) {
-        const float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
-        elem_t* orow = a.out + ((size_t)s * a.H + head) * hd;
+            for (int i = 0; i < 4; ++i) acc_o[dt][i] *= c0;
 #pragma unroll
-        for (int dt = 0; dt < ND; ++dt) {
-            const int d0 = dt * 16 + grp * 4;
-            if (d0 < hd) {
+        for (int w = 0; w < 3; ++w) {
+            const float c = exp_f(sm_m[w][r16] - m_all);
+            l_all += sm_l[w][r16] * c;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) orow[d0 + i] = from_f32<elem_t>(acc_o[dt][i] * inv);
-            }
+            for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc_o[dt][i] += sm_o[w][dt * 16 + grp * 4 + i][r16] * c;
         }
-    } else {
-        const size_t base = ((size_t)s * a.H + head) * a.nsplit + sp;
-        float* po = a.part_o + base * hd;
+        if (valid && a.nsplit == 1) {
+            const float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
+            elem_t* orow = a.out + ((size_t)s * a.H + head) * hd;
 #pragma unroll
-        for (int dt = 0; dt < ND; ++dt) {
-            const int d0 = dt * 16 + grp * 4;
-            if (d0 < hd) {
+            for (int dt = 0; dt < ND; ++dt) {
+                const int d0 = dt * 16 + grp * 4;
+                if (d0 < hd) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) po[d0 + i] = acc_o[dt][i];
+                    for (int i = 0; i < 4; ++i) orow[d0 + i] = from_f32<elem_t>(acc_o[dt][i] * inv);
+                }
             }
+        } else if (valid) {
+            const size_t base = ((size_t)s * a.H + head) * a.nsplit + sp;
+            float* po = a.part_o + base * hd;
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt) {
+                const int d0 = dt * 16 + grp * 4;
+                if (d0 < hd) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) po[d0 + i] = acc_o[dt][i];
+                }
+            }
+            if (grp == 0) { a.part_ml[base * 2] = m_all; a.part_ml[base * 2 + 1] = l_all; }
         }
-        if (grp == 0) { a.part_ml[base * 2] = m_all; a.part_ml[base * 2 + 1] = l_all; }
     }
 }
 
@@ -477,9 +540,35 @@ extern "C" int MS_CAT(ms_decode_attention_nd, MS_ATTN_ND)(
     MS_REQUIRE(ps % 16 == 0 && ps > 0, "decode attention: page size %d must be a multiple of 16", ps);
     MS_REQUIRE(nsplit >= 1 && nsplit <= 65535 && (nsplit == 1 || (part_o && part_ml)), "decode attention: %d splits", nsplit);
     DecodeArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, (elem_t*)out, part_o, part_ml, block_table,
-                 seq_pos0, table_stride, H, KV, hd, ps, window, nsplit, scale};
-    hipLaunchKernelGGL(decode_attention_kernel, dim3((unsigned)S, (unsigned)KV, (unsigned)nsplit), dim3(256), 0, stream, a);
+                 seq_pos0, table_stride, H, KV, hd, ps, window, nsplit, scale, nullptr, nullptr, nullptr, nullptr, 0, 0};
+    hipLaunchKernelGGL(decode_attention_kernel<false>, dim3((unsigned)S, (unsigned)KV, (unsigned)nsplit), dim3(256), 0, stream, a);
     int rc = check_launch("decode_attention");
+    if (rc || nsplit == 1) return rc;
+    hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)(S * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit);
+    return check_launch("decode_merge");
+}
+
+// The same from the partial sums of the q/k/v projection: adds them and the bias, rotates q and k
+// by the row's position, writes k and v into the row's page, and attends; a second launch merges
+// the splits.  (Merging in the block that finishes last needs a device-wide fence in every block,
+// which on this chip writes back a whole L2 and costs more than the launch it saves.)
+// qkv is float [n_partials, S, stride] with the q heads, then the k heads, then the v heads.
+extern "C" int MS_CAT(ms_decode_attention_fused_nd, MS_ATTN_ND)(
+    const float* qkv, int n_partials, int stride, const float* bias, const float* inv_freq, const int* slot_map,
+    void* kpool, void* vpool, void* out, float* part_o, float* part_ml, const int* block_table,
+    int table_stride, const int* seq_pos0, int S, int H, int KV, int hd, int ps, int window, int nsplit, float scale,
+    hipStream_t stream) {
+    MS_REQUIRE(S > 0 && n_partials >= 1, "decode attention: no rows");
+    MS_REQUIRE(hd % 16 == 0 && hd > 0 && hd <= HDT, "decode attention: head size %d does not fit this tile of %d", hd, HDT);
+    MS_REQUIRE(KV > 0 && H % KV == 0 && H / KV <= 16, "decode attention: %d heads over %d key/value heads (at most 16 each)", H, KV);
+    MS_REQUIRE(ps % 16 == 0 && ps > 0, "decode attention: page size %d must be a multiple of 16", ps);
+    MS_REQUIRE(stride >= (H + 2 * KV) * hd, "decode attention: row stride %d too small", stride);
+    MS_REQUIRE(nsplit >= 1 && nsplit <= MAX_SPLITS && (nsplit == 1 || (part_o && part_ml)), "decode attention: %d splits (at most %d)", nsplit, MAX_SPLITS);
+    MS_REQUIRE(slot_map && kpool && vpool, "decode attention: the fused form writes the cache");
+    DecodeArgs a{nullptr, (const elem_t*)kpool, (const elem_t*)vpool, (elem_t*)out, part_o, part_ml, block_table, seq_pos0,
+                 table_stride, H, KV, hd, ps, window, nsplit, scale, qkv, bias, inv_freq, slot_map, n_partials, stride};
+    hipLaunchKernelGGL(decode_attention_kernel<true>, dim3((unsigned)S, (unsigned)KV, (unsigned)nsplit), dim3(256), 0, stream, a);
+    int rc = check_launch("decode_attention_fused");
     if (rc || nsplit == 1) return rc;
     hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)(S * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit);
     return check_launch("decode_merge");

@@ -16,7 +16,7 @@
 
 namespace ms {
 
-constexpr int ST = 256;
+constexpr int ST = 1024;
 
 __device__ __forceinline__ unsigned long long mix64(unsigned long long z) {
     z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
@@ -69,22 +69,29 @@ __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs a) {
     const int i0 = min(V, tid * seg_len), i1 = min(V, i0 + seg_len);
 
     if (T <= 0.0f) {
-        // smallest index among the maxima: segments are in index order, strict > inside
+        // smallest index among the maxima.  A thread walks its strided indices in ascending
+        // order and keeps the first maximum; ties between threads go to the smaller index.
         float best = -INFINITY;
         int bi = 0x7fffffff;
-        for (int i = i0; i < i1; ++i)
-            if (bi == 0x7fffffff || row[i] > best) { best = row[i]; bi = i; }
-        // wave reduce (value desc, index asc)
+        for (int i = tid; i < V; i += ST) {
+            const float x = row[i];
+            if (bi == 0x7fffffff || x > best) { best = x; bi = i; }
+        }
         for (int o = 32; o > 0; o >>= 1) {
             const float ov = __shfl_xor(best, o, WAVE);
             const int oi = __shfl_xor(bi, o, WAVE);
-            if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+            if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > best || (ov == best && oi < bi))) { best = ov; bi = oi; }
         }
         if ((tid & 63) == 0) { s_val[tid >> 6] = best; s_idx[tid >> 6] = bi; }
         __syncthreads();
         if (tid == 0) {
-            for (int w = 1; w < ST / WAVE; ++w)
-                if (s_val[w] > best || (s_val[w] == best && s_idx[w] < bi)) { best = s_val[w]; bi = s_idx[w]; }
+            for (int w = 1; w < ST / WAVE; ++w) {
+                const int oi = s_idx[w];
+                if (oi != 0x7fffffff && (bi == 0x7fffffff || s_val[w] > best || (s_val[w] == best && oi < bi))) {
+                    best = s_val[w];
+                    bi = oi;
+                }
+            }
             a.out_token[r] = bi;
             a.out_logprob[r] = 0.0f;
         }

@@ -102,22 +102,24 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
                     for (int e = 0; e < 4; ++e) dst[((i * NT + j) * 4 + e) * 64 + lane] = acc[i][j][e];
         }
         __syncthreads();
-        if (wk > 0) return;
+        if (wk == 0) {
 #pragma unroll
-        for (int s = 1; s < KSI; ++s) {
-            const float* src = red + ((size_t)((s - 1) * WN + wn) * MT * NT * 4) * 64;
+            for (int s = 1; s < KSI; ++s) {
+                const float* src = red + ((size_t)((s - 1) * WN + wn) * MT * NT * 4) * 64;
 #pragma unroll
-            for (int i = 0; i < MT; ++i)
+                for (int i = 0; i < MT; ++i)
 #pragma unroll
-                for (int j = 0; j < NT; ++j)
+                    for (int j = 0; j < NT; ++j)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[i][j][e] += src[((i * NT + j) * 4 + e) * 64 + lane];
+                        for (int e = 0; e < 4; ++e) acc[i][j][e] += src[((i * NT + j) * 4 + e) * 64 + lane];
+            }
         }
     }
-    if (n0 >= a.N) return;
+    const bool owner = wk == 0 && n0 < a.N;  // this wave holds the finished sums of its columns
 
     if constexpr (EPI == SK_SWIGLU) {
         static_assert(NT % 2 == 0, "gate and up tiles come in pairs");
+        if (!owner) return;
         elem_t* out = reinterpret_cast<elem_t*>(a.out);
 #pragma unroll
         for (int i = 0; i < MT; ++i)
@@ -132,19 +134,21 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
                 }
             }
     } else {
-        float* out = reinterpret_cast<float*>(a.out) + (size_t)blockIdx.y * a.M * a.N;
+        if (owner) {
+            float* out = reinterpret_cast<float*>(a.out) + (size_t)blockIdx.y * a.M * a.N;
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
+            for (int i = 0; i < MT; ++i)
 #pragma unroll
-            for (int j = 0; j < NT; ++j) {
-                const int col = n0 + j * 16 + r16;
-                if (col >= a.N) continue;
+                for (int j = 0; j < NT; ++j) {
+                    const int col = n0 + j * 16 + r16;
+                    if (col >= a.N) continue;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int row = i * 16 + grp * 4 + e;
-                    if (row < a.M) out[(size_t)row * a.N + col] = acc[i][j][e];
+                    for (int e = 0; e < 4; ++e) {
+                        const int row = i * 16 + grp * 4 + e;
+                        if (row < a.M) out[(size_t)row * a.N + col] = acc[i][j][e];
+                    }
                 }
-            }
+        }
     }
 }
 

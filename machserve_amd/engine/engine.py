@@ -54,7 +54,7 @@ class Engine:
             entries.append(StepEntry(it.request.slot, toks, [it.count - 1] if it.sample else []))
             if it.sample:
                 sampled_items.append(it)
-        logits = self.loaded.step(entries)
+        logits = self.loaded.step(entries, borrow_logits=True)
         self.steps += 1
         self.tokens_run += plan.n_tokens
         if not sampled_items:

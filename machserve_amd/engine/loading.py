@@ -39,7 +39,7 @@ class LoadedModel:
 
 def load_model(model_dir: Optional[str] = None, *, dtype="bfloat16", device: str = "cuda:0", page_size: int = 64,
                num_pages: Optional[int] = None, max_tokens: Optional[int] = None, max_requests: int = 64,
-               config=None, tensors=None, ops=None) -> LoadedModel:
+               config=None, tensors=None, ops=None, use_graphs: bool = True) -> LoadedModel:
     """``model_dir`` holds config.json and model.safetensors; alternatively pass a typed
     ``config`` and a dict of ``tensors``.  The cache pool has ``num_pages`` pages per group,
     or enough for ``max_tokens`` tokens."""
@@ -60,5 +60,5 @@ def load_model(model_dir: Optional[str] = None, *, dtype="bfloat16", device: str
     device_cache = DeviceCache(cache, dt, rt.device)
     model.bind_cache(device_cache)
     rows_per_block = getattr(ops, "attention_rows_per_block_default", 64)
-    step = StepFunction(model, cache, rt, rows_per_block)
+    step = StepFunction(model, cache, rt, rows_per_block, use_graphs)
     return LoadedModel(config, model, cache, device_cache, step, rt)

@@ -33,11 +33,27 @@ class StepEntry:
     want: Sequence[int] = ()  # indices into ``tokens`` whose logits are wanted
 
 
+class _DecodeGraph:
+    """One captured decode step for a fixed number of requests and fixed block-table widths:
+    a static int32 buffer the host refills before every replay, and the logits it produces."""
+
+    def __init__(self, graph, dev, pinned, offsets, sizes, logits):
+        self.graph, self.dev, self.pinned, self.offsets, self.sizes, self.logits = graph, dev, pinned, offsets, sizes, logits
+        self.copied = torch.cuda.Event()  # the last upload of `pinned` has finished
+
+
 class StepFunction:
-    def __init__(self, model, cache: CacheManager, rt, attention_rows_per_block: int = 64):
+    TABLE_BUCKET = 8  # captured block tables are this many pages wide, or a multiple
+
+    def __init__(self, model, cache: CacheManager, rt, attention_rows_per_block: int = 64, use_graphs: bool = True):
         self.model, self.cache, self.rt = model, cache, rt
         self.rows_per_block = attention_rows_per_block
         self.heads_per_kv = model.attention_rows_per_token()
+        # a decode step is launch-bound; it is captured once per batch size into a HIP graph and
+        # replayed.  Only for models whose parts read nothing but device memory from the context.
+        self.use_graphs = (use_graphs and rt.device.type == "cuda"
+                           and all(getattr(b.mixer, "graph_safe", False) for b in getattr(model, "blocks", [])))
+        self._graphs: Dict[tuple, _DecodeGraph] = {}
 
     # ------------------------------------------------------------------ context
     def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
@@ -126,12 +142,97 @@ class StepFunction:
             ctx.attention_work[g] = sec(f"work/{g}").view(-1, 2)
         return ctx
 
+    # ------------------------------------------------------------------ captured decode steps
+    def _decode_sections(self, slots: List[int], tokens: List[int], widths: Dict[str, int]) -> Dict[str, np.ndarray]:
+        """The int32 sections of a step in which every request has one row, block tables padded
+        to ``widths``.  The order of the keys is the layout of the captured buffer."""
+        cache, ps = self.cache, self.cache.page_size
+        B = len(slots)
+        pos = np.fromiter((cache.lengths[s] for s in slots), dtype=np.int32, count=B)
+        ar = np.arange(B, dtype=np.int32)
+        sec: Dict[str, np.ndarray] = {
+            "tokens": np.asarray(tokens, dtype=np.int32), "positions": pos, "seq_q_start": ar,
+            "seq_q_len": np.ones(B, dtype=np.int32), "seq_pos0": pos, "seq_slot": np.asarray(slots, dtype=np.int32),
+            "want_rows": ar,
+        }
+        for name, width in widths.items():
+            table = np.full((B, width), -1, dtype=np.int32)
+            slot_map = np.empty(B, dtype=np.int32)
+            for i, s in enumerate(slots):
+                t = cache.table(name, s)
+                table[i, :len(t)] = t
+                slot_map[i] = t[pos[i] // ps] * ps + pos[i] % ps
+            sec[f"table/{name}"] = table.reshape(-1)
+            sec[f"slot_map/{name}"] = slot_map
+        for g in self.heads_per_kv:
+            sec[f"work/{g}"] = np.stack([ar, np.zeros(B, dtype=np.int32)], 1).reshape(-1)
+        return sec
+
+    def _context_from(self, dev: torch.Tensor, offsets, sizes, B: int, widths: Dict[str, int]) -> StepContext:
+        def sec(k):
+            return dev[offsets[k]:offsets[k] + sizes[k]]
+        ctx = StepContext(n_rows=B, n_seqs=B, tokens=sec("tokens"), positions=sec("positions"),
+                          seq_q_start=sec("seq_q_start"), seq_q_len=sec("seq_q_len"), seq_pos0=sec("seq_pos0"),
+                          seq_slot=sec("seq_slot"), want_rows=sec("want_rows"), decode_only=True)
+        for name, width in widths.items():
+            ctx.groups[name] = GroupView(self.cache.page_size, sec(f"slot_map/{name}"), sec(f"table/{name}").view(B, width))
+        for g in self.heads_per_kv:
+            ctx.attention_work[g] = sec(f"work/{g}").view(-1, 2)
+        return ctx
+
+    def _run_decode_graph(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        cache = self.cache
+        slots = [e.slot for e in entries]
+        tokens = [int(e.tokens[0]) for e in entries]
+        vocab = self.model.vocab
+        for s, t in zip(slots, tokens):
+            if not 0 <= t < vocab:
+                raise StepError(f"slot {s}: token {t} is outside the vocabulary of {vocab}")
+            if cache.lengths[s] + 1 > self.model.spec.max_positions:
+                raise StepError(f"slot {s}: position {cache.lengths[s]} is beyond the model's positions")
+        B = len(slots)
+        bucket = self.TABLE_BUCKET
+        widths = {name: -(-max(len(cache.table(name, s)) for s in slots) // bucket) * bucket for name in cache.groups}
+        key = (B, tuple(sorted(widths.items())))
+        sections = self._decode_sections(slots, tokens, widths)
+        dg = self._graphs.get(key)
+        if dg is None:
+            offsets, sizes, total = {}, {}, 0
+            for k, a in sections.items():
+                offsets[k], sizes[k] = total, a.size
+                total += (a.size + 3) // 4 * 4
+            pinned = torch.empty(total, dtype=torch.int32, pin_memory=True)
+            pinned.zero_()
+            dev = torch.zeros(total, dtype=torch.int32, device=self.rt.device)
+            dg = _DecodeGraph(None, dev, pinned, offsets, sizes, None)
+        dg.copied.synchronize()  # the host buffer is free to be refilled
+        host = dg.pinned.numpy()
+        for k, a in sections.items():
+            host[dg.offsets[k]:dg.offsets[k] + a.size] = a
+        dg.dev.copy_(dg.pinned, non_blocking=True)
+        dg.copied.record()
+        if dg.graph is None:
+            ctx = self._context_from(dg.dev, dg.offsets, dg.sizes, B, widths)
+            side = torch.cuda.Stream(device=self.rt.device)
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                self.model.forward(ctx)  # everything is loaded and compiled before the capture
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                dg.logits = self.model.forward(ctx)
+            dg.graph = graph
+            self._graphs[key] = dg
+        dg.graph.replay()
+        return dg.logits
+
     # ------------------------------------------------------------------ the step
-    def __call__(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def __call__(self, entries: Sequence[StepEntry], borrow_logits: bool = False) -> Optional[torch.Tensor]:
         """Float32 logits ``[number of wanted places, vocab]`` in the order of the entries and
         of their ``want`` lists (None if nothing is wanted).  Takes the pages the new tokens
         need (raises ``OutOfPages`` before anything ran if they are not there), runs the
-        model, and advances the requests' lengths."""
+        model, and advances the requests' lengths.  With ``borrow_logits`` the result may be a
+        buffer that the next step overwrites (the engine samples from it at once)."""
         cache = self.cache
         reserved: Dict[str, int] = {}
         for e in entries:
@@ -144,8 +245,17 @@ class StepFunction:
                 raise OutOfPages(f"group {k}: the step needs {v} new pages, {cache.free_pages(k)} are free")
         for e in entries:
             cache.extend(e.slot, len(e.tokens))
-        ctx = self.build_context(entries)
-        logits = self.model.forward(ctx)
+        if self.use_graphs and all(len(e.tokens) == 1 for e in entries) and len({e.slot for e in entries}) == len(entries):
+            logits = self._run_decode_graph(entries)
+            wanted = [i for i, e in enumerate(entries) if len(e.want)]
+            if not wanted:
+                logits = None
+            elif len(wanted) != len(entries):
+                logits = logits[torch.tensor(wanted, device=logits.device)]
+            elif not borrow_logits:
+                logits = logits.clone()  # the graph's own buffer is overwritten by its next replay
+        else:
+            logits = self.model.forward(self.build_context(entries))
         for e in entries:
             cache.commit(e.slot, len(e.tokens))
         return logits

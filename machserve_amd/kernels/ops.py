@@ -193,7 +193,8 @@ class HipOps:
             lib = self._load(build.ensure_library("attention", self.elem, nd))
             self._attn[nd] = (lib, getattr(lib, f"ms_paged_attention_nd{nd}"),
                               getattr(lib, f"ms_attention_rows_per_block_nd{nd}")(),
-                              getattr(lib, f"ms_decode_attention_nd{nd}"), getattr(lib, f"ms_attention_key_tile_nd{nd}")())
+                              getattr(lib, f"ms_decode_attention_nd{nd}"), getattr(lib, f"ms_attention_key_tile_nd{nd}")(),
+                              getattr(lib, f"ms_decode_attention_fused_nd{nd}"))
         return self._attn[nd]
 
     def attention_rows_per_block(self, hd: int) -> int:
@@ -227,13 +228,57 @@ class HipOps:
 
     DECODE_MAX_GROUP = 16  # query heads per key/value head the decode kernel takes
 
+    @staticmethod
+    def _decode_splits(S: int, KV: int, table_width: int, page_size: int, window: Optional[int], key_tile: int) -> int:
+        span = table_width * page_size if not window else min(table_width * page_size, window + key_tile)
+        tiles = max(1, -(-span // key_tile))
+        return max(1, min(-(-1024 // (S * KV)), -(-tiles // 4), 64))
+
+    def decode_attention_fused(self, qkv: torch.Tensor, bias: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor],
+                               slot_map: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
+                               block_table: torch.Tensor, seq_pos0: torch.Tensor, H: int, KV: int, hd: int,
+                               page_size: int, window: Optional[int], scale: float) -> torch.Tensor:
+        """Decode attention from the partial sums ``qkv [P, S, stride]`` of the q/k/v projection: bias,
+        rotation, cache write and attention over the pages in one launch, the merge of the
+        splits in a second."""
+        lib, key_tile, fn = self._attention_lib(hd)[0], self._attention_lib(hd)[4], self._attention_lib(hd)[5]
+        if qkv.dim() == 2:
+            qkv = qkv.unsqueeze(0)
+        P, S, stride = qkv.shape
+        self._want(qkv, torch.float32, "attention qkv")
+        if bias is not None:
+            self._want(bias, torch.float32, "attention bias", stride)
+        if inv_freq is not None:
+            self._want(inv_freq, torch.float32, "attention inv_freq", hd // 2)
+        self._want(slot_map, torch.int32, "attention slot_map", S)
+        pages = kpool.shape[0]
+        self._want(kpool, self.dtype, "key pool", pages, KV, page_size, hd)
+        self._want(vpool, self.dtype, "value pool", pages, KV, hd, page_size)
+        self._want(block_table, torch.int32, "block table")
+        if block_table.dim() != 2 or block_table.shape[0] != S:
+            raise KernelError(f"attention: block table {tuple(block_table.shape)} for {S} requests")
+        self._want(seq_pos0, torch.int32, "seq_pos0", S)
+        if H // KV > self.DECODE_MAX_GROUP:
+            raise KernelError(f"decode attention: {H // KV} heads per key/value head, at most {self.DECODE_MAX_GROUP}")
+        nsplit = self._decode_splits(S, KV, block_table.shape[1], page_size, window, key_tile)
+        out = torch.empty((S, H * hd), dtype=self.dtype, device=qkv.device)
+        part_o = part_ml = None
+        if nsplit > 1:
+            part_o = torch.empty((S, H, nsplit, hd), dtype=torch.float32, device=qkv.device)
+            part_ml = torch.empty((S, H, nsplit, 2), dtype=torch.float32, device=qkv.device)
+        self._check(lib, fn(_ptr(qkv), _c_int(P), _c_int(stride), _ptr(bias), _ptr(inv_freq), _ptr(slot_map), _ptr(kpool),
+                            _ptr(vpool), _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(block_table),
+                            _c_int(block_table.shape[1]), _ptr(seq_pos0), _c_int(S), _c_int(H), _c_int(KV), _c_int(hd),
+                            _c_int(page_size), _c_int(window or 0), _c_int(nsplit), _c_float(scale), _stream()))
+        return out
+
     def decode_attention(self, q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
                          seq_pos0: torch.Tensor, H: int, KV: int, hd: int, page_size: int, window: Optional[int],
                          scale: float) -> torch.Tensor:
         """Attention of a step in which request ``s`` has the single row ``s``.  The keys are cut
         into splits so that the grid fills the chip; how many follows from the number of
         requests and the width of the block table only."""
-        lib, _, _, fn, key_tile = self._attention_lib(hd)
+        lib, _, _, fn, key_tile = self._attention_lib(hd)[:5]
         S = q.shape[0]
         self._want(q, self.dtype, "attention q", S, H * hd)
         pages = kpool.shape[0]
@@ -245,9 +290,7 @@ class HipOps:
         self._want(seq_pos0, torch.int32, "seq_pos0", S)
         if H // KV > self.DECODE_MAX_GROUP:
             raise KernelError(f"decode attention: {H // KV} heads per key/value head, at most {self.DECODE_MAX_GROUP}")
-        span = block_table.shape[1] * page_size if not window else min(block_table.shape[1] * page_size, window + key_tile)
-        tiles = max(1, -(-span // key_tile))
-        nsplit = max(1, min(-(-1024 // (S * KV)), -(-tiles // 4)))
+        nsplit = self._decode_splits(S, KV, block_table.shape[1], page_size, window, key_tile)
         out = torch.empty((S, H * hd), dtype=self.dtype, device=q.device)
         part_o = part_ml = None
         if nsplit > 1:

@@ -16,6 +16,8 @@ from .registry import POSITION_ENCODINGS, register_mixer
 
 @register_mixer("attention")
 class Attention(Mixer):
+    graph_safe = True  # reads positions and addresses from device memory only
+
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
         s = spec
@@ -81,11 +83,18 @@ class Attention(Mixer):
             q = qkv[0, :, :self.nq].unflatten(1, (s.heads, s.head_dim))
             k = qkv[0, :, self.nq:self.nq + self.nkv].unflatten(1, (s.kv_heads, s.head_dim)) if self.writes_cache else None
             self.position.apply(q, k, ctx)
+        g = self.attention_rows_per_token()
+        decode = ctx.decode_only and g <= ops.DECODE_MAX_GROUP
+        if decode and self.writes_cache and (self.position is None or inv_freq is not None):
+            o = ops.decode_attention_fused(qkv, bias, inv_freq, view.slot_map, self.kpool, self.vpool, view.block_table,
+                                           ctx.seq_pos0, s.heads, s.kv_heads, s.head_dim, view.page_size, s.window,
+                                           self.scale)
+            stream.add_linear(o, self.w_o)
+            return
         q = ops.rope_kv_write(qkv, bias, ctx.positions, inv_freq, view.slot_map if self.writes_cache else None,
                               self.kpool if self.writes_cache else None, self.vpool if self.writes_cache else None,
                               s.heads, s.kv_heads, s.head_dim, view.page_size)
-        g = self.attention_rows_per_token()
-        if ctx.decode_only and g <= ops.DECODE_MAX_GROUP:
+        if decode:
             o = ops.decode_attention(q, self.kpool, self.vpool, view.block_table, ctx.seq_pos0, s.heads, s.kv_heads,
                                      s.head_dim, view.page_size, s.window, self.scale)
         else:

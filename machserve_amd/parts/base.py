@@ -89,26 +89,38 @@ class StepContext:
 
 
 class ResidualStream:
-    """The 32-bit residual stream ``x [T, width]`` and, possibly, sums that are still to be added
-    to it.  A product with few rows leaves its result as partial sums; the norm that reads
-    the stream next adds them in the same kernel, which saves a pass over the stream."""
+    """The 32-bit residual stream ``x [T, width]`` and what is still to be added to it.
+
+    ``add_linear`` does not launch its product at once but when the stream is next read.  With
+    few rows the product leaves partial sums (``pending``) that the reading norm adds in its
+    own kernel (``normed``), which saves a pass over the stream; with many rows the product
+    adds to the stream in its epilogue.
+    """
 
     def __init__(self, x: torch.Tensor, ops):
         self.x = x
         self.ops = ops
-        self.pending: Optional[torch.Tensor] = None  # float32 [P, T, width]
+        self.deferred = None                         # (a, w): x += a @ w.T, not yet launched
+        self.pending: Optional[torch.Tensor] = None  # float32 [P, T, width], not yet added
 
     def add_linear(self, a: torch.Tensor, w: torch.Tensor) -> None:
         """``x += a @ w.T``."""
         self.flush()
-        self.pending = self.ops.linear_residual(a, w, self.x)
+        self.deferred = (a, w)
 
     def add(self, y: torch.Tensor) -> None:
         """``x += y`` for a part that computes its output by other means."""
         self.flush()
         self.x += y.to(self.x.dtype)
 
+    def _launch_deferred(self) -> None:
+        if self.deferred is not None:
+            a, w = self.deferred
+            self.deferred = None
+            self.pending = self.ops.linear_residual(a, w, self.x)
+
     def flush(self) -> None:
+        self._launch_deferred()
         if self.pending is not None:
             self.ops.add_partials(self.x, self.pending)
             self.pending = None
@@ -116,6 +128,15 @@ class ResidualStream:
     def value(self) -> torch.Tensor:
         self.flush()
         return self.x
+
+    def normed(self, weight: torch.Tensor, eps: float, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``rmsnorm(x) * weight`` of the stream with everything added (of its ``rows`` if given),
+        in the element type."""
+        self._launch_deferred()
+        h = self.ops.rmsnorm(self.x, weight, eps, rows, False, self.pending)
+        if rows is None:
+            self.pending = None  # the kernel wrote the sum back
+        return h
 
 
 class Part:

@@ -65,6 +65,7 @@ class DecoderModel:
         self.order = list(spec.order)
         self.final_norm = NORMS.build(spec.final_norm, rt)
         self.head = Head(spec.head, rt, self.embedding)
+        self._bindings, self._rebind = [], False
 
     # ------------------------------------------------------------------ structure
     def parts(self) -> List[Part]:
@@ -77,13 +78,28 @@ class DecoderModel:
         return out
 
     def cache_requests(self):
-        return [b.mixer.cache_request() for b in self.blocks]
+        """One cache request per *position of the order*: a layer that runs twice shares its
+        weights between the two runs, but each run keeps a cache (or state) of its own, so
+        what a run reads never depends on how the tokens were cut into steps.  A layer that
+        reads another layer's cache reads that of the layer's latest earlier run."""
+        from .base import SharedKVRequest
+        out = []
+        for p, i in enumerate(self.order):
+            req = self.blocks[i].mixer.cache_request()
+            if isinstance(req, SharedKVRequest):
+                earlier = [q for q in range(p) if self.order[q] == req.source_layer]
+                if not earlier:
+                    raise ValueError(f"layer {i} reads the cache of layer {req.source_layer}, which has not run before it")
+                req = SharedKVRequest(earlier[-1])
+            out.append(req)
+        return out
 
     def bind_cache(self, device_cache) -> None:
-        for i, b in enumerate(self.blocks):
-            binding = device_cache.binding(i)
-            if binding is not None:
-                b.mixer.bind_cache(binding)
+        self._bindings = [device_cache.binding(p) for p in range(len(self.order))]
+        for p, i in enumerate(self.order):  # a layer that runs once keeps its binding for good
+            if self._bindings[p] is not None:
+                self.blocks[i].mixer.bind_cache(self._bindings[p])
+        self._rebind = len(set(self.order)) != len(self.order)
 
     def attention_rows_per_token(self) -> List[int]:
         return sorted({g for g in (b.mixer.attention_rows_per_token() for b in self.blocks) if g})
@@ -97,7 +113,9 @@ class DecoderModel:
         """Run the step's rows through the layers in ``order``; float32 logits ``[W, vocab]`` of
         the wanted rows, or None when none is wanted."""
         stream = ResidualStream(self.embedding.forward(ctx.tokens), self.rt.ops)
-        for i in self.order:
+        for p, i in enumerate(self.order):
+            if self._rebind and self._bindings[p] is not None:
+                self.blocks[i].mixer.bind_cache(self._bindings[p])
             self.blocks[i].forward(stream, ctx)
         if ctx.want_rows.numel() == 0:
             return None

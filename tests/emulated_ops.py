@@ -124,6 +124,11 @@ class EmulatedOps:
         assert len(done) == T * H, "the work list does not cover every row and head"
         return self._r(out)
 
+    def decode_attention_fused(self, qkv, bias, inv_freq, slot_map, kpool, vpool, block_table, seq_pos0, H, KV, hd,
+                               page_size, window, scale):
+        q = self.rope_kv_write(qkv, bias, seq_pos0, inv_freq, slot_map, kpool, vpool, H, KV, hd, page_size)
+        return self.decode_attention(q, kpool, vpool, block_table, seq_pos0, H, KV, hd, page_size, window, scale)
+
     def decode_attention(self, q, kpool, vpool, block_table, seq_pos0, H, KV, hd, page_size, window, scale):
         S = q.shape[0]
         ar = torch.arange(S, dtype=torch.int32)

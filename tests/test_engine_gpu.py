@@ -189,12 +189,12 @@ def test_feed_forward_part_alone(dtype):
     t = {k: v.to(dtype) for k, v in t.items()}
     part.load({k: v.to(DEV) for k, v in t.items()})
     from machserve_amd.parts import ResidualStream
-    for rows in (11, 100):  # few rows: pending partial sums; many: added in the product's epilogue
+    for rows in (11, 100):  # few rows: partial sums for the next reader; many: added in the product's epilogue
         h = torch.randn(rows, 72).to(dtype)
         x = torch.randn(rows, 72)
         stream = ResidualStream(x.to(DEV).clone(), part.rt.ops)
         part.forward(h.to(DEV), stream, None)
-        assert (stream.pending is not None) == (rows <= 64)
+        assert stream.deferred is not None, "the product waits for the stream's next reader"
         ref = x + P.swiglu(h.float(), t["gate.weight"].float(), t["up.weight"].float(), t["down.weight"].float())
         assert_close(stream.value(), ref, dtype)
 

@@ -255,6 +255,42 @@ def test_decode_attention(dtype, H, KV, hd, ps, window):
     assert_close(one, ref[S - 1:], dtype, "decode attention of one request")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,KV,hd,ps,window,P_", [(4, 2, 16, 16, None, 1), (6, 1, 32, 32, None, 3), (5, 5, 48, 16, 40, 1),
+                                                  (14, 2, 64, 64, None, 2), (12, 2, 128, 64, None, 1), (16, 1, 80, 32, 100, 1)])
+def test_decode_attention_fused(dtype, H, KV, hd, ps, window, P_):
+    """Bias, rotation, cache write and attention from partial sums of the projection; twice in a
+    row with the same pages, the second time one position on, as decoding does."""
+    ops, emu = ops_for(dtype), EmulatedOps(dtype)
+    lens = [0, 1, ps - 1, ps, 130, 700, 2049, 63, 64]
+    S = len(lens)
+    gen = torch.Generator().manual_seed(600 + hd)
+    n_pages = sum(-(-(c + 2) // ps) for c in lens) + 2
+    order = torch.randperm(n_pages, generator=gen).tolist()
+    kp, vp = rnd((n_pages, KV, ps, hd), dtype, 601), rnd((n_pages, KV, hd, ps), dtype, 602)
+    width = max(-(-(c + 2) // ps) for c in lens)
+    table = torch.full((S, width), -1, dtype=torch.int32)
+    for i, c in enumerate(lens):
+        for p in range(-(-(c + 2) // ps)):
+            table[i, p] = order.pop()
+    stride = (H + 2 * KV) * hd
+    bias = rnd((stride,), torch.float32, 603)
+    j = torch.arange(hd // 2, dtype=torch.float32)
+    inv = 1.0 / torch.pow(torch.tensor(1e4), 2.0 * j / hd)
+    kd, vd = kp.to(DEV), vp.to(DEV)
+    for step in range(2):
+        pos0 = torch.tensor([c + step for c in lens], dtype=torch.int32)
+        slot_map = torch.tensor([int(table[i, (c + step) // ps]) * ps + (c + step) % ps for i, c in enumerate(lens)], dtype=torch.int32)
+        qkv = rnd((S, stride), torch.float32, 604 + step)
+        parts = torch.stack([qkv / P_ + (k - (P_ - 1) / 2) for k in range(P_)])  # P_ parts that sum to qkv
+        ref = emu.decode_attention_fused(parts, bias, inv, slot_map, kp, vp, table, pos0, H, KV, hd, ps, window, hd ** -0.5)
+        got = ops.decode_attention_fused(parts.to(DEV), bias.to(DEV), inv.to(DEV), slot_map.to(DEV), kd, vd, table.to(DEV),
+                                         pos0.to(DEV), H, KV, hd, ps, window, hd ** -0.5)
+        assert_close(got, ref, dtype, f"fused decode attention, step {step}")
+        assert_close(kd, kp, dtype, "key pages")
+        assert_close(vd, vp, dtype, "value pages")
+
+
 def test_attention_equals_library_attention_without_rotation_or_paging():
     """One request, whole prompt, pages in order: the kernel is plain causal attention."""
     dtype = torch.float32
