@@ -57,6 +57,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (named in config)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiles)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -122,6 +123,11 @@ def main() -> int:
         return min(times[1:])
 
     nums = model_numbers(cfg, dt.itemsize)
+    if args.prefill_only:
+        t = prefill_run()
+        print(json.dumps({"prefill": {"value": round(ctx / t, 1), "tokens": ctx, "ms": round(t * 1e3, 3),
+                                      "frac": round(prefill_flops(cfg, ctx) / t / PEAK_FLOPS[args.dtype], 4)}}))
+        return 0
     tok_s, ms = decode_run(args.batch)
     step_bytes = nums["weight_bytes"] + args.batch * (ctx + args.warmup + args.steps / 2) * nums["kv_bytes_per_token"]
     achieved = step_bytes / (ms * 1e-3) / 1e9

@@ -111,33 +111,56 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
     for (int i = 0; i < ND; ++i) acc_o[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m_run = NEG_BIG, l_run = 0.f;
 
-    for (int kt0 = (kv_lo / BKV) * BKV; kt0 < kv_hi; kt0 += BKV) {
-        __syncthreads();  // the previous tile has been consumed
-        // K tile: [BKV keys][HDT]
-        constexpr int CPRK = HDT / EPC;
-        for (int c = tid; c < BKV * CPRK; c += 256) {
+    // Tiles go global -> registers -> LDS; the registers for the next tile are requested before
+    // the current tile is multiplied, so the memory latency hides behind the MFMAs.
+    constexpr int CPRK = HDT / EPC, CPRV = BKV / EPC;
+    constexpr int NCK = (BKV * CPRK + 255) / 256, NCV = (HDT * CPRV + 255) / 256;
+    u32x4 rk[NCK], rv[NCV];
+    auto load_tile = [&](int kt0) {
+#pragma unroll
+        for (int i = 0; i < NCK; ++i) {
+            const int c = tid + i * 256;
             const int kl = c / CPRK, d0 = (c % CPRK) * EPC, key = kt0 + kl;
             u32x4 v = {0, 0, 0, 0};
-            if (key < kv_hi && d0 < hd) {
+            if (c < BKV * CPRK && key < kv_hi && d0 < hd) {
                 const int page = table[key / ps];
                 if (page >= 0)
                     v = *reinterpret_cast<const u32x4*>(a.kpool + (((size_t)page * a.KV + kvh) * ps + key % ps) * hd + d0);
             }
-            *reinterpret_cast<u32x4*>(&Ks[kl * K_LD + d0]) = v;
+            rk[i] = v;
         }
-        // V^T tile: [HDT][BKV keys]
-        constexpr int CPRV = BKV / EPC;
-        for (int c = tid; c < HDT * CPRV; c += 256) {
+#pragma unroll
+        for (int i = 0; i < NCV; ++i) {
+            const int c = tid + i * 256;
             const int d = c / CPRV, k0 = (c % CPRV) * EPC, key = kt0 + k0;
             u32x4 v = {0, 0, 0, 0};
-            if (key < kv_hi && d < hd) {
+            if (c < HDT * CPRV && key < kv_hi && d < hd) {
                 const int page = table[key / ps];
                 if (page >= 0)
                     v = *reinterpret_cast<const u32x4*>(a.vpool + (((size_t)page * a.KV + kvh) * hd + d) * ps + key % ps);
             }
-            *reinterpret_cast<u32x4*>(&Vs[d * V_LD + k0]) = v;
+            rv[i] = v;
         }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < NCK; ++i) {
+            const int c = tid + i * 256;
+            if (c < BKV * CPRK) *reinterpret_cast<u32x4*>(&Ks[(c / CPRK) * K_LD + (c % CPRK) * EPC]) = rk[i];
+        }
+#pragma unroll
+        for (int i = 0; i < NCV; ++i) {
+            const int c = tid + i * 256;
+            if (c < HDT * CPRV) *reinterpret_cast<u32x4*>(&Vs[(c / CPRV) * V_LD + (c % CPRV) * EPC]) = rv[i];
+        }
+    };
+    const int kt_first = (kv_lo / BKV) * BKV;
+    if (kt_first < kv_hi) load_tile(kt_first);
+    for (int kt0 = kt_first; kt0 < kv_hi; kt0 += BKV) {
+        __syncthreads();  // the previous tile has been consumed
+        store_tile();
         __syncthreads();
+        if (kt0 + BKV < kv_hi) load_tile(kt0 + BKV);
         if (!wave_active) continue;
 
         // S^T = K Q^T: lane holds keys grp * 4 + i of tile nt for query row r16
@@ -259,27 +282,78 @@ struct DecodeArgs {
 
 constexpr int MAX_SPLITS = 64;
 
+// Fragments of one key tile for one lane: keys (K rows) for the scores, V^T groups for the output.
+struct DecodeTile {
+    Frag kf[NT][NKS];
+    Frag vf[NTP][ND];
+};
+
 template <bool FUSED>
 __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
     __shared__ float sm_o[3][HDT][16];  // also the staging area of the fused prologue: (g + 2) * hd floats
     __shared__ float sm_m[3][16], sm_l[3][16];
+    __shared__ float cs[HDT / 2], sn[HDT / 2], knew[HDT], vnew[HDT];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r16 = lane & 15, grp = lane >> 4;
     const int s = blockIdx.x, kvh = blockIdx.y, sp = blockIdx.z;
     const int g = a.H / a.KV, hd = a.hd, ps = a.ps;
-    const int pos = a.seq_pos0[s], kv_len = pos + 1;
+    const int pos = a.seq_pos0[s];
+    // keys read from the pages: all of them, or (fused) those before the row's own position,
+    // whose key and value are still in registers and enter as one extra term
+    const int kv_len = FUSED ? pos : pos + 1;
     const int lo_key = a.window > 0 ? max(0, pos - a.window + 1) : 0;
     const int* table = a.block_table + (size_t)s * a.table_stride;
     const bool valid = r16 < g;
     const int head = kvh * g + (valid ? r16 : 0);
 
     const int t_lo = lo_key / BKV, t_hi = ceil_div(kv_len, BKV);
-    const int tps = ceil_div(t_hi - t_lo, a.nsplit);
+    const int tps = max(1, ceil_div(t_hi - t_lo, a.nsplit));
     const int t0 = t_lo + sp * tps, t1 = min(t_hi, t0 + tps);
+
+    // Loads of a tile depend on nothing the prologue computes: the first tile is requested
+    // before the prologue so that its latency hides behind it.
+    auto load_tile = [&](int t, DecodeTile& td) {
+        const int kt0 = t * BKV;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int key = kt0 + nt * 16 + r16;
+            const int page = key < kv_len ? table[key / ps] : -1;
+            const elem_t* krow = a.kpool + (((size_t)max(page, 0) * a.KV + kvh) * ps + key % ps) * hd;
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+                const int d0 = ks * 32 + grp * 8;
+                td.kf[nt][ks] = (page >= 0 && d0 < hd) ? frag_load(krow + d0) : frag_zero();
+            }
+        }
+#pragma unroll
+        for (int pp = 0; pp < NTP; ++pp) {
+            // the two 4-key groups this lane multiplies: same 16-key tile -> same page
+            const int ka = kt0 + (2 * pp) * 16 + grp * 4, kb = ka + 16;
+            const int pa = ka < kv_len ? table[ka / ps] : -1;
+            const int pb = (2 * pp + 1 < NT && kb < kv_len) ? table[kb / ps] : -1;
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt) {
+                const int d = dt * 16 + r16;
+                Frag vf = frag_zero();
+                if (pa >= 0 && d < hd) {
+                    const elem_t* v0 = a.vpool + (((size_t)pa * a.KV + kvh) * hd + d) * ps + ka % ps;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) vf.v[i] = v0[i];
+                }
+                if (pb >= 0 && d < hd) {
+                    const elem_t* v1 = a.vpool + (((size_t)pb * a.KV + kvh) * hd + d) * ps + kb % ps;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) vf.v[4 + i] = v1[i];
+                }
+                td.vf[pp][dt] = vf;
+            }
+        }
+    };
+    DecodeTile next;
+    if (t0 + wave < t1) load_tile(t0 + wave, next);
 
     Frag qf[NKS];
     if constexpr (FUSED) {
-        __shared__ float cs[HDT / 2], sn[HDT / 2];
         const int half = hd / 2;
         const size_t pstride = (size_t)gridDim.x * a.stride;
         const float* row0 = a.qkv + (size_t)s * a.stride;
@@ -299,19 +373,23 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
             sn[tid] = sv;
         }
         __syncthreads();
-        // the block whose keys include this row's own position writes the row's k and v
-        const int sp_own = (pos / BKV - t_lo) / tps;
-        if (sp == sp_own) {
-            const int slot = a.slot_map[s];
-            const int page = slot / ps, off = slot % ps;
+        // the row's own key (rotated) and value, rounded as the page holds them
+        {
             const float* kv_ = rowv + g * hd;
             const float* vv_ = rowv + (g + 1) * hd;
+            const int slot = a.slot_map[s];
+            const int page = slot / ps, off = slot % ps;
             for (int d = tid; d < hd; d += 256) {
                 const int j = d < half ? d : d - half;
                 const float x0 = kv_[j], x1 = kv_[j + half];
-                const float kv = d < half ? x0 * cs[j] - x1 * sn[j] : x0 * sn[j] + x1 * cs[j];
-                const_cast<elem_t*>(a.kpool)[(((size_t)page * a.KV + kvh) * ps + off) * hd + d] = from_f32<elem_t>(kv);
-                const_cast<elem_t*>(a.vpool)[(((size_t)page * a.KV + kvh) * hd + d) * ps + off] = from_f32<elem_t>(vv_[d]);
+                const elem_t ke = from_f32<elem_t>(d < half ? x0 * cs[j] - x1 * sn[j] : x0 * sn[j] + x1 * cs[j]);
+                const elem_t ve = from_f32<elem_t>(vv_[d]);
+                knew[d] = to_f32(ke);
+                vnew[d] = to_f32(ve);
+                if (sp == 0 && slot >= 0) {  // one block writes the page; nobody reads it in this launch
+                    const_cast<elem_t*>(a.kpool)[(((size_t)page * a.KV + kvh) * ps + off) * hd + d] = ke;
+                    const_cast<elem_t*>(a.vpool)[(((size_t)page * a.KV + kvh) * hd + d) * ps + off] = ve;
+                }
             }
         }
 #pragma unroll
@@ -329,7 +407,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
                 qf[ks] = frag_zero();
             }
         }
-        __syncthreads();  // the row's own key and value are in the page before any wave reads it
+        __syncthreads();  // knew / vnew are complete, and the staging area is free again
     } else {
         const elem_t* qrow = a.q + ((size_t)s * a.H + head) * hd;
 #pragma unroll
@@ -346,19 +424,14 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
 
     for (int t = t0 + wave; t < t1; t += 4) {
         const int kt0 = t * BKV;
+        DecodeTile cur = next;
+        if (t + 4 < t1) load_tile(t + 4, next);
         f32x4 sc[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             sc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-            const int key = kt0 + nt * 16 + r16;
-            const int page = key < kv_len ? table[key / ps] : -1;
-            const elem_t* krow = a.kpool + (((size_t)max(page, 0) * a.KV + kvh) * ps + key % ps) * hd;
 #pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) {
-                const int d0 = ks * 32 + grp * 8;
-                Frag kf = (page >= 0 && d0 < hd) ? frag_load(krow + d0) : frag_zero();
-                mma_16x16x32(sc[nt], kf, qf[ks]);
-            }
+            for (int ks = 0; ks < NKS; ++ks) mma_16x16x32(sc[nt], cur.kf[nt][ks], qf[ks]);
         }
         float tmax = NEG_BIG;
 #pragma unroll
@@ -366,7 +439,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int key = kt0 + nt * 16 + grp * 4 + i;
-                const bool ok = valid && key <= pos && key >= lo_key;
+                const bool ok = valid && key < kv_len && key >= lo_key;
                 const float v = ok ? sc[nt][i] * a.scale : -INFINITY;
                 sc[nt][i] = v;
                 tmax = fmaxf(tmax, v);
@@ -400,32 +473,37 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
                 pf.v[i] = from_f32<elem_t>(sc[2 * pp][i]);
                 pf.v[4 + i] = from_f32<elem_t>((2 * pp + 1 < NT) ? sc[(2 * pp + 1) % NT][i] : 0.f);
             }
-            // the two 4-key groups this lane multiplies: same 16-key tile -> same page
-            const int ka = kt0 + (2 * pp) * 16 + grp * 4, kb = ka + 16;
-            const int pa = ka < kv_len ? table[ka / ps] : -1;
-            const int pb = (2 * pp + 1 < NT && kb < kv_len) ? table[kb / ps] : -1;
 #pragma unroll
-            for (int dt = 0; dt < ND; ++dt) {
-                const int d = dt * 16 + r16;
-                Frag vf;
-                if (pa >= 0 && d < hd) {
-                    const elem_t* v0 = a.vpool + (((size_t)pa * a.KV + kvh) * hd + d) * ps + ka % ps;
+            for (int dt = 0; dt < ND; ++dt) mma_16x16x32(acc_o[dt], cur.vf[pp][dt], pf);
+        }
+    }
+
+    if constexpr (FUSED) {
+        // the row's own key: one more term of the online softmax, in wave 0 of split 0
+        if (sp == 0 && wave == 0) {
+            float dot = 0.f;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) vf.v[i] = v0[i];
-                } else {
+            for (int ks = 0; ks < NKS; ++ks) {
+                const int d0 = ks * 32 + grp * 8;
+                if (d0 < hd) {
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) vf.v[i] = from_f32<elem_t>(0.f);
+                    for (int e = 0; e < 8; ++e) dot += to_f32(qf[ks].v[e]) * knew[d0 + e];
                 }
-                if (pb >= 0 && d < hd) {
-                    const elem_t* v1 = a.vpool + (((size_t)pb * a.KV + kvh) * hd + d) * ps + kb % ps;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) vf.v[4 + i] = v1[i];
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) vf.v[4 + i] = from_f32<elem_t>(0.f);
-                }
-                mma_16x16x32(acc_o[dt], vf, pf);
             }
+            dot += __shfl_xor(dot, 16, WAVE);
+            dot += __shfl_xor(dot, 32, WAVE);
+            const float sv = valid ? dot * a.scale : -INFINITY;
+            const float m_new = fmaxf(m_run, sv);
+            const float alpha = exp_f(m_run - m_new), p = exp_f(sv - m_new);
+            l_run = l_run * alpha + p;
+            m_run = m_new;
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int d = dt * 16 + grp * 4 + i;
+                    acc_o[dt][i] = acc_o[dt][i] * alpha + (d < hd ? p * vnew[d] : 0.f);
+                }
         }
     }
 
@@ -438,66 +516,73 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
             for (int i = 0; i < 4; ++i) sm_o[wave - 1][dt * 16 + grp * 4 + i][r16] = acc_o[dt][i];
     }
     __syncthreads();
-    if (wave == 0) {
-        float m_all = m_run;
+    if (wave > 0) return;
+    float m_all = m_run;
 #pragma unroll
-        for (int w = 0; w < 3; ++w) m_all = fmaxf(m_all, sm_m[w][r16]);
-        const float c0 = exp_f(m_run - m_all);
-        float l_all = l_run * c0;
+    for (int w = 0; w < 3; ++w) m_all = fmaxf(m_all, sm_m[w][r16]);
+    const float c0 = exp_f(m_run - m_all);
+    float l_all = l_run * c0;
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc_o[dt][i] *= c0;
+#pragma unroll
+    for (int w = 0; w < 3; ++w) {
+        const float c = exp_f(sm_m[w][r16] - m_all);
+        l_all += sm_l[w][r16] * c;
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc_o[dt][i] *= c0;
+            for (int i = 0; i < 4; ++i) acc_o[dt][i] += sm_o[w][dt * 16 + grp * 4 + i][r16] * c;
+    }
+    if (!valid) return;
+    if (a.nsplit == 1) {
+        const float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
+        elem_t* orow = a.out + ((size_t)s * a.H + head) * hd;
 #pragma unroll
-        for (int w = 0; w < 3; ++w) {
-            const float c = exp_f(sm_m[w][r16] - m_all);
-            l_all += sm_l[w][r16] * c;
+        for (int dt = 0; dt < ND; ++dt) {
+            const int d0 = dt * 16 + grp * 4;
+            if (d0 < hd) {
 #pragma unroll
-            for (int dt = 0; dt < ND; ++dt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc_o[dt][i] += sm_o[w][dt * 16 + grp * 4 + i][r16] * c;
-        }
-        if (valid && a.nsplit == 1) {
-            const float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
-            elem_t* orow = a.out + ((size_t)s * a.H + head) * hd;
-#pragma unroll
-            for (int dt = 0; dt < ND; ++dt) {
-                const int d0 = dt * 16 + grp * 4;
-                if (d0 < hd) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) orow[d0 + i] = from_f32<elem_t>(acc_o[dt][i] * inv);
-                }
+                for (int i = 0; i < 4; ++i) orow[d0 + i] = from_f32<elem_t>(acc_o[dt][i] * inv);
             }
-        } else if (valid) {
-            const size_t base = ((size_t)s * a.H + head) * a.nsplit + sp;
-            float* po = a.part_o + base * hd;
-#pragma unroll
-            for (int dt = 0; dt < ND; ++dt) {
-                const int d0 = dt * 16 + grp * 4;
-                if (d0 < hd) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) po[d0 + i] = acc_o[dt][i];
-                }
-            }
-            if (grp == 0) { a.part_ml[base * 2] = m_all; a.part_ml[base * 2 + 1] = l_all; }
         }
+    } else {
+        const size_t base = ((size_t)s * a.H + head) * a.nsplit + sp;
+        float* po = a.part_o + base * hd;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) {
+            const int d0 = dt * 16 + grp * 4;
+            if (d0 < hd) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) po[d0 + i] = acc_o[dt][i];
+            }
+        }
+        if (grp == 0) { a.part_ml[base * 2] = m_all; a.part_ml[base * 2 + 1] = l_all; }
     }
 }
 
 // out[row, :] = sum_sp o_sp exp(m_sp - m) / sum_sp l_sp exp(m_sp - m), splits in order
 __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                           elem_t* __restrict__ out, int hd, int nsplit) {
+    __shared__ float coef[MAX_SPLITS];
     const size_t row = blockIdx.x;  // (request, head)
+    const int lane = threadIdx.x;
     const float* ml = part_ml + row * nsplit * 2;
-    float m = NEG_BIG;
-    for (int sp = 0; sp < nsplit; ++sp) m = fmaxf(m, ml[sp * 2]);
+    // every lane holds one split's (max, sum); nsplit <= 64
+    const float m_own = lane < nsplit ? ml[lane * 2] : NEG_BIG;
+    const float l_own = lane < nsplit ? ml[lane * 2 + 1] : 0.f;
+    const float m = wave_max(m_own);
+    const float c = lane < nsplit ? exp_f(m_own - m) : 0.f;
     float l = 0.f;
-    for (int sp = 0; sp < nsplit; ++sp) l += ml[sp * 2 + 1] * exp_f(ml[sp * 2] - m);
+    for (int sp = 0; sp < nsplit; ++sp) l += __shfl(l_own * c, sp, WAVE);  // in split order
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    for (int d = threadIdx.x; d < hd; d += 64) {
+    if (lane < nsplit) coef[lane] = c * inv;
+    __syncthreads();
+    for (int d = lane; d < hd; d += 64) {
         float o = 0.f;
-        for (int sp = 0; sp < nsplit; ++sp) o += part_o[(row * nsplit + sp) * hd + d] * exp_f(ml[sp * 2] - m);
-        out[row * hd + d] = from_f32<elem_t>(o * inv);
+        for (int sp = 0; sp < nsplit; ++sp) o += part_o[(row * nsplit + sp) * hd + d] * coef[sp];
+        out[row * hd + d] = from_f32<elem_t>(o);
     }
 }
 

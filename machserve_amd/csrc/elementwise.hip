@@ -32,16 +32,17 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, con
     float* src = x + r * d;
     float ss = 0.f;
     for (int c = threadIdx.x; c < d; c += 256) {
+        const float wc = w[c];  // requested with the row, not after the reduction
         float v = src[c];
         for (int p = 0; p < n_partials; ++p) v += partials[p * partial_stride + r * d + c];
-        vals[c] = v;
         if (n_partials > 0 && !rows) src[c] = v;
+        vals[c] = v * wc;
         ss += v * v;
     }
     ss = block_sum<256>(ss, scratch);
     const float inv = 1.0f / sqrtf(ss / (float)d + eps);
     OutT* dst = out + (size_t)i * d;
-    for (int c = threadIdx.x; c < d; c += 256) dst[c] = from_f32<OutT>(vals[c] * inv * w[c]);
+    for (int c = threadIdx.x; c < d; c += 256) dst[c] = from_f32<OutT>(vals[c] * inv);
 }
 
 // x[t, :] += sum_p partials[p, t, :] (in order): pending sums folded in without a norm

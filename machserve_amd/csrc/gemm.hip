@@ -160,10 +160,17 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
     MS_REQUIRE((reinterpret_cast<uintptr_t>(A) & 15) == 0 && (reinterpret_cast<uintptr_t>(W) & 15) == 0,
                "gemm: operands must be 16-byte aligned");
 #ifdef MS_ELEM_BF16
+    // the largest tile that still gives every CU of the chip a block or two
     if (M > 64) {
-        const long blocks = (long)ceil_div(M, 128) * ceil_div(N, 128);
-        hipLaunchKernelGGL((gemm_kernel<128, 128, 2, 2, EPI>), dim3((unsigned)blocks), dim3(256), 0, stream, A, W, M, N, K, ep);
-        return check_launch("gemm 128x128");
+        const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128), b12864 = (long)ceil_div(M, 128) * ceil_div(N, 64);
+        if (b128 >= 384) {
+            hipLaunchKernelGGL((gemm_kernel<128, 128, 2, 2, EPI>), dim3((unsigned)b128), dim3(256), 0, stream, A, W, M, N, K, ep);
+            return check_launch("gemm 128x128");
+        }
+        if (b12864 >= 384) {
+            hipLaunchKernelGGL((gemm_kernel<128, 64, 2, 2, EPI>), dim3((unsigned)b12864), dim3(256), 0, stream, A, W, M, N, K, ep);
+            return check_launch("gemm 128x64");
+        }
     }
 #endif
     const long blocks = (long)ceil_div(M, 64) * ceil_div(N, 64);

@@ -33,7 +33,42 @@ struct SampleArgs {
     int* out_token;
     float* out_logprob;
     int vocab;
+    // per-row partial maxima of ARGMAX_CHUNKS chunks of the row, or null: a greedy row scans itself
+    const float* part_val;
+    const int* part_idx;
 };
+
+constexpr int ARGMAX_CHUNKS = 64;
+
+// Stage one of greedy sampling: the row is cut into ARGMAX_CHUNKS contiguous chunks, one block each;
+// a block writes the maximum of its chunk and the smallest index that holds it.
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ logits, int vocab,
+                                                             float* __restrict__ part_val, int* __restrict__ part_idx) {
+    __shared__ float s_v[4];
+    __shared__ int s_i[4];
+    const int r = blockIdx.x, ch = blockIdx.y, tid = threadIdx.x;
+    const float* row = logits + (size_t)r * vocab;
+    const int len = ceil_div(vocab, ARGMAX_CHUNKS), i0 = ch * len, i1 = min(vocab, i0 + len);
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = i0 + tid; i < i1; i += 256) {
+        const float x = row[i];
+        if (bi == 0x7fffffff || x > best) { best = x; bi = i; }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, WAVE);
+        const int oi = __shfl_xor(bi, o, WAVE);
+        if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > best || (ov == best && oi < bi))) { best = ov; bi = oi; }
+    }
+    if ((tid & 63) == 0) { s_v[tid >> 6] = best; s_i[tid >> 6] = bi; }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < 4; ++w)
+            if (s_i[w] != 0x7fffffff && (bi == 0x7fffffff || s_v[w] > best || (s_v[w] == best && s_i[w] < bi))) { best = s_v[w]; bi = s_i[w]; }
+        part_val[r * ARGMAX_CHUNKS + ch] = best;
+        part_idx[r * ARGMAX_CHUNKS + ch] = bi;
+    }
+}
 
 __device__ __forceinline__ float block_max(float v, float* scratch) {
     v = wave_max(v);
@@ -68,6 +103,23 @@ __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs a) {
     const int seg_len = ceil_div(V, ST);
     const int i0 = min(V, tid * seg_len), i1 = min(V, i0 + seg_len);
 
+    if (T <= 0.0f && a.part_val) {
+        // stage two: the chunks' maxima, smallest index first among equals
+        if (tid < WAVE) {
+            float best = tid < ARGMAX_CHUNKS ? a.part_val[r * ARGMAX_CHUNKS + tid] : -INFINITY;
+            int bi = tid < ARGMAX_CHUNKS ? a.part_idx[r * ARGMAX_CHUNKS + tid] : 0x7fffffff;
+            for (int o = 32; o > 0; o >>= 1) {
+                const float ov = __shfl_xor(best, o, WAVE);
+                const int oi = __shfl_xor(bi, o, WAVE);
+                if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > best || (ov == best && oi < bi))) { best = ov; bi = oi; }
+            }
+            if (tid == 0) {
+                a.out_token[r] = bi;
+                a.out_logprob[r] = 0.0f;
+            }
+        }
+        return;
+    }
     if (T <= 0.0f) {
         // smallest index among the maxima.  A thread walks its strided indices in ascending
         // order and keeps the first maximum; ties between threads go to the smaller index.
@@ -201,11 +253,24 @@ __global__ void logit_edit_kernel(float* logits, int vocab, const int* row_of, c
 
 using namespace ms;
 
+// part_val / part_idx: float / int workspaces [rows, ms_sample_chunks()] for the two-stage greedy
+// search, or null (every row scans itself in one block).
+extern "C" int ms_sample_chunks() { return ARGMAX_CHUNKS; }
+
 extern "C" int ms_sample(const float* logits, const float* temperature, const int* top_k, const float* top_p,
-                         unsigned long long* state, int* out_token, float* out_logprob, int rows, int vocab,
-                         hipStream_t stream) {
+                         unsigned long long* state, int* out_token, float* out_logprob, float* part_val, int* part_idx,
+                         int rows, int vocab, hipStream_t stream) {
     MS_REQUIRE(rows > 0 && vocab > 0, "sample: empty problem rows=%d vocab=%d", rows, vocab);
-    SampleArgs a{logits, temperature, top_k, top_p, state, out_token, out_logprob, vocab};
+    static_assert(ARGMAX_CHUNKS <= WAVE, "stage two is one wave");
+    if (part_val && part_idx) {
+        hipLaunchKernelGGL(argmax_partial_kernel, dim3(rows, ARGMAX_CHUNKS), dim3(256), 0, stream, logits, vocab, part_val,
+                           part_idx);
+        if (int rc = check_launch("argmax_partial")) return rc;
+    } else {
+        part_val = nullptr;
+        part_idx = nullptr;
+    }
+    SampleArgs a{logits, temperature, top_k, top_p, state, out_token, out_logprob, vocab, part_val, part_idx};
     hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(ST), 0, stream, a);
     return check_launch("sample");
 }

@@ -70,8 +70,8 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
             aok[i] = m < a.M;
             arow[i] = a.A + (size_t)(aok[i] ? m : 0) * a.K;
         }
-        for (int kk = k0; kk < k1; kk += KSTEP) {
-            Frag fw[NT][4], fa[MT][4];
+        Frag fw[NT][4], fa[MT][4];
+        auto load = [&](int kk) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const int k = kk + (grp * 4 + c) * 8;
@@ -81,12 +81,24 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
 #pragma unroll
                 for (int i = 0; i < MT; ++i) fa[i][c] = (kok && aok[i]) ? frag_load(arow[i] + k) : frag_zero();
             }
+        };
+        if (k0 < k1) load(k0);
+        for (int kk = k0; kk < k1; kk += KSTEP) {
+            Frag cw[NT][4], ca[MT][4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+#pragma unroll
+                for (int j = 0; j < NT; ++j) cw[j][c] = fw[j][c];
+#pragma unroll
+                for (int i = 0; i < MT; ++i) ca[i][c] = fa[i][c];
+            }
+            if (kk + KSTEP < k1) load(kk + KSTEP);  // in flight while this slice is multiplied
 #pragma unroll
             for (int c = 0; c < 4; ++c)
 #pragma unroll
                 for (int i = 0; i < MT; ++i)
 #pragma unroll
-                    for (int j = 0; j < NT; ++j) mma_16x16x32(acc[i][j], fa[i][c], fw[j][c]);
+                    for (int j = 0; j < NT; ++j) mma_16x16x32(acc[i][j], ca[i][c], cw[j][c]);
         }
     }
 
@@ -159,18 +171,17 @@ struct SkinnyPlan { int wn, ksi, ksb, k_per_wave; };
 static SkinnyPlan plan_skinny(int N, int K, bool allow_partials) {
     constexpr int NT = 2;
     const int col_waves = ceil_div(N, 16 * NT);
-    const int max_slices = max(1, K / KSTEP);
-    int want = ceil_div(4096, col_waves);
-    want = max(1, min(want, max_slices));
+    const int slices = ceil_div(K, KSTEP);  // slices of 128 along K: one wave iteration each
+    int want = max(1, min(ceil_div(4096, col_waves), slices));  // waves wanted along K
     SkinnyPlan p;
     if (want == 1) {
-        p = {4, 1, 1, ceil_div(K, 32) * 32};
+        p = {4, 1, 1, slices * KSTEP};
         return p;
     }
     p.wn = 1;
-    p.ksi = want >= 8 ? 8 : (want >= 4 ? 4 : (want >= 2 ? 2 : 1));
-    p.ksb = allow_partials ? max(1, want / p.ksi) : 1;
-    p.k_per_wave = ceil_div(ceil_div(K, p.ksi * p.ksb), 32) * 32;
+    p.ksi = want > 4 ? 8 : (want > 2 ? 4 : 2);
+    p.ksb = (allow_partials && want > p.ksi) ? ceil_div(want, p.ksi) : 1;
+    p.k_per_wave = ceil_div(slices, p.ksi * p.ksb) * KSTEP;
     return p;
 }
 

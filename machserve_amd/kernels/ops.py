@@ -232,7 +232,7 @@ class HipOps:
     def _decode_splits(S: int, KV: int, table_width: int, page_size: int, window: Optional[int], key_tile: int) -> int:
         span = table_width * page_size if not window else min(table_width * page_size, window + key_tile)
         tiles = max(1, -(-span // key_tile))
-        return max(1, min(-(-1024 // (S * KV)), -(-tiles // 4), 64))
+        return max(1, min(-(-512 // (S * KV)), -(-tiles // 4), 64))
 
     def decode_attention_fused(self, qkv: torch.Tensor, bias: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor],
                                slot_map: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
@@ -303,9 +303,10 @@ class HipOps:
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-               state: torch.Tensor):
+               state: torch.Tensor, any_greedy: bool = True):
         """One token per row; ``state`` (int64 SplitMix64 states) advances in place.
-        Returns ``(tokens int32, logprobs float32)``."""
+        Returns ``(tokens int32, logprobs float32)``.  With ``any_greedy`` a first launch finds the
+        maxima of 64 chunks of every row, so that a greedy row is not one block's serial scan."""
         W, V = logits.shape
         self._want(logits, torch.float32, "sample logits")
         self._want(temperature, torch.float32, "sample temperature", W)
@@ -314,8 +315,14 @@ class HipOps:
         self._want(state, torch.int64, "sample state", W)
         tok = torch.empty(W, dtype=torch.int32, device=logits.device)
         lp = torch.empty(W, dtype=torch.float32, device=logits.device)
+        pv = pi = None
+        if any_greedy:
+            chunks = self._core.ms_sample_chunks()
+            pv = torch.empty((W, chunks), dtype=torch.float32, device=logits.device)
+            pi = torch.empty((W, chunks), dtype=torch.int32, device=logits.device)
         self._check(self._core, self._core.ms_sample(_ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p),
-                                                     _ptr(state), _ptr(tok), _ptr(lp), _c_int(W), _c_int(V), _stream()))
+                                                     _ptr(state), _ptr(tok), _ptr(lp), _ptr(pv), _ptr(pi), _c_int(W),
+                                                     _c_int(V), _stream()))
         return tok, lp
 
     def logit_edit(self, logits: torch.Tensor, row_of: torch.Tensor, token: torch.Tensor, delta: torch.Tensor) -> None:

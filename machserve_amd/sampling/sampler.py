@@ -53,6 +53,6 @@ class Sampler:
         fdev = torch.from_numpy(fl).to(self.device)
         kdev = torch.tensor([p.top_k for p in params], dtype=torch.int32, device=self.device)
         sdev = torch.tensor([_signed(s) for s in states], dtype=torch.int64, device=self.device)
-        tok, lp = self.ops.sample(logits, fdev[0], kdev, fdev[1], sdev)
+        tok, lp = self.ops.sample(logits, fdev[0], kdev, fdev[1], sdev, any(p.temperature <= 0.0 for p in params))
         tokens = tok.cpu().tolist()  # the step's one synchronisation
         return tokens, lp.cpu().tolist(), [advance(s) for s in states]

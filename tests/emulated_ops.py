@@ -136,7 +136,7 @@ class EmulatedOps:
         return self.paged_attention(q, kpool, vpool, block_table, ar, torch.ones_like(ar), seq_pos0, work, H, KV, hd,
                                     page_size, window, scale)
 
-    def sample(self, logits, temperature, top_k, top_p, state):
+    def sample(self, logits, temperature, top_k, top_p, state, any_greedy=True):
         from plain.qwen2_plain import sample as plain_sample
         toks, lps = [], []
         for r in range(logits.shape[0]):

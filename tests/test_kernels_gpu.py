@@ -328,7 +328,7 @@ def test_sampler_matches_cpu_mirror():
     seeds = torch.tensor([7000 + i for i in range(n)], dtype=torch.int64)
     state = seeds.clone().to(DEV)
     for rep in range(3):
-        got, _ = ops.sample(logits.to(DEV), temps.to(DEV), ks.to(DEV), ps_.to(DEV), state)
+        got, _ = ops.sample(logits.to(DEV), temps.to(DEV), ks.to(DEV), ps_.to(DEV), state, any_greedy=rep != 1)
         for i in range(n):
             st = int(seeds[i]) + rep * P.RNG_GOLDEN
             want, new = P.sample(logits[i].numpy(), float(temps[i]), int(ks[i]), float(ps_[i]), st & P.MASK64)
@@ -348,6 +348,14 @@ def test_sampler_greedy_ties_and_spread():
     tok, lp = ops.sample(logits.to(DEV), z.to(DEV), torch.zeros(3, dtype=torch.int32, device=DEV), torch.ones(3).to(DEV),
                          torch.zeros(3, dtype=torch.int64, device=DEV))
     assert tok.cpu().tolist() == [5, 999, int(logits[2].argmax())]
+    tok, lp = ops.sample(logits.to(DEV), z.to(DEV), torch.zeros(3, dtype=torch.int32, device=DEV), torch.ones(3).to(DEV),
+                         torch.zeros(3, dtype=torch.int64, device=DEV), any_greedy=False)  # the one-block scan agrees
+    assert tok.cpu().tolist() == [5, 999, int(logits[2].argmax())]
+    big = torch.randn(5, 151936, generator=torch.Generator().manual_seed(2))
+    big[3, [77, 150000]] = 9.0
+    tok, _ = ops.sample(big.to(DEV), torch.zeros(5).to(DEV), torch.zeros(5, dtype=torch.int32, device=DEV), torch.ones(5).to(DEV),
+                        torch.zeros(5, dtype=torch.int64, device=DEV))
+    assert tok.cpu().tolist() == [int(big[i].argmax()) if i != 3 else 77 for i in range(5)]
     # a flat distribution is covered by different seeds
     flat = torch.zeros(64, V)
     st = torch.arange(1, 65, dtype=torch.int64).to(DEV)
