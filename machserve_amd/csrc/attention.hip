@@ -111,12 +111,14 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
     for (int i = 0; i < ND; ++i) acc_o[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m_run = NEG_BIG, l_run = 0.f;
 
-    // Tiles go global -> registers -> LDS; the registers for the next tile are requested before
-    // the current tile is multiplied, so the memory latency hides behind the MFMAs.
+    // Tiles go global -> registers -> LDS.  PF tiles are in flight at any time: a tile's loads are
+    // requested PF tiles before it is multiplied, which covers the memory latency even when few
+    // blocks share a CU.
     constexpr int CPRK = HDT / EPC, CPRV = BKV / EPC;
     constexpr int NCK = (BKV * CPRK + 255) / 256, NCV = (HDT * CPRV + 255) / 256;
-    u32x4 rk[NCK], rv[NCV];
-    auto load_tile = [&](int kt0) {
+    constexpr int PF = ND <= 4 ? 4 : (ND <= 8 ? 2 : 1);
+    u32x4 rk[PF][NCK], rv[PF][NCV];
+    auto load_tile = [&](int kt0, u32x4* pk, u32x4* pv) {
 #pragma unroll
         for (int i = 0; i < NCK; ++i) {
             const int c = tid + i * 256;
@@ -127,7 +129,7 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
                 if (page >= 0)
                     v = *reinterpret_cast<const u32x4*>(a.kpool + (((size_t)page * a.KV + kvh) * ps + key % ps) * hd + d0);
             }
-            rk[i] = v;
+            pk[i] = v;
         }
 #pragma unroll
         for (int i = 0; i < NCV; ++i) {
@@ -139,28 +141,34 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
                 if (page >= 0)
                     v = *reinterpret_cast<const u32x4*>(a.vpool + (((size_t)page * a.KV + kvh) * hd + d) * ps + key % ps);
             }
-            rv[i] = v;
+            pv[i] = v;
         }
     };
-    auto store_tile = [&]() {
+    auto store_tile = [&](const u32x4* pk, const u32x4* pv) {
 #pragma unroll
         for (int i = 0; i < NCK; ++i) {
             const int c = tid + i * 256;
-            if (c < BKV * CPRK) *reinterpret_cast<u32x4*>(&Ks[(c / CPRK) * K_LD + (c % CPRK) * EPC]) = rk[i];
+            if (c < BKV * CPRK) *reinterpret_cast<u32x4*>(&Ks[(c / CPRK) * K_LD + (c % CPRK) * EPC]) = pk[i];
         }
 #pragma unroll
         for (int i = 0; i < NCV; ++i) {
             const int c = tid + i * 256;
-            if (c < HDT * CPRV) *reinterpret_cast<u32x4*>(&Vs[(c / CPRV) * V_LD + (c % CPRV) * EPC]) = rv[i];
+            if (c < HDT * CPRV) *reinterpret_cast<u32x4*>(&Vs[(c / CPRV) * V_LD + (c % CPRV) * EPC]) = pv[i];
         }
     };
     const int kt_first = (kv_lo / BKV) * BKV;
-    if (kt_first < kv_hi) load_tile(kt_first);
-    for (int kt0 = kt_first; kt0 < kv_hi; kt0 += BKV) {
+#pragma unroll
+    for (int j = 0; j < PF; ++j)
+        if (kt_first + j * BKV < kv_hi) load_tile(kt_first + j * BKV, rk[j], rv[j]);
+    for (int kt_base = kt_first; kt_base < kv_hi; kt_base += PF * BKV) {
+#pragma unroll
+      for (int j = 0; j < PF; ++j) {
+        const int kt0 = kt_base + j * BKV;
+        if (kt0 >= kv_hi) break;
         __syncthreads();  // the previous tile has been consumed
-        store_tile();
+        store_tile(rk[j], rv[j]);
         __syncthreads();
-        if (kt0 + BKV < kv_hi) load_tile(kt0 + BKV);
+        if (kt0 + PF * BKV < kv_hi) load_tile(kt0 + PF * BKV, rk[j], rv[j]);
         if (!wave_active) continue;
 
         // S^T = K Q^T: lane holds keys grp * 4 + i of tile nt for query row r16
@@ -233,6 +241,7 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
                 mma_16x16x32(acc_o[dt], vf, pf);
             }
         }
+      }
     }
 
     if (valid) {

@@ -31,6 +31,8 @@ struct EpiArgs {
     const float* bias;  // [N] or null
     int ldo;
     int n_out;          // SWIGLU: number of output columns (intermediate size)
+    int k_per_split;    // K range of one blockIdx.y slice (multiple of 32); K itself without split
+    size_t split_stride;  // STORE_F32 with gridDim.y > 1: elements between the slices' outputs
 };
 
 __device__ __forceinline__ float silu_f(float g) {
@@ -57,20 +59,21 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
     const int m0 = (blockIdx.x % tiles_m) * BM, n0 = (blockIdx.x / tiles_m) * BN;
     const int r16 = lane & 15, grp = lane >> 4;
 
+    const int k_end = min(K, (int)(blockIdx.y + 1) * ep.k_per_split);
     u32x4 ra[A_CHUNKS], rw[W_CHUNKS];
     auto load_global = [&](int k0) {
 #pragma unroll
         for (int i = 0; i < A_CHUNKS; ++i) {
             const int c = tid + i * 256, row = c / CPR, kk = k0 + (c % CPR) * EPC;
             u32x4 v = {0, 0, 0, 0};
-            if (m0 + row < M && kk < K) v = *reinterpret_cast<const u32x4*>(A + (size_t)(m0 + row) * K + kk);
+            if (m0 + row < M && kk < k_end) v = *reinterpret_cast<const u32x4*>(A + (size_t)(m0 + row) * K + kk);
             ra[i] = v;
         }
 #pragma unroll
         for (int i = 0; i < W_CHUNKS; ++i) {
             const int c = tid + i * 256, row = c / CPR, kk = k0 + (c % CPR) * EPC;
             u32x4 v = {0, 0, 0, 0};
-            if (n0 + row < N && kk < K) v = *reinterpret_cast<const u32x4*>(W + (size_t)(n0 + row) * K + kk);
+            if (n0 + row < N && kk < k_end) v = *reinterpret_cast<const u32x4*>(W + (size_t)(n0 + row) * K + kk);
             rw[i] = v;
         }
     };
@@ -93,13 +96,15 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    const int nk = ceil_div(K, BK);
-    load_global(0);
+    // a slice of K per blockIdx.y: partial sums that the consumer adds in slice order
+    const int k_begin = blockIdx.y * ep.k_per_split;
+    const int nk = ceil_div(k_end - k_begin, BK);
+    load_global(k_begin);
     store_lds(0);
     __syncthreads();
     for (int kt = 0; kt < nk; ++kt) {
         const int buf = kt & 1;
-        if (kt + 1 < nk) load_global((kt + 1) * BK);
+        if (kt + 1 < nk) load_global(k_begin + (kt + 1) * BK);
         Frag fa[TM], fb[TN];
 #pragma unroll
         for (int i = 0; i < TM; ++i) fa[i] = frag_load(&As[buf][(wm * (BM / WM) + i * 16 + r16) * LDS_LD + grp * 8]);
@@ -145,7 +150,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
                     if (row >= M) continue;
                     const size_t o = (size_t)row * ep.ldo + col;
                     const float v = acc[i][j][e] + b;
-                    if constexpr (EPI == EPI_STORE_F32) reinterpret_cast<float*>(ep.out)[o] = v;
+                    if constexpr (EPI == EPI_STORE_F32) reinterpret_cast<float*>(ep.out)[blockIdx.y * ep.split_stride + o] = v;
                     else if constexpr (EPI == EPI_STORE_ELEM) reinterpret_cast<elem_t*>(ep.out)[o] = from_f32<elem_t>(v);
                     else reinterpret_cast<float*>(ep.out)[o] += v;  // residual stream, 32-bit
                 }
@@ -154,28 +159,47 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
 }
 
 template <int EPI>
-static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, EpiArgs ep, hipStream_t stream) {
+static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, EpiArgs ep, hipStream_t stream,
+                       int nsplit = 1) {
     MS_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: empty problem M=%d N=%d K=%d", M, N, K);
     MS_REQUIRE(K % 8 == 0, "gemm: the reduction size K=%d must be a multiple of 8", K);
     MS_REQUIRE((reinterpret_cast<uintptr_t>(A) & 15) == 0 && (reinterpret_cast<uintptr_t>(W) & 15) == 0,
                "gemm: operands must be 16-byte aligned");
+    MS_REQUIRE(nsplit >= 1 && (nsplit == 1 || EPI == EPI_STORE_F32), "gemm: %d K slices need the float store", nsplit);
+    ep.k_per_split = ceil_div(ceil_div(K, nsplit), BK) * BK;
+    ep.split_stride = (size_t)M * N;
+    const unsigned ns = (unsigned)ceil_div(K, ep.k_per_split);
 #ifdef MS_ELEM_BF16
     // the largest tile that still gives every CU of the chip a block or two
     if (M > 64) {
         const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128), b12864 = (long)ceil_div(M, 128) * ceil_div(N, 64);
-        if (b128 >= 384) {
-            hipLaunchKernelGGL((gemm_kernel<128, 128, 2, 2, EPI>), dim3((unsigned)b128), dim3(256), 0, stream, A, W, M, N, K, ep);
+        if (b128 * ns >= 300) {
+            hipLaunchKernelGGL((gemm_kernel<128, 128, 2, 2, EPI>), dim3((unsigned)b128, ns), dim3(256), 0, stream, A, W, M, N, K, ep);
             return check_launch("gemm 128x128");
         }
-        if (b12864 >= 384) {
-            hipLaunchKernelGGL((gemm_kernel<128, 64, 2, 2, EPI>), dim3((unsigned)b12864), dim3(256), 0, stream, A, W, M, N, K, ep);
+        if (b12864 * ns >= 300) {
+            hipLaunchKernelGGL((gemm_kernel<128, 64, 2, 2, EPI>), dim3((unsigned)b12864, ns), dim3(256), 0, stream, A, W, M, N, K, ep);
             return check_launch("gemm 128x64");
         }
     }
 #endif
     const long blocks = (long)ceil_div(M, 64) * ceil_div(N, 64);
-    hipLaunchKernelGGL((gemm_kernel<64, 64, 2, 2, EPI>), dim3((unsigned)blocks), dim3(256), 0, stream, A, W, M, N, K, ep);
+    hipLaunchKernelGGL((gemm_kernel<64, 64, 2, 2, EPI>), dim3((unsigned)blocks, ns), dim3(256), 0, stream, A, W, M, N, K, ep);
     return check_launch("gemm 64x64");
+}
+
+// K slices for a product of many rows whose consumer adds partial sums: enough 128x128 blocks to
+// fill the chip, at least 512 of K each.  The 32-bit build never slices: its sums keep one order.
+static int plan_tiled_splits(int M, int N, int K) {
+#ifdef MS_ELEM_BF16
+    const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
+    if (b128 >= 300) return 1;
+    int want = (int)ceil_div(300, b128);
+    return max(1, min(want, K / 512));
+#else
+    (void)M; (void)N; (void)K;
+    return 1;
+#endif
 }
 
 }  // namespace ms
@@ -185,14 +209,14 @@ using namespace ms;
 // out[M, N] = a[M, K] w[N, K]^T (+ bias[N]); out is float when out_f32 != 0, else the element type.
 extern "C" int ms_linear(const void* a, const void* w, const float* bias, void* out, int out_f32, int M, int N, int K,
                          hipStream_t stream) {
-    EpiArgs ep{out, bias, N, N};
+    EpiArgs ep{out, bias, N, N, 0, 0};
     if (out_f32) return launch_gemm<EPI_STORE_F32>((const elem_t*)a, (const elem_t*)w, M, N, K, ep, stream);
     return launch_gemm<EPI_STORE_ELEM>((const elem_t*)a, (const elem_t*)w, M, N, K, ep, stream);
 }
 
 // x[M, N] += a[M, K] w[N, K]^T, x being the 32-bit residual stream.
 extern "C" int ms_linear_residual(const void* a, const void* w, float* x, int M, int N, int K, hipStream_t stream) {
-    EpiArgs ep{x, nullptr, N, N};
+    EpiArgs ep{x, nullptr, N, N, 0, 0};
     return launch_gemm<EPI_RESIDUAL>((const elem_t*)a, (const elem_t*)w, M, N, K, ep, stream);
 }
 
@@ -201,6 +225,15 @@ extern "C" int ms_linear_residual(const void* a, const void* w, float* x, int M,
 // up rows; w has 2 * ceil16(I) rows, the padding rows being zero.
 extern "C" int ms_linear_swiglu(const void* a, const void* w, void* out, int M, int I, int K, hipStream_t stream) {
     const int n = 2 * ceil_div(I, 16) * 16;
-    EpiArgs ep{out, nullptr, I, I};
+    EpiArgs ep{out, nullptr, I, I, 0, 0};
     return launch_gemm<EPI_SWIGLU>((const elem_t*)a, (const elem_t*)w, M, n, K, ep, stream);
+}
+
+// Number of partial sums ms_linear_split_tiled writes for this problem (1 = the complete product).
+extern "C" int ms_tiled_partials(int M, int N, int K) { return plan_tiled_splits(M, N, K); }
+
+// out[ks, M, N] (float) = partial sums of a w^T over ms_tiled_partials(M, N, K) slices of K.
+extern "C" int ms_linear_split_tiled(const void* a, const void* w, float* out, int M, int N, int K, hipStream_t stream) {
+    EpiArgs ep{out, nullptr, N, N, 0, 0};
+    return launch_gemm<EPI_STORE_F32>((const elem_t*)a, (const elem_t*)w, M, N, K, ep, stream, plan_tiled_splits(M, N, K));
 }

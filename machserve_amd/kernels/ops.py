@@ -142,7 +142,13 @@ class HipOps:
         whatever else is in the batch."""
         M, N, K = self._mm_operands(a, w, "linear_split")
         if M > self.SKINNY_ROWS:
-            return self.linear(a, w, None, out_f32=True).unsqueeze(0)
+            P = self._core.ms_tiled_partials(_c_int(M), _c_int(N), _c_int(K)) if allow_partials else 1
+            if P == 1:
+                return self.linear(a, w, None, out_f32=True).unsqueeze(0)
+            out = torch.empty((P, M, N), dtype=torch.float32, device=a.device)
+            self._check(self._core, self._core.ms_linear_split_tiled(_ptr(a), _ptr(w), _ptr(out), _c_int(M), _c_int(N),
+                                                                     _c_int(K), _stream()))
+            return out
         P = self._core.ms_skinny_partials(_c_int(N), _c_int(K), _c_int(int(allow_partials)))
         out = torch.empty((P, M, N), dtype=torch.float32, device=a.device)
         self._check(self._core, self._core.ms_linear_skinny(_ptr(a), _ptr(w), _ptr(out), _c_int(M), _c_int(N), _c_int(K),
@@ -163,12 +169,12 @@ class HipOps:
         return out
 
     def linear_residual(self, a: torch.Tensor, w: torch.Tensor, x: torch.Tensor) -> Optional[torch.Tensor]:
-        """``x += a @ w.T`` in the 32-bit residual stream.  With few rows the sum is not added here:
-        the float32 partial sums ``[P, M, N]`` are returned for the consumer (the next norm) to
-        fold in; otherwise None."""
+        """``x += a @ w.T`` in the 32-bit residual stream.  When the product is cut along K (few rows,
+        or too few tiles to fill the chip) the sum is not added here: the float32 partial sums
+        ``[P, M, N]`` are returned for the consumer (the next norm) to fold in; otherwise None."""
         M, N, K = self._mm_operands(a, w, "linear_residual")
         self._want(x, torch.float32, "residual stream", M, N)
-        if M <= self.SKINNY_ROWS:
+        if M <= self.SKINNY_ROWS or self._core.ms_tiled_partials(_c_int(M), _c_int(N), _c_int(K)) > 1:
             return self.linear_split(a, w)
         self._check(self._core, self._core.ms_linear_residual(_ptr(a), _ptr(w), _ptr(x), _c_int(M), _c_int(N), _c_int(K),
                                                               _stream()))

@@ -71,11 +71,23 @@ def test_linear(dtype, M, N, K):
     assert_close(ops.linear(a.to(DEV), w.to(DEV), None), P.linear(a.double(), w.double()), dtype, "linear")
     x = rnd((M, N), torch.float32, 8)
     xd = x.to(DEV).clone()
-    pending = ops.linear_residual(a.to(DEV), w.to(DEV), xd)
-    assert (pending is not None) == (M <= 64)
+    pending = ops.linear_residual(a.to(DEV), w.to(DEV), xd)  # few rows, or few tiles and a long K: partial sums
+    assert pending is not None or M > 64
     if pending is not None:
         ops.add_partials(xd, pending)
     assert_close(xd, x.double() + P.linear(a.double(), w.double()), torch.float32 if dtype == torch.float32 else dtype, "linear_residual")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(65, 896, 4864), (300, 130, 1096), (2048, 896, 4864), (200, 200, 520)])
+def test_linear_many_rows_cut_along_k(dtype, M, N, K):
+    """A product with too few tiles to fill the chip is cut along K into ordered partial sums."""
+    ops = ops_for(dtype)
+    a, w = rnd((M, K), dtype, 41), rnd((N, K), dtype, 42, K ** -0.5)
+    parts = ops.linear_split(a.to(DEV), w.to(DEV))
+    assert parts.shape[1:] == (M, N) and (dtype == torch.bfloat16 or parts.shape[0] == 1)
+    assert_close(parts.sum(0), P.linear(a.double(), w.double()), torch.float32 if dtype == torch.float32 else dtype)
+    assert ops.linear_split(a.to(DEV), w.to(DEV), allow_partials=False).shape[0] == 1
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
