@@ -54,12 +54,20 @@ class Engine:
             entries.append(StepEntry(it.request.slot, toks, [it.count - 1] if it.sample else []))
             if it.sample:
                 sampled_items.append(it)
-        logits = self.loaded.step(entries, borrow_logits=True)
         self.steps += 1
         self.tokens_run += plan.n_tokens
+        reqs = [it.request for it in sampled_items]
+        if len(sampled_items) == len(plan.items) and not any(r.params.edits_logits() for r in reqs):
+            # every request decodes one token: forward pass and sampling are one captured graph
+            fast = self.loaded.step.decode_and_sample(
+                entries, [r.params.temperature for r in reqs], [r.params.top_k for r in reqs],
+                [r.params.top_p for r in reqs], [r.rng_state for r in reqs])
+            if fast is not None:
+                from ..sampling import advance
+                return self.scheduler.update(plan, fast[0], fast[1], [advance(r.rng_state) for r in reqs])
+        logits = self.loaded.step(entries, borrow_logits=True)
         if not sampled_items:
             return self.scheduler.update(plan, [])
-        reqs = [it.request for it in sampled_items]
         tokens, logprobs, states = self.sampler.sample(logits, [r.params for r in reqs], [r.rng_state for r in reqs],
                                                        [r.generated for r in reqs])
         return self.scheduler.update(plan, tokens, logprobs, states)

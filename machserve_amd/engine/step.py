@@ -39,6 +39,7 @@ class _DecodeGraph:
 
     def __init__(self, graph, dev, pinned, offsets, sizes, logits):
         self.graph, self.dev, self.pinned, self.offsets, self.sizes, self.logits = graph, dev, pinned, offsets, sizes, logits
+        self.sampled = None  # int32 [2, B] when the graph also samples: tokens, bits of the logprobs
         self.copied = torch.cuda.Event()  # the last upload of `pinned` has finished
 
 
@@ -180,7 +181,10 @@ class StepFunction:
             ctx.attention_work[g] = sec(f"work/{g}").view(-1, 2)
         return ctx
 
-    def _run_decode_graph(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def _run_decode_graph(self, entries: Sequence[StepEntry], sampling=None):
+        """Replay (or first capture) the graph of this batch size.  ``sampling`` = (temperatures,
+        top_ks, top_ps, states) makes sampling part of the graph; the result is then the int32
+        ``[2, B]`` tensor of :meth:`HipOps.sample_packed`, else the logits."""
         cache = self.cache
         slots = [e.slot for e in entries]
         tokens = [int(e.tokens[0]) for e in entries]
@@ -193,8 +197,14 @@ class StepFunction:
         B = len(slots)
         bucket = self.TABLE_BUCKET
         widths = {name: -(-max(len(cache.table(name, s)) for s in slots) // bucket) * bucket for name in cache.groups}
-        key = (B, tuple(sorted(widths.items())))
+        key = (B, tuple(sorted(widths.items())), sampling is not None)
         sections = self._decode_sections(slots, tokens, widths)
+        if sampling is not None:
+            temps, top_ks, top_ps, states = sampling
+            sections["sample/temperature"] = np.asarray(temps, dtype=np.float32).view(np.int32)
+            sections["sample/top_p"] = np.asarray(top_ps, dtype=np.float32).view(np.int32)
+            sections["sample/top_k"] = np.asarray(top_ks, dtype=np.int32)
+            sections["sample/state"] = np.asarray(states, dtype=np.uint64).view(np.int32)
         dg = self._graphs.get(key)
         if dg is None:
             offsets, sizes, total = {}, {}, 0
@@ -218,13 +228,42 @@ class StepFunction:
             with torch.cuda.stream(side):
                 self.model.forward(ctx)  # everything is loaded and compiled before the capture
             torch.cuda.current_stream().wait_stream(side)
+            def sec(k):
+                return dg.dev[dg.offsets[k]:dg.offsets[k] + dg.sizes[k]]
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 dg.logits = self.model.forward(ctx)
+                if sampling is not None:
+                    dg.sampled = self.rt.ops.sample_packed(
+                        dg.logits, sec("sample/temperature").view(torch.float32), sec("sample/top_k"),
+                        sec("sample/top_p").view(torch.float32), sec("sample/state").view(torch.int64), True)
             dg.graph = graph
             self._graphs[key] = dg
         dg.graph.replay()
-        return dg.logits
+        return dg.sampled if sampling is not None else dg.logits
+
+    def decode_and_sample(self, entries: Sequence[StepEntry], temperatures, top_ks, top_ps, states):
+        """A decode-only step (one token per request) with sampling inside the captured graph: one
+        upload, one replay, one copy back.  Returns ``(tokens, logprobs)`` as host lists, or None
+        if this step cannot take that path (the caller then uses ``__call__`` and the sampler)."""
+        if not (self.use_graphs and all(len(e.tokens) == 1 for e in entries)
+                and len({e.slot for e in entries}) == len(entries)):
+            return None
+        cache = self.cache
+        reserved: Dict[str, int] = {}
+        for e in entries:
+            for k, v in cache.pages_needed(e.slot, 1).items():
+                reserved[k] = reserved.get(k, 0) + v
+        for k, v in reserved.items():
+            if cache.free_pages(k) < v:
+                from ..cache import OutOfPages
+                raise OutOfPages(f"group {k}: the step needs {v} new pages, {cache.free_pages(k)} are free")
+        for e in entries:
+            cache.extend(e.slot, 1)
+        both = self._run_decode_graph(entries, (temperatures, top_ks, top_ps, states)).cpu()  # the step's one sync
+        for e in entries:
+            cache.commit(e.slot, 1)
+        return both[0].tolist(), both[1].view(torch.float32).tolist()
 
     # ------------------------------------------------------------------ the step
     def __call__(self, entries: Sequence[StepEntry], borrow_logits: bool = False) -> Optional[torch.Tensor]:

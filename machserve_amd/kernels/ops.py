@@ -308,19 +308,26 @@ class HipOps:
         return out
 
     # ------------------------------------------------------------------ sampling
-    def sample(self, logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-               state: torch.Tensor, any_greedy: bool = True):
+    def sample(self, logits, temperature, top_k, top_p, state, any_greedy: bool = True):
         """One token per row; ``state`` (int64 SplitMix64 states) advances in place.
-        Returns ``(tokens int32, logprobs float32)``.  With ``any_greedy`` a first launch finds the
-        maxima of 64 chunks of every row, so that a greedy row is not one block's serial scan."""
+        Returns ``(tokens int32, logprobs float32)``."""
+        both = self.sample_packed(logits, temperature, top_k, top_p, state, any_greedy)
+        return both[0], both[1].view(torch.float32)
+
+    def sample_packed(self, logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+                      state: torch.Tensor, any_greedy: bool = True) -> torch.Tensor:
+        """:meth:`sample` with both results in one int32 tensor ``[2, W]`` (tokens, then the bits of
+        the logprobs) so that one copy brings them to the host.  With ``any_greedy`` a first
+        launch finds the maxima of 64 chunks of every row, so that a greedy row is not one
+        block's serial scan."""
         W, V = logits.shape
         self._want(logits, torch.float32, "sample logits")
         self._want(temperature, torch.float32, "sample temperature", W)
         self._want(top_k, torch.int32, "sample top_k", W)
         self._want(top_p, torch.float32, "sample top_p", W)
         self._want(state, torch.int64, "sample state", W)
-        tok = torch.empty(W, dtype=torch.int32, device=logits.device)
-        lp = torch.empty(W, dtype=torch.float32, device=logits.device)
+        both = torch.empty((2, W), dtype=torch.int32, device=logits.device)  # tokens, then logprob bits
+        tok, lp = both[0], both[1].view(torch.float32)
         pv = pi = None
         if any_greedy:
             chunks = self._core.ms_sample_chunks()
@@ -329,7 +336,7 @@ class HipOps:
         self._check(self._core, self._core.ms_sample(_ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p),
                                                      _ptr(state), _ptr(tok), _ptr(lp), _ptr(pv), _ptr(pi), _c_int(W),
                                                      _c_int(V), _stream()))
-        return tok, lp
+        return both
 
     def logit_edit(self, logits: torch.Tensor, row_of: torch.Tensor, token: torch.Tensor, delta: torch.Tensor) -> None:
         """``logits[row_of[e], token[e]] += delta[e]`` (penalties and biases merged on the host)."""
