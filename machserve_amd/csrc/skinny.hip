@@ -39,7 +39,7 @@ __device__ __forceinline__ float silu_sk(float g) {
 
 template <int MT, int NT, int WN, int KSI, int EPI>
 __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a) {
-    __shared__ float red[(KSI > 1 ? (KSI - 1) : 1) * WN * MT * NT * 4 * 64];
+    __shared__ float red[(KSI > 1 ? (KSI - 1) : 1) * WN * NT * 4 * 64];  // one row tile of every slice at a time
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wn = wave % WN, wk = wave / WN;
     const int r16 = lane & 15, grp = lane >> 4;
@@ -82,48 +82,60 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
                 for (int i = 0; i < MT; ++i) fa[i][c] = (kok && aok[i]) ? frag_load(arow[i] + k) : frag_zero();
             }
         };
-        if (k0 < k1) load(k0);
+        constexpr bool PREFETCH = MT * NT <= 8;  // a second set of fragments fits the registers
+        if (PREFETCH && k0 < k1) load(k0);
         for (int kk = k0; kk < k1; kk += KSTEP) {
-            Frag cw[NT][4], ca[MT][4];
+            if constexpr (PREFETCH) {
+                Frag cw[NT][4], ca[MT][4];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
+                for (int c = 0; c < 4; ++c) {
 #pragma unroll
-                for (int j = 0; j < NT; ++j) cw[j][c] = fw[j][c];
+                    for (int j = 0; j < NT; ++j) cw[j][c] = fw[j][c];
 #pragma unroll
-                for (int i = 0; i < MT; ++i) ca[i][c] = fa[i][c];
+                    for (int i = 0; i < MT; ++i) ca[i][c] = fa[i][c];
+                }
+                if (kk + KSTEP < k1) load(kk + KSTEP);  // in flight while this slice is multiplied
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int i = 0; i < MT; ++i)
+#pragma unroll
+                        for (int j = 0; j < NT; ++j) mma_16x16x32(acc[i][j], ca[i][c], cw[j][c]);
+            } else {
+                load(kk);
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int i = 0; i < MT; ++i)
+#pragma unroll
+                        for (int j = 0; j < NT; ++j) mma_16x16x32(acc[i][j], fa[i][c], fw[j][c]);
             }
-            if (kk + KSTEP < k1) load(kk + KSTEP);  // in flight while this slice is multiplied
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-#pragma unroll
-                for (int i = 0; i < MT; ++i)
-#pragma unroll
-                    for (int j = 0; j < NT; ++j) mma_16x16x32(acc[i][j], ca[i][c], cw[j][c]);
         }
     }
 
-    // sum the K slices of the block in slice order: slice 0 keeps its sums and adds 1, 2, ...
+    // sum the K slices of the block in slice order: slice 0 keeps its sums and adds 1, 2, ...;
+    // one 16-row tile per round keeps the LDS buffer small
     if constexpr (KSI > 1) {
-        if (wk > 0) {
-            float* dst = red + ((size_t)((wk - 1) * WN + wn) * MT * NT * 4) * 64;
 #pragma unroll
-            for (int i = 0; i < MT; ++i)
+        for (int i = 0; i < MT; ++i) {
+            if (i > 0) __syncthreads();
+            if (wk > 0) {
+                float* dst = red + ((size_t)((wk - 1) * WN + wn) * NT * 4) * 64;
 #pragma unroll
                 for (int j = 0; j < NT; ++j)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) dst[((i * NT + j) * 4 + e) * 64 + lane] = acc[i][j][e];
-        }
-        __syncthreads();
-        if (wk == 0) {
+                    for (int e = 0; e < 4; ++e) dst[(j * 4 + e) * 64 + lane] = acc[i][j][e];
+            }
+            __syncthreads();
+            if (wk == 0) {
 #pragma unroll
-            for (int s = 1; s < KSI; ++s) {
-                const float* src = red + ((size_t)((s - 1) * WN + wn) * MT * NT * 4) * 64;
-#pragma unroll
-                for (int i = 0; i < MT; ++i)
+                for (int s = 1; s < KSI; ++s) {
+                    const float* src = red + ((size_t)((s - 1) * WN + wn) * NT * 4) * 64;
 #pragma unroll
                     for (int j = 0; j < NT; ++j)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[i][j][e] += src[((i * NT + j) * 4 + e) * 64 + lane];
+                        for (int e = 0; e < 4; ++e) acc[i][j][e] += src[(j * 4 + e) * 64 + lane];
+                }
             }
         }
     }
@@ -168,8 +180,13 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
 // K per wave).  A function of N and K alone.
 struct SkinnyPlan { int wn, ksi, ksb, k_per_wave; };
 
-static SkinnyPlan plan_skinny(int N, int K, bool allow_partials) {
-    constexpr int NT = 2;
+// Columns per wave in units of 16: with more than 32 rows and enough columns to keep every CU busy,
+// a wave takes 64 columns, so that the rows it re-reads (from L2, they are shared by all waves)
+// weigh no more than the weights it streams.
+static int skinny_nt(int M, int N) { return (M > 32 && N >= 4096) ? 4 : 2; }
+
+static SkinnyPlan plan_skinny(int M, int N, int K, bool allow_partials) {
+    const int NT = skinny_nt(M, N);
     const int col_waves = ceil_div(N, 16 * NT);
     const int slices = ceil_div(K, KSTEP);  // slices of 128 along K: one wave iteration each
     int want = max(1, min(ceil_div(4096, col_waves), slices));  // waves wanted along K
@@ -185,13 +202,13 @@ static SkinnyPlan plan_skinny(int N, int K, bool allow_partials) {
     return p;
 }
 
-template <int MT, int EPI>
+template <int MT, int NT, int EPI>
 static int launch_skinny_mt(const SkinnyArgs& a0, const SkinnyPlan& p, hipStream_t stream) {
     SkinnyArgs a = a0;
     a.k_per_wave = p.k_per_wave;
-    const dim3 grid((unsigned)ceil_div(a.N, 32 * p.wn), (unsigned)p.ksb);
-#define MS_SK(WN_, KSI_)                                                                                         \
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, 2, WN_, KSI_, EPI>), grid, dim3(64 * WN_ * KSI_), 0, stream, a); \
+    const dim3 grid((unsigned)ceil_div(a.N, 16 * NT * p.wn), (unsigned)p.ksb);
+#define MS_SK(WN_, KSI_)                                                                                          \
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, WN_, KSI_, EPI>), grid, dim3(64 * WN_ * KSI_), 0, stream, a); \
     return check_launch("gemm_skinny")
     if (p.wn == 4) { MS_SK(4, 1); }
     if (p.ksi == 8) { MS_SK(1, 8); }
@@ -205,29 +222,33 @@ template <int EPI>
 static int launch_skinny(const SkinnyArgs& a, const SkinnyPlan& p, hipStream_t stream) {
     MS_REQUIRE(a.M > 0 && a.M <= 64, "skinny product: M=%d must be in 1..64", a.M);
     MS_REQUIRE(a.K % 8 == 0, "skinny product: the reduction size K=%d must be a multiple of 8", a.K);
-    if (a.M <= 16) return launch_skinny_mt<1, EPI>(a, p, stream);
-    if (a.M <= 32) return launch_skinny_mt<2, EPI>(a, p, stream);
-    if (a.M <= 48) return launch_skinny_mt<3, EPI>(a, p, stream);
-    return launch_skinny_mt<4, EPI>(a, p, stream);
+    if (a.M <= 16) return launch_skinny_mt<1, 2, EPI>(a, p, stream);
+    if (a.M <= 32) return launch_skinny_mt<2, 2, EPI>(a, p, stream);
+    if (skinny_nt(a.M, a.N) == 4) {
+        if (a.M <= 48) return launch_skinny_mt<3, 4, EPI>(a, p, stream);
+        return launch_skinny_mt<4, 4, EPI>(a, p, stream);
+    }
+    if (a.M <= 48) return launch_skinny_mt<3, 2, EPI>(a, p, stream);
+    return launch_skinny_mt<4, 2, EPI>(a, p, stream);
 }
 
 }  // namespace ms
 
 using namespace ms;
 
-// Number of partial sums ms_linear_skinny writes for this N and K (1 = the complete product).
-extern "C" int ms_skinny_partials(int N, int K, int allow_partials) { return plan_skinny(N, K, allow_partials != 0).ksb; }
+// Number of partial sums ms_linear_skinny writes for M rows of this N and K (1 = the complete product).
+extern "C" int ms_skinny_partials(int M, int N, int K, int allow_partials) { return plan_skinny(M, N, K, allow_partials != 0).ksb; }
 
 // out[ks, M, N] (float) = partial sums of a w^T; ks = ms_skinny_partials(N, K, allow_partials).
 extern "C" int ms_linear_skinny(const void* a, const void* w, float* out, int M, int N, int K, int allow_partials,
                                 hipStream_t stream) {
     SkinnyArgs args{(const elem_t*)a, (const elem_t*)w, out, M, N, K, 0, 0};
-    return launch_skinny<SK_STORE_F32>(args, plan_skinny(N, K, allow_partials != 0), stream);
+    return launch_skinny<SK_STORE_F32>(args, plan_skinny(M, N, K, allow_partials != 0), stream);
 }
 
 // out[M, I] = silu(a g^T) * (a u^T), gate and up rows interleaved in blocks of 16 (see ms_linear_swiglu).
 extern "C" int ms_linear_swiglu_skinny(const void* a, const void* w, void* out, int M, int I, int K, hipStream_t stream) {
     const int n = 2 * ceil_div(I, 16) * 16;
     SkinnyArgs args{(const elem_t*)a, (const elem_t*)w, out, M, n, K, 0, I};
-    return launch_skinny<SK_SWIGLU>(args, plan_skinny(n, K, false), stream);
+    return launch_skinny<SK_SWIGLU>(args, plan_skinny(M, n, K, false), stream);
 }

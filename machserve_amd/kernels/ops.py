@@ -149,7 +149,7 @@ class HipOps:
             self._check(self._core, self._core.ms_linear_split_tiled(_ptr(a), _ptr(w), _ptr(out), _c_int(M), _c_int(N),
                                                                      _c_int(K), _stream()))
             return out
-        P = self._core.ms_skinny_partials(_c_int(N), _c_int(K), _c_int(int(allow_partials)))
+        P = self._core.ms_skinny_partials(_c_int(M), _c_int(N), _c_int(K), _c_int(int(allow_partials)))
         out = torch.empty((P, M, N), dtype=torch.float32, device=a.device)
         self._check(self._core, self._core.ms_linear_skinny(_ptr(a), _ptr(w), _ptr(out), _c_int(M), _c_int(N), _c_int(K),
                                                             _c_int(int(allow_partials)), _stream()))

@@ -106,8 +106,9 @@ def test_linear_few_rows(dtype, M, N, K):
     assert whole.shape == (1, M, N)
     assert_close(whole[0], ref, torch.float32 if dtype == torch.float32 else dtype, "one sum")
     assert_close(ops.linear(a.to(DEV), w.to(DEV), None, out_f32=True), ref, torch.float32 if dtype == torch.float32 else dtype)
-    alone = ops.linear_split(a[M - 1:].to(DEV).contiguous(), w.to(DEV))
-    assert alone.shape[0] == parts.shape[0] and torch.equal(alone[:, 0], parts[:, M - 1]), "a row alone gives the same bits"
+    if M <= 32:  # up to 32 rows K is cut by N and K alone: a row by itself gives the same bits
+        alone = ops.linear_split(a[M - 1:].to(DEV).contiguous(), w.to(DEV))
+        assert alone.shape[0] == parts.shape[0] and torch.equal(alone[:, 0], parts[:, M - 1])
     x = rnd((M, N), torch.float32, 23).to(DEV)
     pend = ops.linear_residual(a.to(DEV), w.to(DEV), x)
     assert pend is not None and torch.equal(pend, parts)
