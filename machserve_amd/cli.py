@@ -76,6 +76,7 @@ def main(argv=None) -> int:
     ap.add_argument("--seed", type=int, default=0, help="sampling seed; 0 uses the request's id")
     ap.add_argument("--presence-penalty", type=float, default=0.0)
     ap.add_argument("--frequency-penalty", type=float, default=0.0)
+    ap.add_argument("--top-logprobs", type=int, default=0, help="report this many most probable tokens per step (--json)")
     ap.add_argument("--eos", type=int, default=None)
     ap.add_argument("--stop", action="append", default=[], help="a stop sequence of token ids, comma separated")
     ap.add_argument("--capacity", type=int, default=int(_env("MACH_CAPACITY", 64)), help="requests running at once")
@@ -120,13 +121,16 @@ def main(argv=None) -> int:
     for i, p in enumerate(prompts):
         params = SamplingParams(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p,
                                 seed=(args.seed + i) if args.seed else 0, presence_penalty=args.presence_penalty,
-                                frequency_penalty=args.frequency_penalty)
+                                frequency_penalty=args.frequency_penalty, top_logprobs=args.top_logprobs)
         ids.append(engine.add(p, args.max_new, params, args.eos, [_ids(s) for s in args.stop]))
     done = engine.run()
     for i, p in zip(ids, prompts):
         r = done[i]
         if args.json:
-            print(json.dumps({"prompt": p, "generated": r.generated, "finish_reason": r.finish_reason}))
+            rec = {"prompt": p, "generated": r.generated, "finish_reason": r.finish_reason, "logprobs": r.logprobs}
+            if args.top_logprobs:
+                rec["top_logprobs"] = r.top_logprobs
+            print(json.dumps(rec))
         else:
             print(" ".join(str(t) for t in r.generated))
     if tmp is not None:

@@ -249,9 +249,82 @@ __global__ void logit_edit_kernel(float* logits, int vocab, const int* row_of, c
     if (e < n && token[e] >= 0 && token[e] < vocab) logits[(size_t)row_of[e] * vocab + token[e]] += delta[e];
 }
 
+constexpr int TOPLP_MAX = 20;
+
+// The k most probable tokens of every row and their log-probabilities under the row's temperature
+// (`inv_t`; the host passes 1 for temperature <= 0), ties to the smaller token id:
+// logprob = (x - max) * inv_t - log(sum exp((x - max) * inv_t)).
+// Role in the reference: topk_batched (crates/mach-model/src/sampling.rs:411-539).  k rounds, each
+// a search for the best token after the previous pick in the order (logit descending, id ascending).
+__global__ __launch_bounds__(ST) void top_logprobs_kernel(const float* __restrict__ logits, const float* __restrict__ inv_t,
+                                                          int* __restrict__ out_tok, float* __restrict__ out_lp, int vocab,
+                                                          int k) {
+    __shared__ float scratch[ST / WAVE];
+    __shared__ float s_val[ST / WAVE];
+    __shared__ int s_idx[ST / WAVE];
+    __shared__ float s_last_v;
+    __shared__ int s_last_i;
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const float* row = logits + (size_t)r * vocab;
+    const float it = inv_t[r];
+    float mx = -INFINITY;
+    for (int i = tid; i < vocab; i += ST) mx = fmaxf(mx, row[i]);
+    const float maxv = block_max(mx, scratch);
+    const int seg_len = ceil_div(vocab, ST);
+    const int i0 = min(vocab, tid * seg_len), i1 = min(vocab, i0 + seg_len);
+    float part = 0.f;
+    for (int i = i0; i < i1; ++i) part += expf((row[i] - maxv) * it);
+    const float logz = logf(block_sum<ST>(part, scratch));
+    float last_v = INFINITY;
+    int last_i = -1;
+    for (int round = 0; round < k; ++round) {
+        float best = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int i = tid; i < vocab; i += ST) {
+            const float x = row[i];
+            const bool after = x < last_v || (x == last_v && i > last_i);
+            if (after && (bi == 0x7fffffff || x > best)) { best = x; bi = i; }
+        }
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(best, o, WAVE);
+            const int oi = __shfl_xor(bi, o, WAVE);
+            if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > best || (ov == best && oi < bi))) { best = ov; bi = oi; }
+        }
+        __syncthreads();
+        if ((tid & 63) == 0) { s_val[tid >> 6] = best; s_idx[tid >> 6] = bi; }
+        __syncthreads();
+        if (tid == 0) {
+            for (int w = 1; w < ST / WAVE; ++w)
+                if (s_idx[w] != 0x7fffffff && (bi == 0x7fffffff || s_val[w] > best || (s_val[w] == best && s_idx[w] < bi))) {
+                    best = s_val[w];
+                    bi = s_idx[w];
+                }
+            const bool found = bi != 0x7fffffff;
+            out_tok[(size_t)r * TOPLP_MAX + round] = found ? bi : -1;
+            out_lp[(size_t)r * TOPLP_MAX + round] = found ? (best - maxv) * it - logz : -INFINITY;
+            s_last_v = best;
+            s_last_i = found ? bi : 0x7fffffff;
+        }
+        __syncthreads();
+        last_v = s_last_v;
+        last_i = s_last_i;
+    }
+}
+
 }  // namespace ms
 
 using namespace ms;
+
+extern "C" int ms_top_logprobs_max() { return TOPLP_MAX; }
+
+// out_tok / out_lp: [rows, ms_top_logprobs_max()], the first k entries of a row are written.
+extern "C" int ms_top_logprobs(const float* logits, const float* inv_t, int* out_tok, float* out_lp, int rows, int vocab,
+                               int k, hipStream_t stream) {
+    MS_REQUIRE(rows > 0 && vocab > 0, "top_logprobs: empty problem rows=%d vocab=%d", rows, vocab);
+    MS_REQUIRE(k >= 1 && k <= TOPLP_MAX, "top_logprobs: k=%d must be in 1..%d", k, TOPLP_MAX);
+    hipLaunchKernelGGL(top_logprobs_kernel, dim3(rows), dim3(ST), 0, stream, logits, inv_t, out_tok, out_lp, vocab, k);
+    return check_launch("top_logprobs");
+}
 
 // part_val / part_idx: float / int workspaces [rows, ms_sample_chunks()] for the two-stage greedy
 // search, or null (every row scans itself in one block).

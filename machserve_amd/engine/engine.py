@@ -57,7 +57,7 @@ class Engine:
         self.steps += 1
         self.tokens_run += plan.n_tokens
         reqs = [it.request for it in sampled_items]
-        if len(sampled_items) == len(plan.items) and not any(r.params.edits_logits() for r in reqs):
+        if len(sampled_items) == len(plan.items) and all(r.params.plain() for r in reqs):
             # every request decodes one token: forward pass and sampling are one captured graph
             fast = self.loaded.step.decode_and_sample(
                 entries, [r.params.temperature for r in reqs], [r.params.top_k for r in reqs],
@@ -68,8 +68,11 @@ class Engine:
         logits = self.loaded.step(entries, borrow_logits=True)
         if not sampled_items:
             return self.scheduler.update(plan, [])
-        tokens, logprobs, states = self.sampler.sample(logits, [r.params for r in reqs], [r.rng_state for r in reqs],
-                                                       [r.generated for r in reqs])
+        tokens, logprobs, states, top = self.sampler.sample(logits, [r.params for r in reqs], [r.rng_state for r in reqs],
+                                                            [r.generated for r in reqs])
+        for r, t in zip(reqs, top):
+            if r.params.top_logprobs:
+                r.top_logprobs.append(t)
         return self.scheduler.update(plan, tokens, logprobs, states)
 
     def run(self) -> Dict[int, Request]:

@@ -45,6 +45,7 @@ class Request:
     slot: Optional[int] = None
     rng_state: int = 0
     logprobs: List[float] = field(default_factory=list)
+    top_logprobs: List[list] = field(default_factory=list)  # per generated token: [(token, logprob), ...]
     finish_reason: Optional[str] = None
     preemptions: int = 0
 

@@ -338,6 +338,19 @@ class HipOps:
                                                      _c_int(V), _stream()))
         return both
 
+    def top_logprobs(self, logits: torch.Tensor, inv_t: torch.Tensor, k: int):
+        """The ``k`` most probable tokens of every row and their log-probabilities at the row's
+        temperature (``inv_t``), ties to the smaller id.  Returns ``(tokens [W, k], logprobs [W, k])``."""
+        W, V = logits.shape
+        self._want(logits, torch.float32, "top_logprobs logits")
+        self._want(inv_t, torch.float32, "top_logprobs inv_t", W)
+        width = self._core.ms_top_logprobs_max()
+        tok = torch.empty((W, width), dtype=torch.int32, device=logits.device)
+        lp = torch.empty((W, width), dtype=torch.float32, device=logits.device)
+        self._check(self._core, self._core.ms_top_logprobs(_ptr(logits), _ptr(inv_t), _ptr(tok), _ptr(lp), _c_int(W),
+                                                           _c_int(V), _c_int(k), _stream()))
+        return tok[:, :k], lp[:, :k]
+
     def logit_edit(self, logits: torch.Tensor, row_of: torch.Tensor, token: torch.Tensor, delta: torch.Tensor) -> None:
         """``logits[row_of[e], token[e]] += delta[e]`` (penalties and biases merged on the host)."""
         n = row_of.numel()

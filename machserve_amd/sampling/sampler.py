@@ -26,7 +26,8 @@ class Sampler:
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], states: Sequence[int],
                generated: Sequence[Sequence[int]]):
         """``logits [W, vocab]`` float32 (edited in place when a row has penalties or biases).
-        Returns ``(tokens, logprobs, new_states)`` as host lists."""
+        Returns ``(tokens, logprobs, new_states, top)`` as host lists; ``top[r]`` is the list of
+        (token, logprob) of the row's ``top_logprobs`` most probable tokens (empty if 0)."""
         W = logits.shape[0]
         rows, toks, deltas = [], [], []
         for r, p in enumerate(params):
@@ -54,5 +55,13 @@ class Sampler:
         kdev = torch.tensor([p.top_k for p in params], dtype=torch.int32, device=self.device)
         sdev = torch.tensor([_signed(s) for s in states], dtype=torch.int64, device=self.device)
         tok, lp = self.ops.sample(logits, fdev[0], kdev, fdev[1], sdev, any(p.temperature <= 0.0 for p in params))
-        tokens = tok.cpu().tolist()  # the step's one synchronisation
-        return tokens, lp.cpu().tolist(), [advance(s) for s in states]
+        top = [[] for _ in params]
+        kmax = max(p.top_logprobs for p in params)
+        if kmax > 0:
+            inv_t = torch.tensor([1.0 / p.temperature if p.temperature > 0.0 else 1.0 for p in params],
+                                 dtype=torch.float32, device=self.device)
+            ttok, tlp = self.ops.top_logprobs(logits, inv_t, kmax)
+            ttok, tlp = ttok.cpu().tolist(), tlp.cpu().tolist()
+            top = [list(zip(ttok[r][:p.top_logprobs], tlp[r][:p.top_logprobs])) for r, p in enumerate(params)]
+        tokens = tok.cpu().tolist()  # the step's synchronisation
+        return tokens, lp.cpu().tolist(), [advance(s) for s in states], top

@@ -147,6 +147,11 @@ class EmulatedOps:
             lps.append(0.0)
         return torch.tensor(toks, dtype=torch.int32), torch.tensor(lps)
 
+    def top_logprobs(self, logits, inv_t, k):
+        lp = torch.log_softmax(logits.double() * inv_t.double()[:, None], -1)
+        order = torch.argsort(-logits.double(), dim=-1, stable=True)[:, :k]
+        return order.to(torch.int32), torch.gather(lp, 1, order).float()
+
     def logit_edit(self, logits, row_of, token, delta):
         for r, t, d in zip(row_of.tolist(), token.tolist(), delta.tolist()):
             logits[r, t] += d

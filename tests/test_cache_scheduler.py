@@ -266,3 +266,31 @@ def test_engine_sampling_is_deterministic_and_survives_preemption(tmp_path):
         tok, st = P.sample(P.forward(w, sizes, seq)[-1].numpy(), 1.0, 50, 1.0, st)
         assert tok == t
         seq.append(tok)
+
+
+def test_engine_reports_logprobs_and_top_logprobs(tmp_path):
+    """Options that need the logits after the draw: the engine leaves its captured-graph path."""
+    from machserve_amd.engine import Engine, load_model
+    from machserve_amd.sampling import SamplingParams
+    d = make_model_dir(tmp_path, "A")
+    w, sizes = read_for_plain(d)
+    lm = load_model(d, dtype="float32", device="cpu", page_size=16, num_pages=8, max_requests=2, ops=EmulatedOps())
+    eng = Engine(lm)
+    p = random_prompt(9, 512, 5)
+    rid = eng.add(p, 4, SamplingParams(top_logprobs=3, presence_penalty=0.5, logit_bias={7: 1.0}))
+    r = eng.run()[rid]
+    assert len(r.generated) == 4 and len(r.top_logprobs) == 4 and all(len(t) == 3 for t in r.top_logprobs)
+    seq, counts = list(p), {}
+    for step, tok in enumerate(r.generated):
+        logits = P.forward(w, sizes, seq)[-1].clone()
+        for t, c in counts.items():
+            logits[t] -= 0.5
+        logits[7] += 1.0
+        lp = torch.log_softmax(logits.double(), -1)
+        best = torch.argsort(-logits.double(), stable=True)[:3].tolist()
+        assert [t for t, _ in r.top_logprobs[step]] == best and tok == best[0]
+        assert abs(r.top_logprobs[step][0][1] - lp[best[0]].item()) < 1e-4
+        counts[tok] = counts.get(tok, 0) + 1
+        seq.append(tok)
+    with pytest.raises(ValueError, match="top_logprobs"):
+        eng.add(p, 1, SamplingParams(top_logprobs=21))

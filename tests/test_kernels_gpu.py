@@ -377,6 +377,28 @@ def test_sampler_greedy_ties_and_spread():
     assert len(set(tok.cpu().tolist())) > 40
 
 
+def test_top_logprobs():
+    """Ranked by probability, ties to the smaller id, logprob = log softmax at the row's temperature
+    (crates/mach-model/src/sampling.rs:405-410)."""
+    ops = ops_for(torch.float32)
+    V = 5000
+    logits = torch.randn(4, V, generator=torch.Generator().manual_seed(3)) * 3
+    logits[1, [10, 4000, 77]] = 20.0     # a three-way tie at the top: ids ascending
+    logits[2] = 0.0                      # all equal: the first ids
+    inv_t = torch.tensor([1.0, 0.5, 2.0, 1.25])
+    tok, lp = ops.top_logprobs(logits.to(DEV), inv_t.to(DEV), 20)
+    tok, lp = tok.cpu(), lp.cpu()
+    assert tok.shape == (4, 20)
+    assert tok[1, :3].tolist() == [10, 77, 4000] and tok[2].tolist() == list(range(20))
+    ref = torch.log_softmax(logits.double() * inv_t.double()[:, None], -1)
+    for r in range(4):
+        order = sorted(range(V), key=lambda i: (-logits[r, i].item(), i))[:20]
+        assert tok[r].tolist() == order
+        assert (lp[r].double() - ref[r, order]).abs().max() < 1e-4
+    tok3, _ = ops.top_logprobs(logits.to(DEV), inv_t.to(DEV), 3)
+    assert tok3.shape == (4, 3) and torch.equal(tok3.cpu(), tok[:, :3])
+
+
 def test_logit_edit():
     ops = ops_for(torch.float32)
     x = torch.zeros(2, 10, device=DEV)
