@@ -67,6 +67,14 @@ __device__ __forceinline__ float exp_f(float x) {
 #endif
 }
 
+__device__ __forceinline__ float exp2_f(float x) {
+#ifdef MS_ELEM_BF16
+    return __builtin_amdgcn_exp2f(x);
+#else
+    return exp2f(x);
+#endif
+}
+
 __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
     __shared__ __attribute__((aligned(16))) elem_t Ks[BKV * K_LD];
     __shared__ __attribute__((aligned(16))) elem_t Vs[HDT * V_LD];
@@ -109,38 +117,54 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
     f32x4 acc_o[ND];
 #pragma unroll
     for (int i = 0; i < ND; ++i) acc_o[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    // running maximum in units of the raw score; exponentials are taken in base 2 with the scale
+    // folded in: exp(scale * (s - m)) = exp2(s * sl - m * sl)
     float m_run = NEG_BIG, l_run = 0.f;
+    const float sl = a.scale * 1.4426950408889634f;
 
     // Tiles go global -> registers -> LDS.  PF tiles are in flight at any time: a tile's loads are
     // requested PF tiles before it is multiplied, which covers the memory latency even when few
-    // blocks share a CU.
+    // blocks share a CU.  Where a tile's 16-key groups lie in the pools is looked up once per tile
+    // by NT threads and shared through LDS (offsets in units of 16 elements).
     constexpr int CPRK = HDT / EPC, CPRV = BKV / EPC;
     constexpr int NCK = (BKV * CPRK + 255) / 256, NCV = (HDT * CPRV + 255) / 256;
     constexpr int PF = ND <= 4 ? 4 : (ND <= 8 ? 2 : 1);
+    constexpr unsigned ABSENT = 0xffffffffu;
+    __shared__ unsigned kofs[PF][NT], vofs[PF][NT];
     u32x4 rk[PF][NCK], rv[PF][NCV];
-    auto load_tile = [&](int kt0, u32x4* pk, u32x4* pv) {
+    auto fill_offsets = [&](int kt0, int slot) {  // threads tid < NT
+        const int key0 = kt0 + tid * 16;
+        unsigned ko = ABSENT, vo = ABSENT;
+        if (key0 < kv_hi) {
+            const int page = table[key0 / ps], off = key0 % ps;
+            if (page >= 0) {
+                const size_t pk = (size_t)page * a.KV + kvh;
+                ko = (unsigned)(((pk * ps + off) * hd) >> 4);
+                vo = (unsigned)((pk * hd * ps + off) >> 4);
+            }
+        }
+        kofs[slot][tid] = ko;
+        vofs[slot][tid] = vo;
+    };
+    auto load_tile = [&](int slot, u32x4* pk, u32x4* pv) {
 #pragma unroll
         for (int i = 0; i < NCK; ++i) {
             const int c = tid + i * 256;
-            const int kl = c / CPRK, d0 = (c % CPRK) * EPC, key = kt0 + kl;
+            const int kl = c / CPRK, d0 = (c % CPRK) * EPC;
+            const unsigned o = kofs[slot][(kl / 16) % NT];
             u32x4 v = {0, 0, 0, 0};
-            if (c < BKV * CPRK && key < kv_hi && d0 < hd) {
-                const int page = table[key / ps];
-                if (page >= 0)
-                    v = *reinterpret_cast<const u32x4*>(a.kpool + (((size_t)page * a.KV + kvh) * ps + key % ps) * hd + d0);
-            }
+            if (c < BKV * CPRK && o != ABSENT && d0 < hd)
+                v = *reinterpret_cast<const u32x4*>(a.kpool + ((size_t)o << 4) + (kl % 16) * hd + d0);
             pk[i] = v;
         }
 #pragma unroll
         for (int i = 0; i < NCV; ++i) {
             const int c = tid + i * 256;
-            const int d = c / CPRV, k0 = (c % CPRV) * EPC, key = kt0 + k0;
+            const int d = c / CPRV, k0 = (c % CPRV) * EPC;
+            const unsigned o = vofs[slot][(k0 / 16) % NT];
             u32x4 v = {0, 0, 0, 0};
-            if (c < HDT * CPRV && key < kv_hi && d < hd) {
-                const int page = table[key / ps];
-                if (page >= 0)
-                    v = *reinterpret_cast<const u32x4*>(a.vpool + (((size_t)page * a.KV + kvh) * hd + d) * ps + key % ps);
-            }
+            if (c < HDT * CPRV && o != ABSENT && d < hd)
+                v = *reinterpret_cast<const u32x4*>(a.vpool + ((size_t)o << 4) + (size_t)d * ps + (k0 % 16));
             pv[i] = v;
         }
     };
@@ -156,10 +180,20 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
             if (c < HDT * CPRV) *reinterpret_cast<u32x4*>(&Vs[(c / CPRV) * V_LD + (c % CPRV) * EPC]) = pv[i];
         }
     };
+    // rows of this wave: the first and the last position decide which tiles need no mask at all
+    const int pos_first = pos0 + (r0 + wave * 16) / g;
+    const int pos_last = pos0 + min(r0 + wave * 16 + 15, max(R - 1, 0)) / g;
+    const int lo_last = a.window > 0 ? pos_last - a.window + 1 : 0;
+
     const int kt_first = (kv_lo / BKV) * BKV;
+    if (tid < NT) {
+#pragma unroll
+        for (int j = 0; j < PF; ++j) fill_offsets(kt_first + j * BKV, j);
+    }
+    __syncthreads();
 #pragma unroll
     for (int j = 0; j < PF; ++j)
-        if (kt_first + j * BKV < kv_hi) load_tile(kt_first + j * BKV, rk[j], rv[j]);
+        if (kt_first + j * BKV < kv_hi) load_tile(j, rk[j], rv[j]);
     for (int kt_base = kt_first; kt_base < kv_hi; kt_base += PF * BKV) {
 #pragma unroll
       for (int j = 0; j < PF; ++j) {
@@ -167,8 +201,9 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
         if (kt0 >= kv_hi) break;
         __syncthreads();  // the previous tile has been consumed
         store_tile(rk[j], rv[j]);
+        if (tid < NT) fill_offsets(kt0 + PF * BKV, j);
         __syncthreads();
-        if (kt0 + PF * BKV < kv_hi) load_tile(kt0 + PF * BKV, rk[j], rv[j]);
+        if (kt0 + PF * BKV < kv_hi) load_tile(j, rk[j], rv[j]);
         if (!wave_active) continue;
 
         // S^T = K Q^T: lane holds keys grp * 4 + i of tile nt for query row r16
@@ -183,27 +218,37 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
                 mma_16x16x32(sc[nt], kf, qf[ks]);
             }
         }
+        // a tile that every row of the wave sees whole needs no mask
+        const bool whole = kt0 + BKV - 1 <= pos_first && kt0 >= lo_last;
         float tmax = NEG_BIG;
+        if (whole) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
+            for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = kt0 + nt * 16 + grp * 4 + i;
-                const bool ok = valid && key <= pos && key >= lo_key;
-                const float v = ok ? sc[nt][i] * a.scale : -INFINITY;
-                sc[nt][i] = v;
-                tmax = fmaxf(tmax, v);
-            }
+                for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, sc[nt][i]);
+        } else {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = kt0 + nt * 16 + grp * 4 + i;
+                    const bool ok = valid && key <= pos && key >= lo_key;
+                    const float v = ok ? sc[nt][i] : -INFINITY;
+                    sc[nt][i] = v;
+                    tmax = fmaxf(tmax, v);
+                }
+        }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
         const float m_new = fmaxf(m_run, tmax);
-        const float alpha = exp_f(m_run - m_new);
+        const float alpha = exp2_f((m_run - m_new) * sl);
+        const float mb = m_new * sl;
         float psum = 0.f;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float p = exp_f(sc[nt][i] - m_new);
+                const float p = exp2_f(fmaf(sc[nt][i], sl, -mb));
                 sc[nt][i] = p;
                 psum += p;
             }
@@ -223,7 +268,7 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 pf.v[i] = from_f32<elem_t>(sc[2 * pp][i]);
-                pf.v[4 + i] = (2 * pp + 1 < NT) ? from_f32<elem_t>(sc[(2 * pp + 1 < NT) ? 2 * pp + 1 : 0][i]) : from_f32<elem_t>(0.f);
+                pf.v[4 + i] = from_f32<elem_t>((2 * pp + 1 < NT) ? sc[(2 * pp + 1) % NT][i] : 0.f);
             }
 #pragma unroll
             for (int dt = 0; dt < ND; ++dt) {
@@ -607,12 +652,13 @@ using namespace ms;
 extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
     const void* q, const void* kpool, const void* vpool, void* out, const int* block_table, int table_stride,
     const int* seq_q_start, const int* seq_q_len, const int* seq_pos0, const int* work, int n_work, int H, int KV,
-    int hd, int ps, int window, float scale, hipStream_t stream) {
+    int hd, int ps, int n_pages, int window, float scale, hipStream_t stream) {
     MS_REQUIRE(n_work > 0, "attention: no work");
     MS_REQUIRE(hd % 16 == 0 && hd > 0 && hd <= HDT, "attention: head size %d does not fit this tile of %d", hd, HDT);
     MS_REQUIRE(KV > 0 && H % KV == 0, "attention: %d heads are not a multiple of %d key/value heads", H, KV);
     MS_REQUIRE(ps % 16 == 0 && ps > 0, "attention: page size %d must be a multiple of 16", ps);
     MS_REQUIRE(window >= 0, "attention: window %d", window);
+    MS_REQUIRE((double)n_pages * KV * ps * hd < 68719476736.0, "attention: a pool of %d pages exceeds 2^36 elements", n_pages);
     AttnArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, (elem_t*)out, block_table, seq_q_start,
                seq_q_len, seq_pos0, work, table_stride, H, KV, hd, ps, window, scale};
     hipLaunchKernelGGL(paged_attention_kernel, dim3((unsigned)n_work, (unsigned)KV), dim3(256), 0, stream, a);

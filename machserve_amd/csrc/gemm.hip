@@ -13,16 +13,13 @@
 
 namespace ms {
 
-constexpr int BK = 32;
 #ifdef MS_ELEM_BF16
 constexpr int EPC = 8;   // elements per 16-byte chunk
-constexpr int KPAD = 8;  // row padding in elements: 80-byte rows
+constexpr int KPAD = 8;  // row padding in elements: rows of 80 (BK 32) or 144 (BK 64) bytes
 #else
 constexpr int EPC = 4;
-constexpr int KPAD = 4;  // 144-byte rows
+constexpr int KPAD = 4;  // rows of 144 bytes (BK 32)
 #endif
-constexpr int LDS_LD = BK + KPAD;
-constexpr int CPR = BK / EPC;  // chunks per tile row
 
 enum EpiKind { EPI_STORE_F32 = 0, EPI_STORE_ELEM = 1, EPI_RESIDUAL = 2, EPI_SWIGLU = 3 };
 
@@ -43,10 +40,13 @@ __device__ __forceinline__ float silu_f(float g) {
 #endif
 }
 
-template <int BM, int BN, int WM, int WN, int EPI>
+template <int BM, int BN, int WM, int WN, int BK, int EPI>
 __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A, const elem_t* __restrict__ W,
                                                    int M, int N, int K, EpiArgs ep) {
     static_assert(WM * WN == 4, "four waves");
+    static_assert(BK % 32 == 0, "K step in MFMA steps of 32");
+    constexpr int LDS_LD = BK + KPAD;
+    constexpr int CPR = BK / EPC;  // chunks per tile row
     constexpr int TM = BM / WM / 16, TN = BN / WN / 16;
     constexpr int A_CHUNKS = BM * CPR / 256, W_CHUNKS = BN * CPR / 256;
     static_assert(BM * CPR % 256 == 0 && BN * CPR % 256 == 0, "tile loads divide over the block");
@@ -105,15 +105,18 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
     for (int kt = 0; kt < nk; ++kt) {
         const int buf = kt & 1;
         if (kt + 1 < nk) load_global(k_begin + (kt + 1) * BK);
-        Frag fa[TM], fb[TN];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fa[i] = frag_load(&As[buf][(wm * (BM / WM) + i * 16 + r16) * LDS_LD + grp * 8]);
+        for (int kk = 0; kk < BK; kk += 32) {
+            Frag fa[TM], fb[TN];
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fb[j] = frag_load(&Ws[buf][(wn * (BN / WN) + j * 16 + r16) * LDS_LD + grp * 8]);
+            for (int i = 0; i < TM; ++i) fa[i] = frag_load(&As[buf][(wm * (BM / WM) + i * 16 + r16) * LDS_LD + kk + grp * 8]);
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+            for (int j = 0; j < TN; ++j) fb[j] = frag_load(&Ws[buf][(wn * (BN / WN) + j * 16 + r16) * LDS_LD + kk + grp * 8]);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) mma_16x16x32(acc[i][j], fa[i], fb[j]);
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) mma_16x16x32(acc[i][j], fa[i], fb[j]);
+        }
         if (kt + 1 < nk) store_lds(buf ^ 1);
         __syncthreads();
     }
@@ -158,6 +161,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
     }
 }
 
+static int g_gemm_config = 0;  // 0: chosen by shape; else a fixed tile (measurements only)
+
 template <int EPI>
 static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, EpiArgs ep, hipStream_t stream,
                        int nsplit = 1) {
@@ -166,26 +171,40 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
     MS_REQUIRE((reinterpret_cast<uintptr_t>(A) & 15) == 0 && (reinterpret_cast<uintptr_t>(W) & 15) == 0,
                "gemm: operands must be 16-byte aligned");
     MS_REQUIRE(nsplit >= 1 && (nsplit == 1 || EPI == EPI_STORE_F32), "gemm: %d K slices need the float store", nsplit);
-    ep.k_per_split = ceil_div(ceil_div(K, nsplit), BK) * BK;
+    // slices of a multiple of 64; rounding up may leave fewer slices than asked for
+    ep.k_per_split = ceil_div(ceil_div(K, nsplit), 64) * 64;
     ep.split_stride = (size_t)M * N;
     const unsigned ns = (unsigned)ceil_div(K, ep.k_per_split);
+    MS_REQUIRE(nsplit == 1 || (int)ns == nsplit, "gemm: %d K slices asked for, %u fit", nsplit, ns);
+#define MS_GEMM(BM_, BN_, WM_, WN_, BK_)                                                                              \
+    do {                                                                                                              \
+        const long nb = (long)ceil_div(M, BM_) * ceil_div(N, BN_);                                                    \
+        hipLaunchKernelGGL((gemm_kernel<BM_, BN_, WM_, WN_, BK_, EPI>), dim3((unsigned)nb, ns), dim3(256), 0, stream, \
+                           A, W, M, N, K, ep);                                                                        \
+        return check_launch("gemm " #BM_ "x" #BN_ "x" #BK_);                                                          \
+    } while (0)
 #ifdef MS_ELEM_BF16
-    // the largest tile that still gives every CU of the chip a block or two
+    const int forced = g_gemm_config;
+    if (forced == 1) MS_GEMM(128, 128, 2, 2, 32);
+    if (forced == 2) MS_GEMM(128, 128, 2, 2, 64);
+    if (forced == 5) MS_GEMM(128, 64, 2, 2, 64);
+    if (forced == 6) MS_GEMM(64, 64, 2, 2, 64);
+    // The largest tile that still gives every CU of the chip a block or two; a K step of 64 (half
+    // the barriers) where the K loop is long enough to pay for the larger tiles in LDS.  Measured
+    // on M = 512..8192 of the 0.5B shapes; larger wave tiles (256x128) lose to register pressure.
     if (M > 64) {
         const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128), b12864 = (long)ceil_div(M, 128) * ceil_div(N, 64);
         if (b128 * ns >= 300) {
-            hipLaunchKernelGGL((gemm_kernel<128, 128, 2, 2, EPI>), dim3((unsigned)b128, ns), dim3(256), 0, stream, A, W, M, N, K, ep);
-            return check_launch("gemm 128x128");
+            if (ep.k_per_split >= 1024) MS_GEMM(128, 128, 2, 2, 64);
+            MS_GEMM(128, 128, 2, 2, 32);
         }
-        if (b12864 * ns >= 300) {
-            hipLaunchKernelGGL((gemm_kernel<128, 64, 2, 2, EPI>), dim3((unsigned)b12864, ns), dim3(256), 0, stream, A, W, M, N, K, ep);
-            return check_launch("gemm 128x64");
-        }
+        if (b12864 * ns >= 300) MS_GEMM(128, 64, 2, 2, 32);
     }
+    MS_GEMM(64, 64, 2, 2, 64);
+#else
+    MS_GEMM(64, 64, 2, 2, 32);
 #endif
-    const long blocks = (long)ceil_div(M, 64) * ceil_div(N, 64);
-    hipLaunchKernelGGL((gemm_kernel<64, 64, 2, 2, EPI>), dim3((unsigned)blocks, ns), dim3(256), 0, stream, A, W, M, N, K, ep);
-    return check_launch("gemm 64x64");
+#undef MS_GEMM
 }
 
 // K slices for a product of many rows whose consumer adds partial sums: enough 128x128 blocks to
@@ -194,8 +213,10 @@ static int plan_tiled_splits(int M, int N, int K) {
 #ifdef MS_ELEM_BF16
     const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
     if (b128 >= 300) return 1;
-    int want = (int)ceil_div(300, b128);
-    return max(1, min(want, K / 512));
+    int want = max(1, min((int)ceil_div(300, b128), K / 512));
+    // what the launcher's rounding of a slice to a multiple of 64 really yields
+    const int k_per_split = ceil_div(ceil_div(K, want), 64) * 64;
+    return ceil_div(K, k_per_split);
 #else
     (void)M; (void)N; (void)K;
     return 1;
@@ -237,3 +258,6 @@ extern "C" int ms_linear_split_tiled(const void* a, const void* w, float* out, i
     EpiArgs ep{out, nullptr, N, N, 0, 0};
     return launch_gemm<EPI_STORE_F32>((const elem_t*)a, (const elem_t*)w, M, N, K, ep, stream, plan_tiled_splits(M, N, K));
 }
+
+// Measurements only: force one tile configuration (0 = choose by shape).
+extern "C" void ms_gemm_force_config(int c) { g_gemm_config = c; }

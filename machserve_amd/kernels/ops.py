@@ -228,8 +228,8 @@ class HipOps:
         out = torch.empty((T, H * hd), dtype=self.dtype, device=q.device)
         self._check(lib, fn(_ptr(q), _ptr(kpool), _ptr(vpool), _ptr(out), _ptr(block_table), _c_int(block_table.shape[1]),
                             _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_pos0), _ptr(work), _c_int(work.shape[0]),
-                            _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), _c_int(window or 0), _c_float(scale),
-                            _stream()))
+                            _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), _c_int(pages), _c_int(window or 0),
+                            _c_float(scale), _stream()))
         return out
 
     DECODE_MAX_GROUP = 16  # query heads per key/value head the decode kernel takes

@@ -79,7 +79,8 @@ def test_linear(dtype, M, N, K):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,N,K", [(65, 896, 4864), (300, 130, 1096), (2048, 896, 4864), (200, 200, 520)])
+@pytest.mark.parametrize("M,N,K", [(65, 896, 4864), (300, 130, 1096), (2048, 896, 4864), (200, 200, 520), (100, 1536, 8960),
+                                   (100, 1536, 1536), (130, 136, 264)])
 def test_linear_many_rows_cut_along_k(dtype, M, N, K):
     """A product with too few tiles to fill the chip is cut along K into ordered partial sums."""
     ops = ops_for(dtype)
