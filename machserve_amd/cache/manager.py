@@ -15,14 +15,16 @@ handed out again.  A request also holds one *state slot*: an index into arrays
 Layout of a page: keys ``[kv_heads, page_size, head_dim]``, values transposed
 ``[kv_heads, head_dim, page_size]``.
 
-This module is host logic only; device tensors are made by ``allocate_device``.
+Host logic only.  The bookkeeping itself (pools, tables, windows, the step's address buffer) is
+the native ``CacheCore`` of ``csrc/host/host.cpp``; this class sorts the layers' requests into
+groups, names them, and hands device tensors to the layers (``DeviceCache``).
 """
 from __future__ import annotations
 
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Tuple
 
-from .pool import BlockPool, CacheError, OutOfPages, SlotPool
+from .pool import CacheCore, CacheError, OutOfPages
 
 
 def group_name(window: Optional[int]) -> str:
@@ -52,13 +54,38 @@ class StateBinding:
     tensors: Dict[str, object]
 
 
+class _PoolView:
+    """Counts of one group's page pool."""
+
+    def __init__(self, core: CacheCore, index: int):
+        self._core, self._index = core, index
+
+    @property
+    def num_pages(self) -> int:
+        return self._core.group_pages(self._index)
+
+    def available(self) -> int:
+        return self._core.group_available(self._index)
+
+    def live_pages(self) -> List[int]:
+        return self._core.group_live_pages(self._index)
+
+
 class _Group:
-    def __init__(self, spec: GroupSpec, page_size: int, num_pages: int):
-        self.spec = spec
-        self.page_size = page_size
-        self.pool = BlockPool(num_pages)
-        self.tables: Dict[int, List[int]] = {}
-        self.first_live: Dict[int, int] = {}  # first logical page not yet given back
+    def __init__(self, spec: GroupSpec, core: CacheCore, index: int):
+        self.spec, self.index = spec, index
+        self.pool = _PoolView(core, index)
+
+
+class _SlotsView:
+    def __init__(self, core: CacheCore):
+        self._core = core
+
+    def available(self) -> int:
+        return self._core.slots_available()
+
+    def is_live(self, slot: int) -> bool:
+        return self._core.slot_is_live(slot)
 
 
 class CacheManager:
@@ -66,14 +93,10 @@ class CacheManager:
         """``layer_requests[p]`` is the cache request of the p-th layer run of a step (see
         ``parts.base`` and ``DecoderModel.cache_requests``); "layer" below means such a run."""
         from ..parts.base import PagedKVRequest, SharedKVRequest, StateRequest
-        if page_size < 16 or page_size % 16:
-            raise CacheError(f"page size {page_size} must be a positive multiple of 16")
-        if max_requests < 1:
-            raise CacheError("at least one request slot is needed")
+        self.core = CacheCore(page_size, max_requests)
         self.page_size = page_size
         self.max_requests = max_requests
-        self.slots = SlotPool(max_requests)
-        self.lengths: Dict[int, int] = {}
+        self.slots = _SlotsView(self.core)
         self.groups: Dict[str, _Group] = {}
         self.layer_group: Dict[int, str] = {}
         self.layer_source: Dict[int, int] = {}
@@ -102,94 +125,55 @@ class CacheManager:
                 raise CacheError(f"layer {i} reads the cache of layer {src}, which keeps none")
             self.layer_group[i] = self.layer_group[src]
         for name, spec in specs.items():
-            self.groups[name] = _Group(spec, page_size, num_pages)
-        self.device = None  # filled by allocate_device
+            index = self.core.add_group(name, spec.window or 0, num_pages)
+            self.groups[name] = _Group(spec, self.core, index)
+        self._names = list(self.groups)
+        self.device = None  # filled by DeviceCache
 
     # ------------------------------------------------------------------ requests
     def admit(self) -> int:
         """A state slot for a new request; its block tables start empty and its state zero."""
-        slot = self.slots.alloc()
-        if slot is None:
-            raise CacheError(f"all {self.max_requests} request slots are in use")
-        self.lengths[slot] = 0
-        for g in self.groups.values():
-            g.tables[slot] = []
-            g.first_live[slot] = 0
+        slot = self.core.admit()
         if self.device is not None:
             self.device.zero_state(slot)
         return slot
 
     def length(self, slot: int) -> int:
-        return self.lengths[slot]
+        return self.core.length(slot)
+
+    @property
+    def lengths(self) -> Dict[int, int]:
+        return self.core.lengths()
 
     def pages_needed(self, slot: int, n_new: int) -> Dict[str, int]:
         """Pages each group must add before ``n_new`` more tokens of ``slot`` can be written."""
-        end = self.lengths[slot] + n_new
-        need = {}
-        for name, g in self.groups.items():
-            have = len(g.tables[slot])
-            need[name] = max(0, -(-end // self.page_size) - have)
-        return need
+        return dict(zip(self._names, self.core.pages_needed(slot, n_new)))
 
     def can_extend(self, slot: int, n_new: int, reserved: Optional[Dict[str, int]] = None) -> bool:
-        need = self.pages_needed(slot, n_new)
-        return all(self.groups[n].pool.available() - (reserved or {}).get(n, 0) >= k for n, k in need.items())
+        return self.core.can_extend(slot, n_new, [(reserved or {}).get(n, 0) for n in self._names])
 
     def extend(self, slot: int, n_new: int) -> None:
-        """Take the pages for the next ``n_new`` tokens of ``slot`` in every group, or none at all."""
-        if not self.slots.is_live(slot):
-            raise CacheError(f"slot {slot} is not in use")
-        need = self.pages_needed(slot, n_new)
-        for name, k in need.items():
-            if self.groups[name].pool.available() < k:
-                raise OutOfPages(f"group {name}: {k} pages needed for {n_new} tokens of slot {slot}, "
-                                 f"{self.groups[name].pool.available()} free")
-        for name, k in need.items():
-            g = self.groups[name]
-            for _ in range(k):
-                g.tables[slot].append(g.pool.alloc())
+        """Take the pages for the next ``n_new`` tokens of ``slot`` in every group, or none at all
+        (``OutOfPages``)."""
+        self.core.extend(slot, n_new)
 
     def commit(self, slot: int, n_new: int) -> None:
         """The step wrote ``n_new`` tokens: advance the length and give back the pages that no
         later row's window reaches."""
-        self.lengths[slot] += n_new
-        L = self.lengths[slot]
-        for g in self.groups.values():
-            W = g.spec.window
-            if W is None:
-                continue
-            # the next row is at position L and sees keys > L - W
-            dead = max(0, L - W + 1) // self.page_size
-            table = g.tables[slot]
-            for p in range(g.first_live[slot], min(dead, len(table))):
-                if table[p] >= 0:
-                    g.pool.free(table[p])
-                    table[p] = -1
-            g.first_live[slot] = max(g.first_live[slot], min(dead, len(table)))
+        self.core.commit(slot, n_new)
 
     def release(self, slot: int) -> None:
         """The request ended (or is preempted): all its pages and its slot go back."""
-        if not self.slots.is_live(slot):
-            raise CacheError(f"slot {slot} released twice or never admitted")
-        for g in self.groups.values():
-            for p in g.tables.pop(slot):
-                if p >= 0:
-                    g.pool.free(p)
-            g.first_live.pop(slot)
-        del self.lengths[slot]
-        self.slots.free(slot)
+        self.core.release(slot)
 
     # ------------------------------------------------------------------ addresses
     def table(self, group: str, slot: int) -> List[int]:
-        return self.groups[group].tables[slot]
+        return self.core.table(self.groups[group].index, slot)
 
     def slot_of_position(self, group: str, slot: int, pos: int) -> int:
         """``page * page_size + offset`` of position ``pos``
         (``crates/mach-model/src/paged_kv.rs:68`` page_offsets)."""
-        page = self.groups[group].tables[slot][pos // self.page_size]
-        if page < 0:
-            raise CacheError(f"group {group}: position {pos} of slot {slot} lies in a page already given back")
-        return page * self.page_size + pos % self.page_size
+        return self.core.slot_of_position(self.groups[group].index, slot, pos)
 
     def free_pages(self, group: Optional[str] = None) -> int:
         if group is not None:
@@ -197,22 +181,14 @@ class CacheManager:
         return min(g.pool.available() for g in self.groups.values()) if self.groups else 0
 
     def live_requests(self) -> List[int]:
-        return sorted(self.lengths)
+        return self.core.live_requests()
 
     def check(self) -> None:
         """Invariants: a page is owned by at most one table entry, and every live page of a pool
         is owned.  Raises CacheError otherwise."""
-        for name, g in self.groups.items():
-            owned: Dict[int, Tuple[int, int]] = {}
-            for slot, table in g.tables.items():
-                for i, p in enumerate(table):
-                    if p < 0:
-                        continue
-                    if p in owned:
-                        raise CacheError(f"group {name}: page {p} held by slot {owned[p][0]} and slot {slot}")
-                    owned[p] = (slot, i)
-            live = set(g.pool.live_pages())
-            if live != set(owned):
-                raise CacheError(f"group {name}: live pages {sorted(live)} differ from owned pages {sorted(owned)}")
-            if len(live) + g.pool.available() != g.pool.num_pages:
-                raise CacheError(f"group {name}: {len(live)} live + {g.pool.available()} free != {g.pool.num_pages}")
+        self.core.check()
+
+    def build_step(self, slots, counts, tokens, want_rows, heads_per_kv, rows_per_block: int, table_multiple: int = 1):
+        """The step's int32 buffer as ``(numpy array, {section: (start, size)}, {group: table width})``;
+        see ``CacheCore::build_step`` for the sections."""
+        return self.core.build_step(slots, counts, tokens, want_rows, list(heads_per_kv), rows_per_block, table_multiple)

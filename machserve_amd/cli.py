@@ -12,6 +12,7 @@ top_p, seed, presence_penalty, frequency_penalty, max_new, eos, stop.
 
     python -m machserve_amd --model DIR --prompt-ids 1,2,3 --max-new 16
     python -m machserve_amd --random-config config.json --seed 0 --prompt-file prompts.txt
+    python -m machserve_amd random-weights --config config.json --seed 0 --out DIR [--dtype f32|bf16]
     python -m machserve_amd doctor
 """
 from __future__ import annotations
@@ -57,10 +58,29 @@ def doctor() -> int:
     return 0
 
 
+def random_weights(argv) -> int:
+    """Write a model folder (config.json, model.safetensors) with random weights."""
+    import torch
+    from .weights import write_random_model
+    ap = argparse.ArgumentParser(prog="machserve_amd random-weights", description=random_weights.__doc__)
+    ap.add_argument("--config", required=True, help="config.json of the architecture")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--out", required=True, help="folder to write")
+    ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"], help="dtype the tensors are stored in")
+    args = ap.parse_args(argv)
+    with open(args.config) as f:
+        raw = json.load(f)
+    out = write_random_model(raw, args.seed, args.out, torch.float32 if args.dtype == "f32" else torch.bfloat16)
+    print(out)
+    return 0
+
+
 def main(argv=None) -> int:
     argv = list(sys.argv[1:] if argv is None else argv)
     if argv and argv[0] == "doctor":
         return doctor()
+    if argv and argv[0] == "random-weights":
+        return random_weights(argv[1:])
     ap = argparse.ArgumentParser(prog="machserve_amd", description=__doc__.split("\n\n")[0])
     ap.add_argument("--version", action="version", version=f"machserve_amd {__version__}")
     ap.add_argument("--model", default=_env("MACH_MODEL"), help="folder with config.json and model.safetensors")

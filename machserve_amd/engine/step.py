@@ -18,7 +18,7 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..cache import CacheManager
+from ..cache import CacheError, CacheManager, OutOfPages
 from ..parts.base import GroupView, StepContext
 
 
@@ -37,8 +37,8 @@ class _DecodeGraph:
     """One captured decode step for a fixed number of requests and fixed block-table widths:
     a static int32 buffer the host refills before every replay, and the logits it produces."""
 
-    def __init__(self, graph, dev, pinned, offsets, sizes, logits):
-        self.graph, self.dev, self.pinned, self.offsets, self.sizes, self.logits = graph, dev, pinned, offsets, sizes, logits
+    def __init__(self, graph, dev, pinned, offsets, widths, logits):
+        self.graph, self.dev, self.pinned, self.offsets, self.widths, self.logits = graph, dev, pinned, offsets, widths, logits
         self.sampled = None  # int32 [2, B] when the graph also samples: tokens, bits of the logprobs
         self.copied = torch.cuda.Event()  # the last upload of `pinned` has finished
 
@@ -57,15 +57,13 @@ class StepFunction:
         self._graphs: Dict[tuple, _DecodeGraph] = {}
 
     # ------------------------------------------------------------------ context
-    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
-        cache, ps = self.cache, self.cache.page_size
+    def _check_entries(self, entries: Sequence[StepEntry]):
+        """Validates the entries; returns their slots, token counts, flattened tokens and wanted rows."""
         if not entries:
             raise StepError("a step needs at least one entry")
+        cache, vocab, limit = self.cache, self.model.vocab, self.model.spec.max_positions
         seen = set()
-        vocab = self.model.vocab
-        tokens: List[int] = []
-        positions: List[int] = []
-        q_start, q_len, pos0, slots, want = [], [], [], [], []
+        slots, counts, tokens, want = [], [], [], []
         for e in entries:
             n = len(e.tokens)
             if n == 0:
@@ -73,163 +71,92 @@ class StepFunction:
             if e.slot in seen:
                 raise StepError(f"slot {e.slot} appears twice in one step")
             seen.add(e.slot)
-            p0 = cache.length(e.slot)
-            if p0 + n > self.model.spec.max_positions:
-                raise StepError(f"slot {e.slot}: position {p0 + n - 1} is beyond the model's "
-                                f"{self.model.spec.max_positions} positions")
-            for t in e.tokens:
-                if not 0 <= int(t) < vocab:
-                    raise StepError(f"slot {e.slot}: token {t} is outside the vocabulary of {vocab}")
+            if cache.length(e.slot) + n > limit:
+                raise StepError(f"slot {e.slot}: position {cache.length(e.slot) + n - 1} is beyond the model's {limit} positions")
+            toks = [int(t) for t in e.tokens]
+            if min(toks) < 0 or max(toks) >= vocab:
+                bad = next(t for t in toks if not 0 <= t < vocab)
+                raise StepError(f"slot {e.slot}: token {bad} is outside the vocabulary of {vocab}")
             for w in e.want:
                 if not 0 <= w < n:
                     raise StepError(f"slot {e.slot}: wanted place {w} is outside its {n} tokens")
                 want.append(len(tokens) + w)
-            q_start.append(len(tokens))
-            q_len.append(n)
-            pos0.append(p0)
             slots.append(e.slot)
-            tokens.extend(int(t) for t in e.tokens)
-            positions.extend(range(p0, p0 + n))
-        T, S = len(tokens), len(entries)
+            counts.append(n)
+            tokens.extend(toks)
+        return slots, counts, tokens, want
 
-        sections: Dict[str, np.ndarray] = {
-            "tokens": np.asarray(tokens, dtype=np.int32), "positions": np.asarray(positions, dtype=np.int32),
-            "seq_q_start": np.asarray(q_start, dtype=np.int32), "seq_q_len": np.asarray(q_len, dtype=np.int32),
-            "seq_pos0": np.asarray(pos0, dtype=np.int32), "seq_slot": np.asarray(slots, dtype=np.int32),
-            "want_rows": np.asarray(want, dtype=np.int32),
-        }
-        group_shapes = {}
-        for name in cache.groups:
-            width = max(1, max(len(cache.table(name, s)) for s in slots))
-            table = np.full((S, width), -1, dtype=np.int32)
-            slot_map = np.empty(T, dtype=np.int32)
-            for i, s in enumerate(slots):
-                t = cache.table(name, s)
-                table[i, :len(t)] = t
-                pos = np.arange(pos0[i], pos0[i] + q_len[i])
-                pages = np.asarray(t, dtype=np.int64)[pos // ps]
-                if (pages < 0).any():
-                    raise StepError(f"group {name}: slot {s} writes into a page already given back")
-                slot_map[q_start[i]:q_start[i] + q_len[i]] = pages * ps + pos % ps
-            sections[f"table/{name}"] = table.reshape(-1)
-            sections[f"slot_map/{name}"] = slot_map
-            group_shapes[name] = (S, width)
-        for g in self.heads_per_kv:
-            work = [(i, r0) for i in range(S) for r0 in range(0, q_len[i] * g, self.rows_per_block)]
-            sections[f"work/{g}"] = np.asarray(work, dtype=np.int32).reshape(-1)
-
-        # one buffer, one copy; every section starts on a 16-byte boundary
-        offsets, total = {}, 0
-        for k, a in sections.items():
-            offsets[k] = total
-            total += (a.size + 3) // 4 * 4
-        host = np.zeros(max(total, 4), dtype=np.int32)
-        for k, a in sections.items():
-            host[offsets[k]:offsets[k] + a.size] = a
-        dev = torch.from_numpy(host).to(self.rt.device)
-
+    def _context_from(self, dev: torch.Tensor, offsets, widths: Dict[str, int], host=None) -> StepContext:
+        """A step context over the device copy of a buffer laid out by ``CacheManager.build_step``."""
         def sec(k):
-            return dev[offsets[k]:offsets[k] + sections[k].size]
-
-        ctx = StepContext(
-            n_rows=T, n_seqs=S, tokens=sec("tokens"), positions=sec("positions"), seq_q_start=sec("seq_q_start"),
-            seq_q_len=sec("seq_q_len"), seq_pos0=sec("seq_pos0"), seq_slot=sec("seq_slot"), want_rows=sec("want_rows"),
-            host={"tokens": tokens, "positions": positions, "seq_q_start": q_start, "seq_q_len": q_len,
-                  "seq_pos0": pos0, "seq_slot": slots, "want_rows": want},
-            decode_only=all(n == 1 for n in q_len))
-        for name, (S_, width) in group_shapes.items():
-            ctx.groups[name] = GroupView(ps, sec(f"slot_map/{name}"), sec(f"table/{name}").view(S_, width))
+            start, size = offsets[k]
+            return dev[start:start + size]
+        S, T = offsets["seq_slot"][1], offsets["tokens"][1]
+        ctx = StepContext(n_rows=T, n_seqs=S, tokens=sec("tokens"), positions=sec("positions"),
+                          seq_q_start=sec("seq_q_start"), seq_q_len=sec("seq_q_len"), seq_pos0=sec("seq_pos0"),
+                          seq_slot=sec("seq_slot"), want_rows=sec("want_rows"), host=host or {}, decode_only=S == T)
+        for name, width in widths.items():
+            ctx.groups[name] = GroupView(self.cache.page_size, sec(f"slot_map/{name}"), sec(f"table/{name}").view(S, width))
         for g in self.heads_per_kv:
             ctx.attention_work[g] = sec(f"work/{g}").view(-1, 2)
         return ctx
+
+    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+        slots, counts, tokens, want = self._check_entries(entries)
+        try:
+            host, offsets, widths = self.cache.build_step(slots, counts, tokens, want, self.heads_per_kv, self.rows_per_block)
+        except CacheError as e:
+            raise StepError(str(e)) from e
+        dev = torch.from_numpy(host).to(self.rt.device)  # one buffer, one copy
+        lists = {k: host[offsets[k][0]:offsets[k][0] + offsets[k][1]].tolist()
+                 for k in ("tokens", "positions", "seq_q_start", "seq_q_len", "seq_pos0", "seq_slot", "want_rows")}
+        return self._context_from(dev, offsets, widths, lists)
 
     # ------------------------------------------------------------------ captured decode steps
-    def _decode_sections(self, slots: List[int], tokens: List[int], widths: Dict[str, int]) -> Dict[str, np.ndarray]:
-        """The int32 sections of a step in which every request has one row, block tables padded
-        to ``widths``.  The order of the keys is the layout of the captured buffer."""
-        cache, ps = self.cache, self.cache.page_size
-        B = len(slots)
-        pos = np.fromiter((cache.lengths[s] for s in slots), dtype=np.int32, count=B)
-        ar = np.arange(B, dtype=np.int32)
-        sec: Dict[str, np.ndarray] = {
-            "tokens": np.asarray(tokens, dtype=np.int32), "positions": pos, "seq_q_start": ar,
-            "seq_q_len": np.ones(B, dtype=np.int32), "seq_pos0": pos, "seq_slot": np.asarray(slots, dtype=np.int32),
-            "want_rows": ar,
-        }
-        for name, width in widths.items():
-            table = np.full((B, width), -1, dtype=np.int32)
-            slot_map = np.empty(B, dtype=np.int32)
-            for i, s in enumerate(slots):
-                t = cache.table(name, s)
-                table[i, :len(t)] = t
-                slot_map[i] = t[pos[i] // ps] * ps + pos[i] % ps
-            sec[f"table/{name}"] = table.reshape(-1)
-            sec[f"slot_map/{name}"] = slot_map
-        for g in self.heads_per_kv:
-            sec[f"work/{g}"] = np.stack([ar, np.zeros(B, dtype=np.int32)], 1).reshape(-1)
-        return sec
-
-    def _context_from(self, dev: torch.Tensor, offsets, sizes, B: int, widths: Dict[str, int]) -> StepContext:
-        def sec(k):
-            return dev[offsets[k]:offsets[k] + sizes[k]]
-        ctx = StepContext(n_rows=B, n_seqs=B, tokens=sec("tokens"), positions=sec("positions"),
-                          seq_q_start=sec("seq_q_start"), seq_q_len=sec("seq_q_len"), seq_pos0=sec("seq_pos0"),
-                          seq_slot=sec("seq_slot"), want_rows=sec("want_rows"), decode_only=True)
-        for name, width in widths.items():
-            ctx.groups[name] = GroupView(self.cache.page_size, sec(f"slot_map/{name}"), sec(f"table/{name}").view(B, width))
-        for g in self.heads_per_kv:
-            ctx.attention_work[g] = sec(f"work/{g}").view(-1, 2)
-        return ctx
-
     def _run_decode_graph(self, entries: Sequence[StepEntry], sampling=None):
         """Replay (or first capture) the graph of this batch size.  ``sampling`` = (temperatures,
         top_ks, top_ps, states) makes sampling part of the graph; the result is then the int32
         ``[2, B]`` tensor of :meth:`HipOps.sample_packed`, else the logits."""
-        cache = self.cache
-        slots = [e.slot for e in entries]
-        tokens = [int(e.tokens[0]) for e in entries]
-        vocab = self.model.vocab
-        for s, t in zip(slots, tokens):
-            if not 0 <= t < vocab:
-                raise StepError(f"slot {s}: token {t} is outside the vocabulary of {vocab}")
-            if cache.lengths[s] + 1 > self.model.spec.max_positions:
-                raise StepError(f"slot {s}: position {cache.lengths[s]} is beyond the model's positions")
+        slots, counts, tokens, _ = self._check_entries(entries)
         B = len(slots)
-        bucket = self.TABLE_BUCKET
-        widths = {name: -(-max(len(cache.table(name, s)) for s in slots) // bucket) * bucket for name in cache.groups}
+        host, offsets, widths = self.cache.build_step(slots, counts, tokens, list(range(B)), self.heads_per_kv,
+                                                      self.rows_per_block, self.TABLE_BUCKET)
+        # for a given number of requests and given table widths the layout is always the same
         key = (B, tuple(sorted(widths.items())), sampling is not None)
-        sections = self._decode_sections(slots, tokens, widths)
+        extra: Dict[str, np.ndarray] = {}
         if sampling is not None:
             temps, top_ks, top_ps, states = sampling
-            sections["sample/temperature"] = np.asarray(temps, dtype=np.float32).view(np.int32)
-            sections["sample/top_p"] = np.asarray(top_ps, dtype=np.float32).view(np.int32)
-            sections["sample/top_k"] = np.asarray(top_ks, dtype=np.int32)
-            sections["sample/state"] = np.asarray(states, dtype=np.uint64).view(np.int32)
+            extra["sample/temperature"] = np.asarray(temps, dtype=np.float32).view(np.int32)
+            extra["sample/top_p"] = np.asarray(top_ps, dtype=np.float32).view(np.int32)
+            extra["sample/top_k"] = np.asarray(top_ks, dtype=np.int32)
+            extra["sample/state"] = np.asarray(states, dtype=np.uint64).view(np.int32)
         dg = self._graphs.get(key)
         if dg is None:
-            offsets, sizes, total = {}, {}, 0
-            for k, a in sections.items():
-                offsets[k], sizes[k] = total, a.size
+            offsets = dict(offsets)
+            total = host.size
+            for k, a in extra.items():
+                offsets[k] = (total, a.size)
                 total += (a.size + 3) // 4 * 4
             pinned = torch.empty(total, dtype=torch.int32, pin_memory=True)
             pinned.zero_()
             dev = torch.zeros(total, dtype=torch.int32, device=self.rt.device)
-            dg = _DecodeGraph(None, dev, pinned, offsets, sizes, None)
+            dg = _DecodeGraph(None, dev, pinned, offsets, widths, None)
         dg.copied.synchronize()  # the host buffer is free to be refilled
-        host = dg.pinned.numpy()
-        for k, a in sections.items():
-            host[dg.offsets[k]:dg.offsets[k] + a.size] = a
+        staged = dg.pinned.numpy()
+        staged[:host.size] = host
+        for k, a in extra.items():
+            staged[dg.offsets[k][0]:dg.offsets[k][0] + a.size] = a
         dg.dev.copy_(dg.pinned, non_blocking=True)
         dg.copied.record()
         if dg.graph is None:
-            ctx = self._context_from(dg.dev, dg.offsets, dg.sizes, B, widths)
+            ctx = self._context_from(dg.dev, dg.offsets, widths)
             side = torch.cuda.Stream(device=self.rt.device)
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
                 self.model.forward(ctx)  # everything is loaded and compiled before the capture
             torch.cuda.current_stream().wait_stream(side)
             def sec(k):
-                return dg.dev[dg.offsets[k]:dg.offsets[k] + dg.sizes[k]]
+                return dg.dev[dg.offsets[k][0]:dg.offsets[k][0] + dg.offsets[k][1]]
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 dg.logits = self.model.forward(ctx)
@@ -256,7 +183,6 @@ class StepFunction:
                 reserved[k] = reserved.get(k, 0) + v
         for k, v in reserved.items():
             if cache.free_pages(k) < v:
-                from ..cache import OutOfPages
                 raise OutOfPages(f"group {k}: the step needs {v} new pages, {cache.free_pages(k)} are free")
         for e in entries:
             cache.extend(e.slot, 1)
@@ -280,7 +206,6 @@ class StepFunction:
                 reserved[k] = reserved.get(k, 0) + v
         for k, v in reserved.items():
             if cache.free_pages(k) < v:
-                from ..cache import OutOfPages
                 raise OutOfPages(f"group {k}: the step needs {v} new pages, {cache.free_pages(k)} are free")
         for e in entries:
             cache.extend(e.slot, len(e.tokens))

@@ -107,7 +107,7 @@ def _run_with_heartbeat(cmd, what: str) -> None:
     out, _ = proc.communicate()
     done.set()
     if proc.returncode != 0:
-        raise BuildError(f"{what}: hipcc failed\n$ {' '.join(cmd)}\n{out}")
+        raise BuildError(f"{what}: the compiler failed\n$ {' '.join(cmd)}\n{out}")
 
 
 _locks: dict = {}
@@ -153,8 +153,60 @@ def ensure_library(kind: str, elem: str, nd: int | None = None, force: bool = Fa
         return so
 
 
+HOST_SOURCE = os.path.join("host", "host.cpp")
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall"]
+_host_module = None
+
+
+def ensure_host_module(force: bool = False):
+    """The host runtime (pools, cache manager, step buffer builder) as an imported module; it is
+    compiled from ``csrc/host/host.cpp`` with the C++ compiler and pybind11 when missing or stale."""
+    global _host_module
+    import importlib.util
+    import sysconfig
+    with _lock_of("ms_host"):
+        if _host_module is not None and not force:
+            return _host_module
+        src = os.path.join(CSRC, HOST_SOURCE)
+        libdir = _lib_dir()
+        so = os.path.join(libdir, "ms_host" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
+        stamp = so + ".stamp"
+        h = hashlib.sha256(" ".join(HOST_FLAGS).encode())
+        with open(src, "rb") as fh:
+            h.update(fh.read())
+        digest = h.hexdigest()
+        fresh = False
+        if not force and os.path.exists(so) and os.path.exists(stamp):
+            with open(stamp) as f:
+                fresh = f.read().strip() == digest
+        if not fresh:
+            try:
+                import pybind11
+            except ImportError as e:
+                raise BuildError("pybind11 is needed to build the host runtime") from e
+            cxx = next((c for c in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"))
+                        if c), None)
+            if cxx is None:
+                raise BuildError("no C++ compiler found (looked at $CXX, g++, c++, clang++): the host runtime cannot be built")
+            _say("compiling the host runtime (ms_host)")
+            t0 = time.time()
+            tmp = so + f".tmp{os.getpid()}"
+            cmd = [cxx, *HOST_FLAGS, f"-I{pybind11.get_include()}", f"-I{sysconfig.get_paths()['include']}", src, "-o", tmp]
+            _run_with_heartbeat(cmd, "ms_host")
+            os.replace(tmp, so)
+            with open(stamp, "w") as f:
+                f.write(digest)
+            _say(f"built {os.path.basename(so)} in {time.time() - t0:.0f} s")
+        spec = importlib.util.spec_from_file_location("ms_host", so)
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        _host_module = mod
+        return mod
+
+
 def build_all(force: bool = True, workers: int = 4) -> list:
-    """Every library of both element types (what ``__graft_entry__.build`` calls)."""
+    """Every library of both element types and the host runtime (what ``__graft_entry__.build`` calls)."""
+    ensure_host_module(force=force)
     jobs = []
     for elem in ELEM_DEFINE:
         jobs.append(("core", elem, None))

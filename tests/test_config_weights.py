@@ -218,3 +218,17 @@ def test_shards_equal_single_file_and_renaming(tmp_path):
     save_file({names[0]: whole[names[0]]}, str(sh / "model-00003.safetensors"))
     with pytest.raises(SafetensorsError, match="appears in"):
         Checkpoint(str(sh))
+
+
+def test_random_weights_command(tmp_path):
+    from safetensors.torch import load_file
+    from machserve_amd.cli import main
+    from machserve_amd.weights import random_tensor_dict
+    from machserve_amd.config import config_from_dict
+    cfg = tmp_path / "c.json"
+    cfg.write_text(json.dumps(TINY_B))
+    assert main(["random-weights", "--config", str(cfg), "--seed", "5", "--out", str(tmp_path / "m"), "--dtype", "bf16"]) == 0
+    got = load_file(str(tmp_path / "m" / "model.safetensors"))
+    want = random_tensor_dict(config_from_dict(dict(TINY_B)), 5, torch.bfloat16)
+    assert sorted(got) == sorted(want) and all(torch.equal(got[k], want[k]) for k in got)
+    assert json.load(open(tmp_path / "m" / "config.json"))["torch_dtype"] == "bfloat16"

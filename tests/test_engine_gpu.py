@@ -82,6 +82,40 @@ def test_long_decoding(dirs, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_long_context(tmp_path, dtype):
+    """A 5,000-token prompt in portions of 1,500 and then decoded tokens: positions in the
+    thousands (rotation angles, dozens of pages, split keys in the decode kernel), checked at
+    the ends of the portions and at every decoded position."""
+    from machserve_amd.engine import StepEntry, load_model
+    from machserve_amd.weights import write_random_model
+    from tiny_configs import TINY_A
+    raw = dict(TINY_A, max_position_embeddings=8192, rope_theta=1000000.0)
+    d = write_random_model(raw, 4, str(tmp_path / "long"))
+    w, sizes = read_for_plain(d)
+    ww = w if dtype == torch.float32 else {k: v.to(torch.bfloat16).float() if v.dim() == 2 else v for k, v in w.items()}
+    toks = random_prompt(5010, 512, 6)
+    ref = P.forward(ww, sizes, toks)
+    lm = load_model(d, dtype=dtype, device=DEV, page_size=64, num_pages=80)
+    slot = lm.cache.admit()
+    got, where, i = [], [], 0
+    for c in (1500, 1500, 1500, 500):
+        want = [0, c // 2, c - 1]
+        got.append(lm.step([StepEntry(slot, toks[i:i + c], want)]))
+        where += [i + k for k in want]
+        i += c
+    for j in range(5000, 5010):
+        got.append(lm.step([StepEntry(slot, [toks[j]], [0])]))
+        where.append(j)
+    got = torch.cat(got).float().cpu()
+    scale = ref.abs().max().item()
+    allowed = 1e-4 + 1e-4 * scale if dtype == torch.float32 else 3e-2 * scale
+    # 32-bit: the angle pos * freq itself carries 2^-24 * 5000 of relative error at these positions,
+    # five times the bound used at short positions
+    err = (got - ref[where]).abs().max().item()
+    assert err <= allowed, f"max error {err:.3e}, allowed {allowed:.3e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("which", ["A", "B", "C"])
 def test_first_tokens_of_a_sequence(dirs, which, dtype):
     """Positions 0, 1, 2 alone and together: a one-token prompt, and the first rows of a portion."""
@@ -178,6 +212,18 @@ def test_norm_part_alone(dtype):
     from machserve_amd.parts import ResidualStream
     x = torch.randn(9, 200) * 3
     assert_close(part.forward(ResidualStream(x.to(DEV), part.rt.ops)), P.rms_norm(x, w, 1e-5), dtype)
+
+
+def test_rotary_part_alone():
+    """The position-encoding part owns the table of inverse frequencies, made in 32-bit as
+    1 / theta^(2j / head_dim) (crates/mach-model/src/ref_model.rs:636-643)."""
+    from machserve_amd.config import RotarySpec
+    from machserve_amd.parts import POSITION_ENCODINGS
+    for hd, theta in ((16, 1e4), (64, 1e6), (48, 5e4)):
+        part = POSITION_ENCODINGS.build(RotarySpec("rotary", hd, theta), _runtime(torch.float32))
+        assert part.tensor_decls() == []
+        want = P.rope_angles(torch.tensor([1]), hd, theta)[0]   # the angles at position 1 are the frequencies
+        assert torch.equal(part.rotary_inv_freq().cpu(), want)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -122,9 +122,9 @@ def test_mixed_with_page_reuse(models, which, dtype):
     from machserve_amd.engine import StepEntry
     d, w, sizes, prompts, _ = models[which]
     ps = PAGE[which]
-    seqs = [prompts[i % len(prompts)] for i in range(7)]
-    refs = [plain_logits(models, which, dtype, i % len(prompts)) for i in range(7)]
-    live_cap = 3
+    seqs = [prompts[i % len(prompts)] for i in range(9)]
+    refs = [plain_logits(models, which, dtype, i % len(prompts)) for i in range(9)]
+    live_cap = 4
     pages = sum(sorted(-(-len(s) // ps) for s in seqs)[-live_cap:])
     lm = engine(models, which, dtype, pages)
     got = [[] for _ in seqs]
