@@ -16,7 +16,7 @@ Layout of a page: keys ``[kv_heads, page_size, head_dim]``, values transposed
 ``[kv_heads, head_dim, page_size]``.
 
 Host logic only.  The bookkeeping itself (pools, tables, windows, the step's address buffer) is
-the native ``CacheCore`` of ``csrc/host/host.cpp``; this class sorts the layers' requests into
+the native ``CacheCore`` of ``csrc/host/cache.hpp``; this class sorts the layers' requests into
 groups, names them, and hands device tensors to the layers (``DeviceCache``).
 """
 from __future__ import annotations
@@ -137,6 +137,11 @@ class CacheManager:
         if self.device is not None:
             self.device.zero_state(slot)
         return slot
+
+    def on_admitted(self, slot: int) -> None:
+        """The native scheduler admitted a request into ``slot`` by itself: zero its state."""
+        if self.device is not None:
+            self.device.zero_state(slot)
 
     def length(self, slot: int) -> int:
         return self.core.length(slot)

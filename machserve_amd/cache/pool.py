@@ -1,4 +1,4 @@
-"""Pools of page ids and of state slots, from the native host runtime (``csrc/host/host.cpp``).
+"""Pools of page ids and of state slots, from the native host runtime (``csrc/host/cache.hpp``).
 
 ``BlockPool`` follows the reference's allocator (``crates/mach-model/src/paged_kv.rs:229-289``):
 a LIFO free list over a bump pointer, with a bitmap of live pages so that freeing a page

@@ -5,6 +5,7 @@ produced, ``generate`` runs a list of prompts to the end.  Role of ``ContinuousM
 the reference (``crates/mach-model/src/continuous.rs:715, 943, 1294``)."""
 from __future__ import annotations
 
+import gc
 from typing import Dict, List, Optional, Sequence
 
 from ..sampling import Sampler, SamplingParams
@@ -22,6 +23,11 @@ class Engine:
         self.sampler = Sampler(loaded.rt.ops, loaded.rt.device)
         self.steps = 0
         self.tokens_run = 0
+        # Every step makes a few hundred short-lived objects; with the interpreter's whole heap in the
+        # collector's oldest generation its full passes cost more than the scheduling itself.  What
+        # exists now (modules, the model) is taken out of the collector's reach.
+        gc.collect()
+        gc.freeze()
 
     @classmethod
     def from_dir(cls, model_dir: str, *, dtype="bfloat16", device="cuda:0", page_size: int = 64,

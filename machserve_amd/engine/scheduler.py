@@ -19,16 +19,15 @@ new token appended.
 """
 from __future__ import annotations
 
-from collections import deque
 from dataclasses import dataclass, field
-from typing import Deque, Dict, List, Optional, Sequence
+from typing import Dict, List, Optional, Sequence
 
 from ..cache import CacheManager
+from ..kernels.build import ensure_host_module
 from ..sampling.params import SamplingParams
 
-
-class SchedulerError(ValueError):
-    pass
+_host = ensure_host_module()
+SchedulerError = _host.SchedulerError  # a ValueError
 
 
 @dataclass
@@ -71,6 +70,7 @@ class StepPlan:
     items: List[PlanItem] = field(default_factory=list)
     preempted: List[Request] = field(default_factory=list)
     admitted: List[Request] = field(default_factory=list)
+    native: list = field(default_factory=list)  # the core's own items, handed back to it after the step
 
     @property
     def n_tokens(self) -> int:
@@ -78,153 +78,83 @@ class StepPlan:
 
 
 class Scheduler:
+    """Queues and decisions live in the native ``SchedulerCore`` (``csrc/host/scheduler.hpp``); this
+    class keeps the requests' tokens, sampling options and results, and mirrors ``fed``, ``slot``
+    and ``preemptions`` from the core's plans."""
+
     def __init__(self, cache: CacheManager, max_batch_tokens: int = 512, chunk_size: Optional[int] = None,
                  max_running: Optional[int] = None, max_positions: Optional[int] = None):
-        if max_batch_tokens < 1:
-            raise SchedulerError("max_batch_tokens must be at least 1")
         self.cache = cache
-        self.max_batch_tokens = max_batch_tokens
-        self.chunk_size = chunk_size or max_batch_tokens
-        self.max_running = min(max_running or cache.max_requests, cache.max_requests)
+        self.core = _host.SchedulerCore(cache.core, max_batch_tokens, chunk_size or 0, max_running or 0, max_positions or 0)
+        self.max_batch_tokens = self.core.max_batch_tokens
+        self.chunk_size = self.core.chunk_size
+        self.max_running = self.core.max_running
         self.max_positions = max_positions
-        self.waiting: Deque[Request] = deque()
-        self.running: List[Request] = []  # oldest first
+        self.requests: Dict[int, Request] = {}  # waiting or running
         self.finished: Dict[int, Request] = {}
         self._next_id = 1
+
+    @property
+    def waiting(self) -> List[Request]:
+        return [self.requests[i] for i in self.core.waiting()]
+
+    @property
+    def running(self) -> List[Request]:
+        """Oldest first."""
+        return [self.requests[i] for i in self.core.running()]
 
     # ------------------------------------------------------------------ admission
     def add(self, prompt: Sequence[int], max_new: int, params: Optional[SamplingParams] = None,
             eos: Optional[int] = None, stop_seqs: Sequence[Sequence[int]] = ()) -> int:
-        """Queue a request; returns its id.  Refusals follow ``continuous.rs:788-800``: empty
-        prompt, prompt beyond the model's positions; and, ours, a request the pool could
-        never hold."""
+        """Queue a request; returns its id.  Refused: an empty prompt, a prompt beyond the model's
+        positions (``continuous.rs:788-800``), and a request the pool could never hold."""
         prompt = [int(t) for t in prompt]
-        if not prompt:
-            raise SchedulerError("empty prompt")
-        if max_new < 1:
-            raise SchedulerError(f"max_new {max_new} must be at least 1")
-        if self.max_positions is not None and len(prompt) >= self.max_positions:
-            raise SchedulerError(f"prompt of {len(prompt)} tokens leaves no room within {self.max_positions} positions")
-        total = len(prompt) + max_new - 1  # the last generated token is never fed
-        if self.max_positions is not None:
-            total = min(total, self.max_positions)
-        ps = self.cache.page_size
-        for name, g in self.cache.groups.items():
-            if -(-total // ps) > g.pool.num_pages:
-                raise SchedulerError(f"request of up to {total} cached tokens needs {-(-total // ps)} pages; "
-                                     f"group {name} has {g.pool.num_pages}")
         params = params or SamplingParams()
         params.validate()
         rid = self._next_id
+        self.core.add(rid, len(prompt), max_new)
         self._next_id += 1
         seed = params.seed if params.seed != 0 else rid  # continuous.rs:803
         req = Request(rid, prompt, max_new, params, eos, [list(s) for s in stop_seqs if len(s)],
                       tokens=list(prompt), rng_state=seed & ((1 << 64) - 1))
-        self.waiting.append(req)
+        self.requests[rid] = req
         return rid
 
     def cancel(self, rid: int) -> bool:
-        for r in list(self.waiting):
-            if r.id == rid:
-                self.waiting.remove(r)
-                self._finish(r, "cancelled")
-                return True
-        for r in self.running:
-            if r.id == rid:
-                self._finish(r, "cancelled")
-                return True
-        return False
+        r = self.requests.get(rid)
+        if r is None:
+            return False
+        self._finish(r, "cancelled")
+        return True
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.running)
+        return self.core.has_work()
 
     # ------------------------------------------------------------------ planning
-    def _preempt_youngest(self, plan: StepPlan) -> Request:
-        victim = self.running.pop()
-        self.cache.release(victim.slot)
-        victim.slot, victim.fed = None, 0
-        victim.preemptions += 1
-        self.waiting.appendleft(victim)
-        plan.preempted.append(victim)
-        plan.items = [i for i in plan.items if i.request is not victim]
-        return victim
-
-    def _reserved(self, plan: StepPlan) -> Dict[str, int]:
-        res: Dict[str, int] = {}
-        for it in plan.items:
-            for k, v in self.cache.pages_needed(it.request.slot, it.count).items():
-                res[k] = res.get(k, 0) + v
-        return res
-
     def schedule(self) -> StepPlan:
         """The next step: every decoding request's token first, then prompt portions of running
         requests, then newly admitted requests, under the token budget and the free pages."""
-        plan = StepPlan()
-        while True:
-            plan.items = []
-            budget = self.max_batch_tokens
-            # 1. decoded tokens, oldest request first; they must all fit, or the youngest goes
-            decoders = [r for r in self.running if r.decoding]
-            need: Dict[str, int] = {}
-            for r in decoders:
-                for k, v in self.cache.pages_needed(r.slot, 1).items():
-                    need[k] = need.get(k, 0) + v
-            if any(self.cache.free_pages(k) < v for k, v in need.items()):
-                self._preempt_youngest(plan)
-                continue
-            for r in decoders:
-                if budget == 0:
-                    break
-                plan.items.append(PlanItem(r, r.fed, 1, True))
-                budget -= 1
-            # 2. portions of prompts (or of a recomputation) already running, oldest first; an
-            #    older request that lacks pages takes them from the youngest
-            restart = False
-            for r in self.running:
-                if r.decoding or budget == 0:
-                    continue
-                n = min(len(r.tokens) - r.fed, self.chunk_size, budget)
-                if not self.cache.can_extend(r.slot, n, self._reserved(plan)):
-                    if r is not self.running[-1]:
-                        self._preempt_youngest(plan)
-                        restart = True
-                        break
-                    continue
-                plan.items.append(PlanItem(r, r.fed, n, r.fed + n == len(r.tokens)))
-                budget -= n
-            if restart:
-                continue
-            # 3. admission, first come first served
-            while self.waiting and budget > 0 and len(self.running) < self.max_running \
-                    and self.cache.slots.available() > 0:
-                r = self.waiting[0]
-                if r in plan.preempted:  # it lost its pages in this very step
-                    break
-                n = min(len(r.tokens), self.chunk_size, budget)
-                res = self._reserved(plan)
-                ps = self.cache.page_size
-                if any(self.cache.free_pages(k) - res.get(k, 0) < -(-n // ps) for k in self.cache.groups):
-                    break
-                self.waiting.popleft()
-                r.slot = self.cache.admit()
-                r.fed = 0
-                self.running.append(r)
-                plan.admitted.append(r)
-                plan.items.append(PlanItem(r, 0, n, n == len(r.tokens)))
-                budget -= n
-            if plan.items or not self.running:
-                return plan
-            # running requests exist but none can move: they hold each other's pages
-            self._preempt_youngest(plan)
+        native = self.core.schedule()
+        plan = StepPlan(native=native.items)
+        for rid in native.preempted:
+            r = self.requests[rid]
+            r.slot, r.fed = None, 0
+            r.preemptions += 1
+            plan.preempted.append(r)
+        for rid, slot in native.admitted:
+            r = self.requests[rid]
+            r.slot, r.fed = slot, 0
+            self.cache.on_admitted(slot)
+            plan.admitted.append(r)
+        plan.items = [PlanItem(self.requests[i.id], i.start, i.count, i.sample) for i in native.items]
+        return plan
 
     # ------------------------------------------------------------------ after the step
     def _finish(self, r: Request, reason: str) -> None:
         r.finish_reason = reason
-        if r in self.running:
-            self.running.remove(r)
-        if r.slot is not None:
-            self.cache.release(r.slot)
-            r.slot = None
+        self.core.finish(r.id)  # its pages and slot go back
+        r.slot = None
+        del self.requests[r.id]
         self.finished[r.id] = r
 
     def update(self, plan: StepPlan, sampled: Sequence[int], logprobs: Optional[Sequence[float]] = None,
@@ -232,6 +162,7 @@ class Scheduler:
         """The step ran: ``sampled[i]`` is the token of the i-th item with ``sample`` set.
         Returns the list of (request id, token) emitted and the requests that finished."""
         emitted, done = [], []
+        self.core.advance(plan.native)
         k = 0
         for it in plan.items:
             r = it.request
@@ -246,13 +177,13 @@ class Scheduler:
             k += 1
             r.tokens.append(tok)
             emitted.append((r.id, tok))
-            gen = r.generated
+            n_gen = len(r.tokens) - len(r.prompt)
             reason = None
             if r.eos is not None and tok == r.eos:
                 reason = "stop"
-            elif any(len(gen) >= len(s) and gen[-len(s):] == list(s) for s in r.stop_seqs):
+            elif any(n_gen >= len(s) and r.tokens[-len(s):] == s for s in r.stop_seqs):
                 reason = "stop"
-            elif len(gen) >= r.max_new:
+            elif n_gen >= r.max_new:
                 reason = "length"
             elif self.max_positions is not None and len(r.tokens) > self.max_positions:
                 reason = "length"

@@ -153,27 +153,28 @@ def ensure_library(kind: str, elem: str, nd: int | None = None, force: bool = Fa
         return so
 
 
-HOST_SOURCE = os.path.join("host", "host.cpp")
+HOST_SOURCES = [os.path.join("host", f) for f in ("module.cpp", "cache.hpp", "scheduler.hpp")]  # the first is compiled
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall"]
 _host_module = None
 
 
 def ensure_host_module(force: bool = False):
     """The host runtime (pools, cache manager, step buffer builder) as an imported module; it is
-    compiled from ``csrc/host/host.cpp`` with the C++ compiler and pybind11 when missing or stale."""
+    compiled from ``csrc/host/module.cpp`` with the C++ compiler and pybind11 when missing or stale."""
     global _host_module
     import importlib.util
     import sysconfig
     with _lock_of("ms_host"):
         if _host_module is not None and not force:
             return _host_module
-        src = os.path.join(CSRC, HOST_SOURCE)
+        src = os.path.join(CSRC, HOST_SOURCES[0])
         libdir = _lib_dir()
         so = os.path.join(libdir, "ms_host" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
         stamp = so + ".stamp"
         h = hashlib.sha256(" ".join(HOST_FLAGS).encode())
-        with open(src, "rb") as fh:
-            h.update(fh.read())
+        for f in HOST_SOURCES:
+            with open(os.path.join(CSRC, f), "rb") as fh:
+                h.update(fh.read())
         digest = h.hexdigest()
         fresh = False
         if not force and os.path.exists(so) and os.path.exists(stamp):
