@@ -44,6 +44,11 @@ constexpr int NTP = (NT + 1) / 2;        // pairs of score tiles = K steps of th
 constexpr int K_LD = HDT + KPAD, V_LD = BKV + VPAD;
 constexpr int ROWS_PER_BLOCK = 64;
 constexpr float NEG_BIG = -1e30f;
+#ifdef MS_ELEM_BF16
+constexpr int MAX_KEY_GROUPS = ND <= 4 ? 4 : 2;  // groups of four waves that may share a block's keys
+#else
+constexpr int MAX_KEY_GROUPS = 2;
+#endif
 
 struct AttnArgs {
     const elem_t* q;         // [T, H, hd]
@@ -67,6 +72,12 @@ __device__ __forceinline__ float exp_f(float x) {
 #endif
 }
 
+// The value unchanged, but of unknown origin to the optimiser.
+__device__ __forceinline__ int opaque(int x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
+
 __device__ __forceinline__ float exp2_f(float x) {
 #ifdef MS_ELEM_BF16
     return __builtin_amdgcn_exp2f(x);
@@ -75,11 +86,21 @@ __device__ __forceinline__ float exp2_f(float x) {
 #endif
 }
 
-__global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
-    __shared__ __attribute__((aligned(16))) elem_t Ks[BKV * K_LD];
-    __shared__ __attribute__((aligned(16))) elem_t Vs[HDT * V_LD];
+// KG "key groups" of four waves each share a block: group kg takes the key tiles whose absolute
+// index is kg modulo KG, with its own staging buffers, and the groups' running (max, sum, output)
+// are merged through LDS at the end.  A block's time is the length of its serial chain of tiles,
+// and a causal prompt's last rows see every key: more groups cut that chain.
+template <int KG>
+__global__ __launch_bounds__(256 * KG) void paged_attention_kernel(AttnArgs a) {
+    constexpr int KS_ELEMS = BKV * K_LD, VS_ELEMS = HDT * V_LD;
+    constexpr int STAGE_BYTES = (KS_ELEMS + VS_ELEMS) * (int)sizeof(elem_t);
+    constexpr int MERGE_FLOATS = 4 * 64 * (4 * ND + 2);  // per group: four waves, per lane the output and (max, sum)
+    constexpr int SMEM_BYTES = KG * STAGE_BYTES > (KG - 1) * MERGE_FLOATS * 4 ? KG * STAGE_BYTES : (KG - 1) * MERGE_FLOATS * 4;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kg = threadIdx.x >> 8, tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
+    elem_t* Ks = reinterpret_cast<elem_t*>(smem + kg * STAGE_BYTES);
+    elem_t* Vs = Ks + KS_ELEMS;
     const int r16 = lane & 15, grp = lane >> 4;
     const int s = a.work[blockIdx.x * 2], r0 = a.work[blockIdx.x * 2 + 1];
     const int kvh = blockIdx.y;
@@ -122,62 +143,104 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
     float m_run = NEG_BIG, l_run = 0.f;
     const float sl = a.scale * 1.4426950408889634f;
 
-    // Tiles go global -> registers -> LDS.  PF tiles are in flight at any time: a tile's loads are
-    // requested PF tiles before it is multiplied, which covers the memory latency even when few
-    // blocks share a CU.  Where a tile's 16-key groups lie in the pools is looked up once per tile
-    // by NT threads and shared through LDS (offsets in units of 16 elements).
+    // Tiles go global -> registers -> LDS.  PF tiles per group are in flight at any time: a tile's
+    // loads are requested PF rounds before it is multiplied, which covers the memory latency even
+    // when few blocks share a CU.  Where a tile's 16-key groups lie in the pools is looked up once
+    // per tile by NT threads and shared through LDS (offsets in units of 16 elements).
     constexpr int CPRK = HDT / EPC, CPRV = BKV / EPC;
     constexpr int NCK = (BKV * CPRK + 255) / 256, NCV = (HDT * CPRV + 255) / 256;
-    constexpr int PF = ND <= 4 ? 4 : (ND <= 8 ? 2 : 1);
+    constexpr int PF = KG == 1 ? (ND <= 4 ? 4 : (ND <= 8 ? 2 : 1)) : (ND <= 8 ? 2 : 1);
     constexpr unsigned ABSENT = 0xffffffffu;
-    __shared__ unsigned kofs[PF][NT], vofs[PF][NT];
+    __shared__ unsigned kofs[KG][PF][NT], vofs[KG][PF][NT];
     u32x4 rk[PF][NCK], rv[PF][NCV];
-    auto fill_offsets = [&](int kt0, int slot) {  // threads tid < NT
-        const int key0 = kt0 + tid * 16;
-        unsigned ko = ABSENT, vo = ABSENT;
-        if (key0 < kv_hi) {
-            const int page = table[key0 / ps], off = key0 % ps;
-            if (page >= 0) {
-                const size_t pk = (size_t)page * a.KV + kvh;
-                ko = (unsigned)(((pk * ps + off) * hd) >> 4);
-                vo = (unsigned)((pk * hd * ps + off) >> 4);
-            }
-        }
-        kofs[slot][tid] = ko;
-        vofs[slot][tid] = vo;
+    // what does not change from tile to tile: where in a 16-key group this thread's chunks lie (an
+    // unused chunk, beyond the head size or the tile, reads the start of the pool)
+    const elem_t* k_base[NCK];
+    const elem_t* v_base[NCV];
+    bool k_on[NCK], v_on[NCV];
+#pragma unroll
+    for (int i = 0; i < NCK; ++i) {
+        const int c = tid + i * 256, kl = c / CPRK, d0 = (c % CPRK) * EPC;
+        k_on[i] = c < BKV * CPRK && d0 < hd;
+        k_base[i] = a.kpool + (k_on[i] ? (kl % 16) * hd + d0 : 0);
+    }
+#pragma unroll
+    for (int i = 0; i < NCV; ++i) {
+        const int c = tid + i * 256, d = c / CPRV, k0 = (c % CPRV) * EPC;
+        v_on[i] = c < HDT * CPRV && d < hd;
+        v_base[i] = a.vpool + (v_on[i] ? d * ps + (k0 % 16) : 0);
+    }
+    // Every load below is unconditional (an absent or unused chunk reads the start of the pool and is
+    // zeroed when it is stored to LDS, PF rounds later): with loads on one straight path, and no use
+    // of the loaded values before that, the compiler counts the loads and waits only for the tile it
+    // is about to use, and the younger tiles stay in flight.  The page of a tile's 16-key group is
+    // read one round before its offsets are needed; which logical page that is, is stepped from
+    // round to round rather than divided out.
+    constexpr int ROUND = KG * BKV;  // keys per round of the block
+    const int tsub = tid % NT;
+    const int round_pages = ROUND / ps, round_rem = ROUND % ps;
+    int key_next, lp_next, off_next;  // this thread's 16-key group of the next tile to look up
+    auto start_lookup = [&](int kt0) {
+        key_next = kt0 + tsub * 16;
+        lp_next = key_next / ps;
+        off_next = key_next % ps;
     };
+    struct Entry { int page, off; };
+    auto lookup = [&]() {  // page (or -1) and offset in it of the group; moves on by one round
+        Entry e{table[min(lp_next, a.table_stride - 1)] | (key_next < kv_hi ? 0 : -1), off_next};
+        key_next += ROUND;
+        lp_next += round_pages;
+        off_next += round_rem;
+        if (off_next >= ps) {
+            off_next -= ps;
+            ++lp_next;
+        }
+        return e;
+    };
+    auto fill_offsets = [&](int slot, Entry e) {
+        if (tid < NT) {
+            const size_t pk = (size_t)max(e.page, 0) * a.KV + kvh;
+            kofs[kg][slot][tid] = e.page >= 0 ? (unsigned)(((pk * ps + e.off) * hd) >> 4) : ABSENT;
+            vofs[kg][slot][tid] = e.page >= 0 ? (unsigned)((pk * hd * ps + e.off) >> 4) : ABSENT;
+        }
+    };
+    unsigned live[PF];  // bit i: chunk i of the slot's tile was really read (K chunks first, then V)
     auto load_tile = [&](int slot, u32x4* pk, u32x4* pv) {
+        unsigned bits = 0;
 #pragma unroll
         for (int i = 0; i < NCK; ++i) {
-            const int c = tid + i * 256;
-            const int kl = c / CPRK, d0 = (c % CPRK) * EPC;
-            const unsigned o = kofs[slot][(kl / 16) % NT];
-            u32x4 v = {0, 0, 0, 0};
-            if (c < BKV * CPRK && o != ABSENT && d0 < hd)
-                v = *reinterpret_cast<const u32x4*>(a.kpool + ((size_t)o << 4) + (kl % 16) * hd + d0);
-            pk[i] = v;
+            const int kl = (tid + i * 256) / CPRK;
+            const unsigned o = kofs[kg][slot][(kl / 16) % NT];
+            const bool on = k_on[i] && o != ABSENT;
+            pk[i] = *reinterpret_cast<const u32x4*>(k_base[i] + ((size_t)(on ? o : 0u) << 4));
+            bits |= (on ? 1u : 0u) << i;
         }
 #pragma unroll
         for (int i = 0; i < NCV; ++i) {
-            const int c = tid + i * 256;
-            const int d = c / CPRV, k0 = (c % CPRV) * EPC;
-            const unsigned o = vofs[slot][(k0 / 16) % NT];
-            u32x4 v = {0, 0, 0, 0};
-            if (c < HDT * CPRV && o != ABSENT && d < hd)
-                v = *reinterpret_cast<const u32x4*>(a.vpool + ((size_t)o << 4) + (size_t)d * ps + (k0 % 16));
-            pv[i] = v;
+            const int k0 = ((tid + i * 256) % CPRV) * EPC;
+            const unsigned o = vofs[kg][slot][(k0 / 16) % NT];
+            const bool on = v_on[i] && o != ABSENT;
+            pv[i] = *reinterpret_cast<const u32x4*>(v_base[i] + ((size_t)(on ? o : 0u) << 4));
+            bits |= (on ? 1u : 0u) << (NCK + i);
         }
+        live[slot] = bits;
     };
-    auto store_tile = [&](const u32x4* pk, const u32x4* pv) {
+    auto store_tile = [&](int slot, const u32x4* pk, const u32x4* pv) {
+        const unsigned bits = live[slot];
+        const bool all = bits == (1u << (NCK + NCV)) - 1;  // nearly always: the masks cost nothing then
 #pragma unroll
         for (int i = 0; i < NCK; ++i) {
             const int c = tid + i * 256;
-            if (c < BKV * CPRK) *reinterpret_cast<u32x4*>(&Ks[(c / CPRK) * K_LD + (c % CPRK) * EPC]) = pk[i];
+            const unsigned keep = (all || (bits >> i & 1)) ? 0xffffffffu : 0u;
+            if (c < BKV * CPRK)
+                *reinterpret_cast<u32x4*>(&Ks[(c / CPRK) * K_LD + (c % CPRK) * EPC]) = all ? pk[i] : pk[i] & (u32x4){keep, keep, keep, keep};
         }
 #pragma unroll
         for (int i = 0; i < NCV; ++i) {
             const int c = tid + i * 256;
-            if (c < HDT * CPRV) *reinterpret_cast<u32x4*>(&Vs[(c / CPRV) * V_LD + (c % CPRV) * EPC]) = pv[i];
+            const unsigned keep = (all || (bits >> (NCK + i) & 1)) ? 0xffffffffu : 0u;
+            if (c < HDT * CPRV)
+                *reinterpret_cast<u32x4*>(&Vs[(c / CPRV) * V_LD + (c % CPRV) * EPC]) = all ? pv[i] : pv[i] & (u32x4){keep, keep, keep, keep};
         }
     };
     // rows of this wave: the first and the last position decide which tiles need no mask at all
@@ -185,26 +248,27 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
     const int pos_last = pos0 + min(r0 + wave * 16 + 15, max(R - 1, 0)) / g;
     const int lo_last = a.window > 0 ? pos_last - a.window + 1 : 0;
 
-    const int kt_first = (kv_lo / BKV) * BKV;
-    if (tid < NT) {
+    // round r, slot j: group kg has the tile of absolute index (round_first + r * PF + j) * KG + kg
+    const int kt_first = (kv_lo / ROUND) * ROUND;
+    start_lookup(kt_first + kg * BKV);
 #pragma unroll
-        for (int j = 0; j < PF; ++j) fill_offsets(kt_first + j * BKV, j);
-    }
+    for (int j = 0; j < PF; ++j) fill_offsets(j, lookup());
+    Entry ahead = lookup();
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < PF; ++j)
-        if (kt_first + j * BKV < kv_hi) load_tile(j, rk[j], rv[j]);
-    for (int kt_base = kt_first; kt_base < kv_hi; kt_base += PF * BKV) {
+    for (int j = 0; j < PF; ++j) load_tile(j, rk[j], rv[j]);
+    for (int kt_base = kt_first; kt_base < kv_hi; kt_base += PF * ROUND) {
 #pragma unroll
       for (int j = 0; j < PF; ++j) {
-        const int kt0 = kt_base + j * BKV;
-        if (kt0 >= kv_hi) break;
-        __syncthreads();  // the previous tile has been consumed
-        store_tile(rk[j], rv[j]);
-        if (tid < NT) fill_offsets(kt0 + PF * BKV, j);
+        if (kt_base + j * ROUND >= kv_hi) break;  // the same for every thread of the block
+        const int kt0 = kt_base + j * ROUND + kg * BKV;
+        __syncthreads();  // the previous tiles have been consumed
+        store_tile(j, rk[j], rv[j]);
+        fill_offsets(j, ahead);
+        ahead = lookup();
         __syncthreads();
-        if (kt0 + PF * BKV < kv_hi) load_tile(j, rk[j], rv[j]);
-        if (!wave_active) continue;
+        load_tile(j, rk[j], rv[j]);
+        if (!wave_active || kt0 >= kv_hi) continue;
 
         // S^T = K Q^T: lane holds keys grp * 4 + i of tile nt for query row r16
         f32x4 sc[NT];
@@ -241,7 +305,6 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
         tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
         const float m_new = fmaxf(m_run, tmax);
-        const float alpha = exp2_f((m_run - m_new) * sl);
         const float mb = m_new * sl;
         float psum = 0.f;
 #pragma unroll
@@ -254,12 +317,17 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
             }
         psum += __shfl_xor(psum, 16, WAVE);
         psum += __shfl_xor(psum, 32, WAVE);
-        l_run = l_run * alpha + psum;
+        // where no row's maximum rose the factor is exactly one: after the first tiles that is the rule
+        if (__any(m_new > m_run)) {
+            const float alpha = exp2_f((m_run - m_new) * sl);
+            l_run *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc_o[dt][i] *= alpha;
+        }
+        l_run += psum;
         m_run = m_new;
-#pragma unroll
-        for (int dt = 0; dt < ND; ++dt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc_o[dt][i] *= alpha;
 
         // O^T += V^T P^T: the probabilities of two score tiles form one B fragment
 #pragma unroll
@@ -287,6 +355,36 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
             }
         }
       }
+    }
+
+    if constexpr (KG > 1) {
+        // groups 1.. hand (output, max, sum) to group 0 through LDS, which adds them in group order
+        __syncthreads();  // the staging buffers are free
+        float* mg = reinterpret_cast<float*>(smem);
+        if (kg > 0) {
+            float* mine = mg + ((size_t)(kg - 1) * 4 + wave) * 64 * (4 * ND + 2);
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) mine[(dt * 4 + i) * 64 + lane] = acc_o[dt][i];
+            mine[(4 * ND) * 64 + lane] = m_run;
+            mine[(4 * ND + 1) * 64 + lane] = l_run;
+        }
+        __syncthreads();
+        if (kg > 0) return;
+#pragma unroll
+        for (int o = 0; o < KG - 1; ++o) {
+            const float* other = mg + ((size_t)o * 4 + wave) * 64 * (4 * ND + 2);
+            const float m_o = other[(4 * ND) * 64 + lane], l_o = other[(4 * ND + 1) * 64 + lane];
+            const float m_new = fmaxf(m_run, m_o);
+            const float c0 = exp2_f((m_run - m_new) * sl), c1 = exp2_f((m_o - m_new) * sl);
+            l_run = l_run * c0 + l_o * c1;
+            m_run = m_new;
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc_o[dt][i] = acc_o[dt][i] * c0 + other[(dt * 4 + i) * 64 + lane] * c1;
+        }
     }
 
     if (valid) {
@@ -364,47 +462,82 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
     const int tps = max(1, ceil_div(t_hi - t_lo, a.nsplit));
     const int t0 = t_lo + sp * tps, t1 = min(t_hi, t0 + tps);
 
-    // Loads of a tile depend on nothing the prologue computes: the first tile is requested
-    // before the prologue so that its latency hides behind it.
-    auto load_tile = [&](int t, DecodeTile& td) {
+    // Where the keys of a tile sit in the MFMA rows is free, as long as the probabilities meet the
+    // values of the same keys.  With an even number of 16-key score tiles, the pair (2pp, 2pp + 1)
+    // covers 32 keys so that the lane of key group `grp` ends up with the probabilities of the eight
+    // consecutive keys pp * 32 + grp * 8 ..: its V^T fragment is then one contiguous read.  Row r16 of
+    // score tile 2pp + j holds key pp * 32 + (r16 / 4) * 8 + j * 4 + r16 % 4.
+    constexpr bool PAIRED = NT % 2 == 0;
+    auto k_row = [&](int nt) { return PAIRED ? (nt / 2) * 32 + (r16 >> 2) * 8 + (nt & 1) * 4 + (r16 & 3) : nt * 16 + r16; };
+    auto score_key = [&](int nt, int i) { return PAIRED ? (nt / 2) * 32 + grp * 8 + (nt & 1) * 4 + i : nt * 16 + grp * 4 + i; };
+    // Loads are unconditional and on one straight path, so that the compiler counts them and a wait
+    // for one tile leaves the next in flight: a key that is not there (beyond the row, in a page
+    // given back, in a tile past the split) is read from the start of the pool instead and masked in
+    // the scores.  The pools hold finite values everywhere, so a value that meets a zero probability
+    // adds nothing.  The pages of a tile's 16-key groups are looked up one tile ahead.
+    const float inv_gpp = 1.0f / (float)(ps >> 4);  // 1 / (16-key groups per page)
+    // of this lane's groups: page as the table has it, -1 if the group is not to be read (else 0), offset in the page
+    struct Pages { int kp[NTP], kx[NTP], ko[NTP], vp[NTP], vx[NTP], vo[NTP]; };
+    auto lookup = [&](int t) {
+        Pages pg;
         const int kt0 = t * BKV;
 #pragma unroll
+        for (int pp = 0; pp < NTP; ++pp) {
+            // 16-key groups of this lane: of its K rows of score tiles 2pp and 2pp + 1, and of its V keys
+            const int gk = (kt0 >> 4) + (PAIRED ? 2 * pp + (r16 >> 3) : pp), gv = (kt0 >> 4) + (PAIRED ? 2 * pp + (grp >> 1) : pp);
+            const int lk = (int)(((float)gk + 0.5f) * inv_gpp), lv = (int)(((float)gv + 0.5f) * inv_gpp);
+            const int pk = table[min(lk, a.table_stride - 1)], pv = table[min(lv, a.table_stride - 1)];
+            // The loaded pages are not touched here (a use would wait for them), and are later "or"-ed with
+            // a mask the compiler cannot see through: it would turn a select (and an "or" with a known
+            // 0 / -1, which it reads as one) into a branch around the load.
+            pg.kp[pp] = pk;
+            pg.kx[pp] = opaque((t < t1 && gk * 16 < kv_len) ? 0 : -1);
+            pg.ko[pp] = gk * 16 - lk * ps;
+            pg.vp[pp] = pv;
+            pg.vx[pp] = opaque((t < t1 && gv * 16 < kv_len) ? 0 : -1);
+            pg.vo[pp] = gv * 16 - lv * ps;
+        }
+        return pg;
+    };
+    const size_t page_elems = (size_t)ps * hd;
+    auto load_tile = [&](const Pages& pg, DecodeTile& td) {
+#pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            const int key = kt0 + nt * 16 + r16;
-            const int page = key < kv_len ? table[key / ps] : -1;
-            const elem_t* krow = a.kpool + (((size_t)max(page, 0) * a.KV + kvh) * ps + key % ps) * hd;
+            // the row of (page, kvh, offset of the row's 16-key group + place in the group) in [pages, KV, ps, hd]
+            const int pp = PAIRED ? nt / 2 : nt;
+            const int page = pg.kp[pp] | pg.kx[pp], off = pg.ko[pp] + (k_row(nt) & 15);
+            const elem_t* krow = page >= 0 ? a.kpool + ((size_t)page * a.KV + kvh) * page_elems + (size_t)off * hd : a.kpool;
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) {
                 const int d0 = ks * 32 + grp * 8;
-                td.kf[nt][ks] = (page >= 0 && d0 < hd) ? frag_load(krow + d0) : frag_zero();
+                td.kf[nt][ks] = frag_load(krow + (d0 < hd ? d0 : 0));  // beyond the head size q is zero
             }
         }
 #pragma unroll
         for (int pp = 0; pp < NTP; ++pp) {
-            // the two 4-key groups this lane multiplies: same 16-key tile -> same page
-            const int ka = kt0 + (2 * pp) * 16 + grp * 4, kb = ka + 16;
-            const int pa = ka < kv_len ? table[ka / ps] : -1;
-            const int pb = (2 * pp + 1 < NT && kb < kv_len) ? table[kb / ps] : -1;
+            const int page = pg.vp[pp] | pg.vx[pp], off = pg.vo[pp] + (PAIRED ? (grp & 1) * 8 : grp * 4);
+            const elem_t* vcol = page >= 0 ? a.vpool + ((size_t)page * a.KV + kvh) * page_elems + off : a.vpool;
 #pragma unroll
             for (int dt = 0; dt < ND; ++dt) {
                 const int d = dt * 16 + r16;
-                Frag vf = frag_zero();
-                if (pa >= 0 && d < hd) {
-                    const elem_t* v0 = a.vpool + (((size_t)pa * a.KV + kvh) * hd + d) * ps + ka % ps;
+                const elem_t* v0 = vcol + (page >= 0 && d < hd ? (size_t)d * ps : 0);
+                if constexpr (PAIRED) {
+                    td.vf[pp][dt] = frag_load(v0);
+                } else {
+                    Frag vf = frag_zero();
 #pragma unroll
                     for (int i = 0; i < 4; ++i) vf.v[i] = v0[i];
+                    td.vf[pp][dt] = vf;
                 }
-                if (pb >= 0 && d < hd) {
-                    const elem_t* v1 = a.vpool + (((size_t)pb * a.KV + kvh) * hd + d) * ps + kb % ps;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) vf.v[4 + i] = v1[i];
-                }
-                td.vf[pp][dt] = vf;
             }
         }
     };
+    // The first tile depends on nothing the prologue computes: it is requested before the prologue
+    // so that its latency hides behind it.
     DecodeTile next;
-    if (t0 + wave < t1) load_tile(t0 + wave, next);
+    Pages ahead = lookup(t0 + wave);
+    load_tile(ahead, next);
+    ahead = lookup(t0 + wave + 4);
 
     Frag qf[NKS];
     if constexpr (FUSED) {
@@ -476,10 +609,8 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
     for (int i = 0; i < ND; ++i) acc_o[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m_run = NEG_BIG, l_run = 0.f;
 
-    for (int t = t0 + wave; t < t1; t += 4) {
+    auto process = [&](const DecodeTile& cur, int t) {
         const int kt0 = t * BKV;
-        DecodeTile cur = next;
-        if (t + 4 < t1) load_tile(t + 4, next);
         f32x4 sc[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
@@ -492,7 +623,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int key = kt0 + nt * 16 + grp * 4 + i;
+                const int key = kt0 + score_key(nt, i);
                 const bool ok = valid && key < kv_len && key >= lo_key;
                 const float v = ok ? sc[nt][i] * a.scale : -INFINITY;
                 sc[nt][i] = v;
@@ -530,6 +661,21 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
 #pragma unroll
             for (int dt = 0; dt < ND; ++dt) mma_16x16x32(acc_o[dt], cur.vf[pp][dt], pf);
         }
+    };
+    // Two tile buffers take turns, so that no tile is copied.  The loads of the tile after next are
+    // issued before the current tile is multiplied, and the scheduler may not move them below it:
+    // it would, to keep fewer registers live, and the loads' latency would then lie open.
+    DecodeTile other;
+    for (int t = t0 + wave; t < t1; t += 8) {
+        load_tile(ahead, other);  // of tile t + 4; past the split it reads one line of the pool's start
+        ahead = lookup(t + 8);
+        __builtin_amdgcn_sched_barrier(0);
+        process(next, t);
+        if (t + 4 >= t1) break;
+        load_tile(ahead, next);
+        ahead = lookup(t + 12);
+        __builtin_amdgcn_sched_barrier(0);
+        process(other, t + 4);
     }
 
     if constexpr (FUSED) {
@@ -648,11 +794,13 @@ using namespace ms;
 #define MS_CAT(a, b) MS_CAT2(a, b)
 
 // Attention of a mixed batch.  `work` lists (request index, first flat row) for every block
-// of 64 flat rows; see the file comment.  window = 0 means all keys.
+// of 64 flat rows; see the file comment.  window = 0 means all keys.  max_key_groups = 0 lets the
+// launcher choose how many key groups share a block (1, 2 or 4) from the width of the block tables;
+// a positive value asks for that many (as far as this tile has them).
 extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
     const void* q, const void* kpool, const void* vpool, void* out, const int* block_table, int table_stride,
     const int* seq_q_start, const int* seq_q_len, const int* seq_pos0, const int* work, int n_work, int H, int KV,
-    int hd, int ps, int n_pages, int window, float scale, hipStream_t stream) {
+    int hd, int ps, int n_pages, int window, float scale, int max_key_groups, hipStream_t stream) {
     MS_REQUIRE(n_work > 0, "attention: no work");
     MS_REQUIRE(hd % 16 == 0 && hd > 0 && hd <= HDT, "attention: head size %d does not fit this tile of %d", hd, HDT);
     MS_REQUIRE(KV > 0 && H % KV == 0, "attention: %d heads are not a multiple of %d key/value heads", H, KV);
@@ -661,7 +809,25 @@ extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
     MS_REQUIRE((double)n_pages * KV * ps * hd < 68719476736.0, "attention: a pool of %d pages exceeds 2^36 elements", n_pages);
     AttnArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, (elem_t*)out, block_table, seq_q_start,
                seq_q_len, seq_pos0, work, table_stride, H, KV, hd, ps, window, scale};
-    hipLaunchKernelGGL(paged_attention_kernel, dim3((unsigned)n_work, (unsigned)KV), dim3(256), 0, stream, a);
+    // key groups per block by the longest context the block tables allow (the lengths themselves
+    // are on the device): short contexts have no chain worth cutting
+    const long span = window > 0 ? (long)window + BKV : (long)table_stride * ps;
+    int groups = MAX_KEY_GROUPS;
+    if (max_key_groups > 0) {
+        groups = max_key_groups < MAX_KEY_GROUPS ? max_key_groups : MAX_KEY_GROUPS;
+    } else {
+        if (span < 16 * BKV && groups > 2) groups = 2;
+        if (span < 4 * BKV) groups = 1;
+    }
+    const dim3 grid((unsigned)n_work, (unsigned)KV);
+    if (groups >= 4 && MAX_KEY_GROUPS >= 4) {
+        // sixteen waves leave each 128 registers, which only the small bfloat16 tiles fit into
+        if constexpr (MAX_KEY_GROUPS >= 4) hipLaunchKernelGGL(paged_attention_kernel<4>, grid, dim3(1024), 0, stream, a);
+    } else if (groups >= 2) {
+        hipLaunchKernelGGL(paged_attention_kernel<2>, grid, dim3(512), 0, stream, a);
+    } else {
+        hipLaunchKernelGGL(paged_attention_kernel<1>, grid, dim3(256), 0, stream, a);
+    }
     return check_launch("paged_attention");
 }
 

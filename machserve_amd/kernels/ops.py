@@ -209,7 +209,8 @@ class HipOps:
     def paged_attention(self, q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
                         seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_pos0: torch.Tensor,
                         work: torch.Tensor, H: int, KV: int, hd: int, page_size: int, window: Optional[int],
-                        scale: float) -> torch.Tensor:
+                        scale: float, max_key_groups: int = 0) -> torch.Tensor:
+        """``max_key_groups`` asks for that many groups of waves sharing a block's keys (0: the kernel's choice)."""
         lib, fn = self._attention_lib(hd)[:2]
         T = q.shape[0]
         self._want(q, self.dtype, "attention q", T, H * hd)
@@ -229,7 +230,7 @@ class HipOps:
         self._check(lib, fn(_ptr(q), _ptr(kpool), _ptr(vpool), _ptr(out), _ptr(block_table), _c_int(block_table.shape[1]),
                             _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_pos0), _ptr(work), _c_int(work.shape[0]),
                             _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), _c_int(pages), _c_int(window or 0),
-                            _c_float(scale), _stream()))
+                            _c_float(scale), _c_int(max_key_groups), _stream()))
         return out
 
     DECODE_MAX_GROUP = 16  # query heads per key/value head the decode kernel takes

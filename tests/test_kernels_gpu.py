@@ -164,7 +164,7 @@ def test_rope_kv_write(dtype, H, KV, hd, ps, theta):
     assert_close(vd, vp2, dtype, "value pages from partial sums")
 
 
-def _attention_case(dtype, H, KV, hd, ps, window, seqs, seed, peak=False):
+def _attention_case(dtype, H, KV, hd, ps, window, seqs, seed, peak=False, groups=0):
     """seqs: list of (cached length, rows in this step).  Builds scattered pages holding random
     keys and values for positions < cached + rows and queries for the step's rows."""
     ops, emu = ops_for(dtype), EmulatedOps(dtype)
@@ -197,9 +197,11 @@ def _attention_case(dtype, H, KV, hd, ps, window, seqs, seed, peak=False):
         q[row, head * hd:(head + 1) * hd] = (qv / qv.norm() * 8.0 * math.sqrt(hd) / 4).to(dtype)
     i32 = lambda x: torch.tensor(x, dtype=torch.int32)
     args = (i32(q_start), i32(q_len), i32(pos0), i32(work).view(-1, 2))
+    if groups:
+        emu = EmulatedOps(torch.float32)  # the reference unrounded: the tolerance allows the output's one rounding
     ref = emu.paged_attention(q, kp, vp, table, *args, H, KV, hd, ps, window, hd ** -0.5)
     got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV), table.to(DEV), *[a.to(DEV) for a in args], H, KV, hd,
-                              ps, window, hd ** -0.5)
+                              ps, window, hd ** -0.5, groups)
     return got, ref
 
 
@@ -210,6 +212,18 @@ def test_attention_mixed_batch(dtype, H, KV, hd, ps):
     seqs = [(0, 1), (0, 70), (130, 1), (37, 45), (ps - 1, 2), (ps, 1), (2 * ps - 1, 1)]
     got, ref = _attention_case(dtype, H, KV, hd, ps, None, seqs, 100 + hd)
     assert_close(got, ref, dtype, "attention")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("groups", [1, 2, 4])
+@pytest.mark.parametrize("H,KV,hd,ps,window", [(4, 2, 16, 16, None), (14, 2, 64, 64, None), (6, 3, 128, 32, None),
+                                               (2, 1, 256, 16, None), (6, 2, 64, 16, 100), (3, 1, 48, 32, 333)])
+def test_attention_key_groups(dtype, groups, H, KV, hd, ps, window):
+    """The keys of a block shared by 1, 2 or 4 groups of waves: short and long requests in one
+    launch, lengths that end inside a round of tiles, and a far key that must not be missed."""
+    seqs = [(0, 1), (0, 300), (517, 1), (700, 37), (3, 2), (1023, 1), (64 * groups, 1), (64 * groups - 1, 2)]
+    got, ref = _attention_case(dtype, H, KV, hd, ps, window, seqs, 300 + hd + groups, peak=True, groups=groups)
+    assert_close(got, ref, dtype, f"attention with {groups} key groups")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
