@@ -45,6 +45,58 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, con
     for (int c = threadIdx.x; c < d; c += 256) dst[c] = from_f32<OutT>(vals[c] * inv);
 }
 
+// The same for widths that are a multiple of four and at most 1024 * G.  A thread owns G groups of
+// four consecutive columns (group t, t + 256, ...) and asks for all of the row it needs - stream,
+// weights and the NP pending sums - before it uses the first value, so the kernel pays one memory
+// round trip instead of one per column and pending sum.  The sums are added in the same order.
+template <typename OutT, int G, int NP>
+__global__ __launch_bounds__(256) void rmsnorm_wide_kernel(float* __restrict__ x, const float* __restrict__ partials,
+                                                           size_t partial_stride, const int* __restrict__ rows,
+                                                           const float* __restrict__ w, OutT* __restrict__ out, int d,
+                                                           float eps) {
+    __shared__ float scratch[4];
+    const int i = blockIdx.x, ng = d / 4;
+    const size_t r = rows ? rows[i] : i;
+    f32x4* src = reinterpret_cast<f32x4*>(x + r * d);
+    const f32x4* w4 = reinterpret_cast<const f32x4*>(w);
+    f32x4 v[G], wv[G], pend[NP > 0 ? NP : 1][G];
+    int at[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int c4 = threadIdx.x + g * 256;
+        at[g] = c4 < ng ? c4 : 0;  // a group beyond the row reads group 0 and is dropped
+        v[g] = src[at[g]];
+        wv[g] = w4[at[g]];
+    }
+#pragma unroll
+    for (int p = 0; p < NP; ++p)
+#pragma unroll
+        for (int g = 0; g < G; ++g) pend[p][g] = reinterpret_cast<const f32x4*>(partials + p * partial_stride + r * d)[at[g]];
+    float ss = 0.f;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p) v[g] += pend[p][g];
+        if (threadIdx.x + g * 256 < ng) {
+            if (NP > 0 && !rows) src[at[g]] = v[g];
+            ss += v[g].x * v[g].x + v[g].y * v[g].y + v[g].z * v[g].z + v[g].w * v[g].w;
+        }
+    }
+    ss = block_sum<256>(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+    OutT* dst = out + (size_t)i * d;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        if (threadIdx.x + g * 256 >= ng) continue;
+        const f32x4 o = v[g] * wv[g] * inv;
+        OutT* q = dst + (size_t)at[g] * 4;
+        q[0] = from_f32<OutT>(o.x);
+        q[1] = from_f32<OutT>(o.y);
+        q[2] = from_f32<OutT>(o.z);
+        q[3] = from_f32<OutT>(o.w);
+    }
+}
+
 // x[t, :] += sum_p partials[p, t, :] (in order): pending sums folded in without a norm
 __global__ __launch_bounds__(256) void add_partials_kernel(float* __restrict__ x, const float* __restrict__ partials,
                                                            int n_partials, size_t partial_stride, size_t n) {
@@ -135,7 +187,36 @@ extern "C" int ms_rmsnorm(float* x, const float* partials, int n_partials, int T
     MS_REQUIRE(d * sizeof(float) <= 60000, "rmsnorm: width %d exceeds the row buffer", d);
     MS_REQUIRE(n_partials == 0 || partials, "rmsnorm: %d partial sums without a buffer", n_partials);
     const size_t ps = (size_t)T * d, smem = (size_t)d * sizeof(float);
-    if (out_f32 || !kBf16)
+    const bool f32_out = out_f32 || !kBf16;
+    const int groups = d % 4 == 0 ? (d <= 1024 ? 1 : (d <= 2048 ? 2 : (d <= 4096 ? 4 : 0))) : 0;
+    const bool aligned = (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(partials)) % 16 == 0;
+    if (groups && aligned && n_partials <= 8) {
+#define MS_NORM(OUT_, G_, NP_)                                                                                   \
+    hipLaunchKernelGGL((rmsnorm_wide_kernel<OUT_, G_, NP_>), dim3(n), dim3(256), 0, stream, x, partials, ps, rows, w, \
+                       (OUT_*)out, d, eps)
+#define MS_NORM_NP(OUT_, G_)                                    \
+    switch (n_partials) {                                       \
+        case 0: MS_NORM(OUT_, G_, 0); break;                    \
+        case 1: MS_NORM(OUT_, G_, 1); break;                    \
+        case 2: MS_NORM(OUT_, G_, 2); break;                    \
+        case 3: MS_NORM(OUT_, G_, 3); break;                    \
+        case 4: MS_NORM(OUT_, G_, 4); break;                    \
+        case 5: MS_NORM(OUT_, G_, 5); break;                    \
+        case 6: MS_NORM(OUT_, G_, 6); break;                    \
+        case 7: MS_NORM(OUT_, G_, 7); break;                    \
+        default: MS_NORM(OUT_, G_, 8); break;                   \
+    }
+#define MS_NORM_G(OUT_)                                         \
+    if (groups == 1) { MS_NORM_NP(OUT_, 1) }                    \
+    else if (groups == 2) { MS_NORM_NP(OUT_, 2) }               \
+    else { MS_NORM_NP(OUT_, 4) }
+        if (f32_out) { MS_NORM_G(float) } else { MS_NORM_G(elem_t) }
+#undef MS_NORM_G
+#undef MS_NORM_NP
+#undef MS_NORM
+        return check_launch("rmsnorm");
+    }
+    if (f32_out)
         hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(n), dim3(256), smem, stream, x, partials, n_partials, ps, rows, w,
                            (float*)out, d, eps);
     else

@@ -5,8 +5,10 @@
 // kernels (crates/mach-model/src/kernels.rs:5772-5798, 6416-6455, 131-160).
 //
 // Both operands are contiguous along K, so a 16x32 MFMA fragment of either is "row
-// l % 16, elements (l / 16) * 8 .. + 8": tiles go global -> registers -> LDS (padded rows,
-// conflict-free 16-byte reads) -> fragments.  Two LDS buffers, one barrier per K step.
+// l % 16, elements (l / 16) * 8 .. + 8": tiles go global -> registers -> LDS -> fragments.  LDS has
+// 64 banks of 4 bytes; the 16-byte fragment reads of a wave are free of bank conflicts when the
+// row pitch is 32 modulo 64 bytes (measured: pitches of 80 or 144 bytes take twice as long).
+// Two LDS buffers, one barrier per K step.
 // Every output element is the sum over K in steps of 32 in ascending order whatever the
 // tile shape or the number of rows, so a row's result does not depend on its batch.
 #include "common.cuh"
@@ -15,10 +17,10 @@ namespace ms {
 
 #ifdef MS_ELEM_BF16
 constexpr int EPC = 8;   // elements per 16-byte chunk
-constexpr int KPAD = 8;  // row padding in elements: rows of 80 (BK 32) or 144 (BK 64) bytes
+constexpr int KPAD = 16;  // row padding in elements: rows of 96 (BK 32) or 160 (BK 64) bytes
 #else
 constexpr int EPC = 4;
-constexpr int KPAD = 4;  // rows of 144 bytes (BK 32)
+constexpr int KPAD = 8;  // rows of 160 bytes (BK 32)
 #endif
 
 enum EpiKind { EPI_STORE_F32 = 0, EPI_STORE_ELEM = 1, EPI_RESIDUAL = 2, EPI_SWIGLU = 3 };

@@ -54,61 +54,69 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
         for (int j = 0; j < NT; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     if (n0 < a.N) {
+        // Every load is unconditional, so that all of a slice's fragments are in flight at once and
+        // one wait serves them: a row or column beyond the matrix reads row 0 instead (what it adds
+        // to is never stored), and elements beyond the end of K are read from the last eight of the
+        // row and dropped from A, so that they add nothing whatever W holds there.
         const elem_t* wrow[NT];
-        bool wok[NT];
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
             const int n = n0 + j * 16 + r16;
-            wok[j] = n < a.N;
-            wrow[j] = a.W + (size_t)(wok[j] ? n : 0) * a.K;
+            wrow[j] = a.W + (size_t)(n < a.N ? n : 0) * a.K;
         }
         const elem_t* arow[MT];
-        bool aok[MT];
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             const int m = i * 16 + r16;
-            aok[i] = m < a.M;
-            arow[i] = a.A + (size_t)(aok[i] ? m : 0) * a.K;
+            arow[i] = a.A + (size_t)(m < a.M ? m : 0) * a.K;
         }
-        Frag fw[NT][4], fa[MT][4];
-        auto load = [&](int kk) {
+        // `spread` 0 makes every lane of a row read the same 16 bytes: a load that is only there to
+        // keep the loop's shape (after the last step) then costs one line per row
+        auto load = [&](int kk, int spread, Frag (&fw)[NT][4], Frag (&fa)[MT][4]) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                const int k = kk + (grp * 4 + c) * 8;
-                const bool kok = k < k1;
+                const int k = min(kk + (grp * 4 + c) * 8 * spread, a.K - 8);
 #pragma unroll
-                for (int j = 0; j < NT; ++j) fw[j][c] = (kok && wok[j]) ? frag_load(wrow[j] + k) : frag_zero();
+                for (int j = 0; j < NT; ++j) fw[j][c] = frag_load(wrow[j] + k);
 #pragma unroll
-                for (int i = 0; i < MT; ++i) fa[i][c] = (kok && aok[i]) ? frag_load(arow[i] + k) : frag_zero();
+                for (int i = 0; i < MT; ++i) fa[i][c] = frag_load(arow[i] + k);
             }
         };
+        auto multiply = [&](int kk, Frag (&fw)[NT][4], Frag (&fa)[MT][4]) {
+            if (kk + KSTEP > k1) {  // the slice ends inside this step (the same for the whole wave)
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    if (kk + (grp * 4 + c) * 8 >= k1) {
+#pragma unroll
+                        for (int i = 0; i < MT; ++i) fa[i][c] = frag_zero();
+                    }
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int j = 0; j < NT; ++j) mma_16x16x32(acc[i][j], fa[i][c], fw[j][c]);
+        };
         constexpr bool PREFETCH = MT * NT <= 8;  // a second set of fragments fits the registers
-        if (PREFETCH && k0 < k1) load(k0);
-        for (int kk = k0; kk < k1; kk += KSTEP) {
-            if constexpr (PREFETCH) {
-                Frag cw[NT][4], ca[MT][4];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-#pragma unroll
-                    for (int j = 0; j < NT; ++j) cw[j][c] = fw[j][c];
-#pragma unroll
-                    for (int i = 0; i < MT; ++i) ca[i][c] = fa[i][c];
-                }
-                if (kk + KSTEP < k1) load(kk + KSTEP);  // in flight while this slice is multiplied
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-#pragma unroll
-                    for (int i = 0; i < MT; ++i)
-#pragma unroll
-                        for (int j = 0; j < NT; ++j) mma_16x16x32(acc[i][j], ca[i][c], cw[j][c]);
-            } else {
-                load(kk);
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-#pragma unroll
-                    for (int i = 0; i < MT; ++i)
-#pragma unroll
-                        for (int j = 0; j < NT; ++j) mma_16x16x32(acc[i][j], fa[i][c], fw[j][c]);
+        Frag fw0[NT][4], fa0[MT][4];
+        if (!PREFETCH || k1 - k0 <= KSTEP) {
+            for (int kk = k0; kk < k1; kk += KSTEP) {
+                load(kk, 1, fw0, fa0);
+                multiply(kk, fw0, fa0);
+            }
+        } else {
+            // two sets of fragments take turns: the next step is in flight while this one is multiplied
+            Frag fw1[NT][4], fa1[MT][4];
+            load(k0, 1, fw0, fa0);
+            for (int kk = k0; kk < k1; kk += 2 * KSTEP) {
+                const bool more1 = kk + KSTEP < k1;
+                load(more1 ? kk + KSTEP : k0, more1, fw1, fa1);
+                multiply(kk, fw0, fa0);
+                if (!more1) break;
+                const bool more2 = kk + 2 * KSTEP < k1;
+                load(more2 ? kk + 2 * KSTEP : k0, more2, fw0, fa0);
+                multiply(kk + KSTEP, fw1, fa1);
             }
         }
     }
