@@ -547,11 +547,29 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
         // stage this KV head's share of the row: its g query heads, its key, its value
         float* rowv = &sm_o[0][0][0];
         const int qcol = kvh * g * hd, kcol = a.H * hd + kvh * hd, vcol = (a.H + a.KV) * hd + kvh * hd;
-        for (int c = tid; c < (g + 2) * hd; c += 256) {
-            const int col = c < g * hd ? qcol + c : (c < (g + 1) * hd ? kcol + c - g * hd : vcol + c - (g + 1) * hd);
-            float v = a.bias ? a.bias[col] : 0.f;
-            for (int p = 0; p < a.n_partials; ++p) v += row0[p * pstride + col];
-            rowv[c] = v;
+        // four columns per thread at a time, all of their loads asked for before the first is used
+        const float* bias = a.bias ? a.bias : row0;  // without a bias: finite values, times zero
+        const float bias_on = a.bias ? 1.f : 0.f;
+        const int width = (g + 2) * hd;
+        for (int c0 = tid; c0 < width; c0 += 4 * 256) {
+            int col[4];
+            float v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int c = min(c0 + u * 256, width - 1);
+                col[u] = c < g * hd ? qcol + c : (c < (g + 1) * hd ? kcol + c - g * hd : vcol + c - (g + 1) * hd);
+                v[u] = bias[col[u]] * bias_on;
+            }
+            for (int p = 0; p < a.n_partials; ++p) {
+                float t[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) t[u] = row0[p * pstride + col[u]];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] += t[u];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (c0 + u * 256 < width) rowv[c0 + u * 256] = v[u];
         }
         if (tid < half) {
             float c = 1.f, sv = 0.f;
@@ -762,27 +780,48 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
     }
 }
 
-// out[row, :] = sum_sp o_sp exp(m_sp - m) / sum_sp l_sp exp(m_sp - m), splits in order
+// out[row, :] = sum_sp o_sp exp(m_sp - m) / sum_sp l_sp exp(m_sp - m), splits in order.
+// One wave per (request, head); lane = element of the head (in chunks of 64).  The splits' outputs are
+// asked for eight at a time, the first eight together with the (max, sum) pairs and before anything
+// is computed from those, so that the kernel waits for memory once.
 __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                           elem_t* __restrict__ out, int hd, int nsplit) {
-    __shared__ float coef[MAX_SPLITS];
+    constexpr int BATCH = 8;
     const size_t row = blockIdx.x;  // (request, head)
     const int lane = threadIdx.x;
     const float* ml = part_ml + row * nsplit * 2;
+    const float* po = part_o + row * nsplit * hd;
+    auto fetch = [&](int d, int sp0, float (&v)[BATCH]) {
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) v[u] = po[(size_t)min(sp0 + u, nsplit - 1) * hd + min(d, hd - 1)];
+    };
+    float first[BATCH];
+    fetch(lane, 0, first);
     // every lane holds one split's (max, sum); nsplit <= 64
-    const float m_own = lane < nsplit ? ml[lane * 2] : NEG_BIG;
-    const float l_own = lane < nsplit ? ml[lane * 2 + 1] : 0.f;
+    const int own = min(lane, nsplit - 1);
+    const float m_ld = ml[own * 2], l_ld = ml[own * 2 + 1];
+    const float m_own = lane < nsplit ? m_ld : NEG_BIG;
+    const float l_own = lane < nsplit ? l_ld : 0.f;
     const float m = wave_max(m_own);
     const float c = lane < nsplit ? exp_f(m_own - m) : 0.f;
     float l = 0.f;
     for (int sp = 0; sp < nsplit; ++sp) l += __shfl(l_own * c, sp, WAVE);  // in split order
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    if (lane < nsplit) coef[lane] = c * inv;
-    __syncthreads();
-    for (int d = lane; d < hd; d += 64) {
+    const float coef = c * inv;  // of split `lane`; zero beyond the last split
+    for (int d = lane; d - lane < hd; d += 64) {
         float o = 0.f;
-        for (int sp = 0; sp < nsplit; ++sp) o += part_o[(row * nsplit + sp) * hd + d] * coef[sp];
-        out[row * hd + d] = from_f32<elem_t>(o);
+        for (int sp0 = 0; sp0 < nsplit; sp0 += BATCH) {
+            float v[BATCH];
+            if (d == lane && sp0 == 0) {
+#pragma unroll
+                for (int u = 0; u < BATCH; ++u) v[u] = first[u];
+            } else {
+                fetch(d, sp0, v);
+            }
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u) o += v[u] * __shfl(coef, min(sp0 + u, 63), WAVE);  // zero beyond the last split
+        }
+        if (d < hd) out[row * hd + d] = from_f32<elem_t>(o);
     }
 }
 
