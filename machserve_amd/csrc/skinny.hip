@@ -16,7 +16,8 @@
 
 namespace ms {
 
-constexpr int KSTEP = 128;  // K elements per wave iteration: four fragments per lane, 64 contiguous bytes (bf16)
+constexpr int KSTEP = 128;  // K elements per wave iteration: four fragments per lane; fragment c of the wave is the
+                            // contiguous chunk c of 32 elements (the four key groups side by side: 64 bytes a row in bf16)
 
 enum SkinnyEpi { SK_STORE_F32 = 0, SK_SWIGLU = 1 };
 
@@ -75,7 +76,7 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
         auto load = [&](int kk, int spread, Frag (&fw)[NT][4], Frag (&fa)[MT][4]) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                const int k = min(kk + (grp * 4 + c) * 8 * spread, a.K - 8);
+                const int k = min(kk + (c * 4 + grp) * 8 * spread, a.K - 8);
 #pragma unroll
                 for (int j = 0; j < NT; ++j) fw[j][c] = frag_load(wrow[j] + k);
 #pragma unroll
@@ -86,7 +87,7 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
             if (kk + KSTEP > k1) {  // the slice ends inside this step (the same for the whole wave)
 #pragma unroll
                 for (int c = 0; c < 4; ++c)
-                    if (kk + (grp * 4 + c) * 8 >= k1) {
+                    if (kk + (c * 4 + grp) * 8 >= k1) {
 #pragma unroll
                         for (int i = 0; i < MT; ++i) fa[i][c] = frag_zero();
                     }
@@ -193,11 +194,14 @@ struct SkinnyPlan { int wn, ksi, ksb, k_per_wave; };
 // weigh no more than the weights it streams.
 static int skinny_nt(int M, int N) { return (M > 32 && N >= 4096) ? 4 : 2; }
 
+static int g_force_ksi = 0;  // measurements only: waves along K inside a block (1 = four column waves)
+
 static SkinnyPlan plan_skinny(int M, int N, int K, bool allow_partials) {
     const int NT = skinny_nt(M, N);
     const int col_waves = ceil_div(N, 16 * NT);
     const int slices = ceil_div(K, KSTEP);  // slices of 128 along K: one wave iteration each
     int want = max(1, min(ceil_div(4096, col_waves), slices));  // waves wanted along K
+    if (g_force_ksi > 0) want = min(g_force_ksi, slices);
     SkinnyPlan p;
     if (want == 1) {
         p = {4, 1, 1, slices * KSTEP};
@@ -243,6 +247,8 @@ static int launch_skinny(const SkinnyArgs& a, const SkinnyPlan& p, hipStream_t s
 }  // namespace ms
 
 using namespace ms;
+
+extern "C" void ms_skinny_force_ksi(int ksi) { g_force_ksi = ksi; }
 
 // Number of partial sums ms_linear_skinny writes for M rows of this N and K (1 = the complete product).
 extern "C" int ms_skinny_partials(int M, int N, int K, int allow_partials) { return plan_skinny(M, N, K, allow_partials != 0).ksb; }
