@@ -195,6 +195,7 @@ struct SkinnyPlan { int wn, ksi, ksb, k_per_wave; };
 static int skinny_nt(int M, int N) { return (M > 32 && N >= 4096) ? 4 : 2; }
 
 static int g_force_ksi = 0;  // measurements only: waves along K inside a block (1 = four column waves)
+static int g_max_ksb = 0;    // measurements only: most blocks along K
 
 static SkinnyPlan plan_skinny(int M, int N, int K, bool allow_partials) {
     const int NT = skinny_nt(M, N);
@@ -210,6 +211,7 @@ static SkinnyPlan plan_skinny(int M, int N, int K, bool allow_partials) {
     p.wn = 1;
     p.ksi = want > 4 ? 8 : (want > 2 ? 4 : 2);
     p.ksb = (allow_partials && want > p.ksi) ? ceil_div(want, p.ksi) : 1;
+    if (g_max_ksb > 0) p.ksb = min(p.ksb, g_max_ksb);
     p.k_per_wave = ceil_div(slices, p.ksi * p.ksb) * KSTEP;
     return p;
 }
@@ -249,6 +251,7 @@ static int launch_skinny(const SkinnyArgs& a, const SkinnyPlan& p, hipStream_t s
 using namespace ms;
 
 extern "C" void ms_skinny_force_ksi(int ksi) { g_force_ksi = ksi; }
+extern "C" void ms_skinny_max_ksb(int ksb) { g_max_ksb = ksb; }
 
 // Number of partial sums ms_linear_skinny writes for M rows of this N and K (1 = the complete product).
 extern "C" int ms_skinny_partials(int M, int N, int K, int allow_partials) { return plan_skinny(M, N, K, allow_partials != 0).ksb; }
