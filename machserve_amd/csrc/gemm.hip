@@ -211,11 +211,15 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
 
 // K slices for a product of many rows whose consumer adds partial sums: enough 128x128 blocks to
 // fill the chip, at least 512 of K each.  The 32-bit build never slices: its sums keep one order.
+static int g_force_splits = 0;  // measurements only
+
 static int plan_tiled_splits(int M, int N, int K) {
 #ifdef MS_ELEM_BF16
     const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
-    if (b128 >= 300) return 1;
-    int want = max(1, min((int)ceil_div(300, b128), K / 512));
+    if (b128 >= 300 && g_force_splits == 0) return 1;
+    // about 1.75 blocks a CU; more than six slices cost more in the consumer's sums than they gain here
+    int want = max(1, min(min((int)ceil_div(448, b128), K / 512), 6));
+    if (g_force_splits > 0) want = g_force_splits;
     // what the launcher's rounding of a slice to a multiple of 64 really yields
     const int k_per_split = ceil_div(ceil_div(K, want), 64) * 64;
     return ceil_div(K, k_per_split);
@@ -263,3 +267,4 @@ extern "C" int ms_linear_split_tiled(const void* a, const void* w, float* out, i
 
 // Measurements only: force one tile configuration (0 = choose by shape).
 extern "C" void ms_gemm_force_config(int c) { g_gemm_config = c; }
+extern "C" void ms_gemm_force_splits(int n) { g_force_splits = n; }
