@@ -33,7 +33,9 @@ constexpr int NKS = (HDT + 31) / 32;     // K steps of 32 over the head size
 #ifdef MS_ELEM_BF16
 constexpr int BKV = ND <= 8 ? 64 : 32;
 constexpr int EPC = 8;
-constexpr int KPAD = 8, VPAD = 8;
+// LDS has 64 banks of 4 bytes: the 16-byte reads of K fragments (row l % 16, chunk l / 16) are free of
+// conflicts at a row pitch of 32 modulo 64 bytes, the 8-byte reads of V^T fragments at 16 modulo 32.
+constexpr int KPAD = (ND * 16 * 2) % 64 == 0 ? 16 : 0, VPAD = 8;
 #else
 constexpr int BKV = ND <= 4 ? 64 : (ND <= 8 ? 32 : 16);
 constexpr int EPC = 4;
@@ -433,11 +435,18 @@ struct DecodeArgs {
 };
 
 constexpr int MAX_SPLITS = 64;
+// The decode kernel's key tile: a wave holds two tiles in registers (one being multiplied, one in
+// flight), and smaller tiles leave room for more waves on a CU, which is what keeps memory busy.
+#ifndef MS_DECODE_BKV
+#define MS_DECODE_BKV (BKV >= 32 ? 32 : BKV)
+#endif
+constexpr int DBKV = MS_DECODE_BKV;
+constexpr int DNT = DBKV / 16, DNTP = (DNT + 1) / 2;
 
 // Fragments of one key tile for one lane: keys (K rows) for the scores, V^T groups for the output.
 struct DecodeTile {
-    Frag kf[NT][NKS];
-    Frag vf[NTP][ND];
+    Frag kf[DNT][NKS];
+    Frag vf[DNTP][ND];
 };
 
 template <bool FUSED>
@@ -458,7 +467,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
     const bool valid = r16 < g;
     const int head = kvh * g + (valid ? r16 : 0);
 
-    const int t_lo = lo_key / BKV, t_hi = ceil_div(kv_len, BKV);
+    const int t_lo = lo_key / DBKV, t_hi = ceil_div(kv_len, DBKV);
     const int tps = max(1, ceil_div(t_hi - t_lo, a.nsplit));
     const int t0 = t_lo + sp * tps, t1 = min(t_hi, t0 + tps);
 
@@ -467,7 +476,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
     // covers 32 keys so that the lane of key group `grp` ends up with the probabilities of the eight
     // consecutive keys pp * 32 + grp * 8 ..: its V^T fragment is then one contiguous read.  Row r16 of
     // score tile 2pp + j holds key pp * 32 + (r16 / 4) * 8 + j * 4 + r16 % 4.
-    constexpr bool PAIRED = NT % 2 == 0;
+    constexpr bool PAIRED = DNT % 2 == 0;
     auto k_row = [&](int nt) { return PAIRED ? (nt / 2) * 32 + (r16 >> 2) * 8 + (nt & 1) * 4 + (r16 & 3) : nt * 16 + r16; };
     auto score_key = [&](int nt, int i) { return PAIRED ? (nt / 2) * 32 + grp * 8 + (nt & 1) * 4 + i : nt * 16 + grp * 4 + i; };
     // Loads are unconditional and on one straight path, so that the compiler counts them and a wait
@@ -477,12 +486,12 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
     // adds nothing.  The pages of a tile's 16-key groups are looked up one tile ahead.
     const float inv_gpp = 1.0f / (float)(ps >> 4);  // 1 / (16-key groups per page)
     // of this lane's groups: page as the table has it, -1 if the group is not to be read (else 0), offset in the page
-    struct Pages { int kp[NTP], kx[NTP], ko[NTP], vp[NTP], vx[NTP], vo[NTP]; };
+    struct Pages { int kp[DNTP], kx[DNTP], ko[DNTP], vp[DNTP], vx[DNTP], vo[DNTP]; };
     auto lookup = [&](int t) {
         Pages pg;
-        const int kt0 = t * BKV;
+        const int kt0 = t * DBKV;
 #pragma unroll
-        for (int pp = 0; pp < NTP; ++pp) {
+        for (int pp = 0; pp < DNTP; ++pp) {
             // 16-key groups of this lane: of its K rows of score tiles 2pp and 2pp + 1, and of its V keys
             const int gk = (kt0 >> 4) + (PAIRED ? 2 * pp + (r16 >> 3) : pp), gv = (kt0 >> 4) + (PAIRED ? 2 * pp + (grp >> 1) : pp);
             const int lk = (int)(((float)gk + 0.5f) * inv_gpp), lv = (int)(((float)gv + 0.5f) * inv_gpp);
@@ -502,7 +511,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
     const size_t page_elems = (size_t)ps * hd;
     auto load_tile = [&](const Pages& pg, DecodeTile& td) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
+        for (int nt = 0; nt < DNT; ++nt) {
             // the row of (page, kvh, offset of the row's 16-key group + place in the group) in [pages, KV, ps, hd]
             const int pp = PAIRED ? nt / 2 : nt;
             const int page = pg.kp[pp] | pg.kx[pp], off = pg.ko[pp] + (k_row(nt) & 15);
@@ -514,7 +523,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
             }
         }
 #pragma unroll
-        for (int pp = 0; pp < NTP; ++pp) {
+        for (int pp = 0; pp < DNTP; ++pp) {
             const int page = pg.vp[pp] | pg.vx[pp], off = pg.vo[pp] + (PAIRED ? (grp & 1) * 8 : grp * 4);
             const elem_t* vcol = page >= 0 ? a.vpool + ((size_t)page * a.KV + kvh) * page_elems + off : a.vpool;
 #pragma unroll
@@ -628,17 +637,17 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
     float m_run = NEG_BIG, l_run = 0.f;
 
     auto process = [&](const DecodeTile& cur, int t) {
-        const int kt0 = t * BKV;
-        f32x4 sc[NT];
+        const int kt0 = t * DBKV;
+        f32x4 sc[DNT];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
+        for (int nt = 0; nt < DNT; ++nt) {
             sc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) mma_16x16x32(sc[nt], cur.kf[nt][ks], qf[ks]);
         }
         float tmax = NEG_BIG;
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
+        for (int nt = 0; nt < DNT; ++nt)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int key = kt0 + score_key(nt, i);
@@ -653,7 +662,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
         const float alpha = exp_f(m_run - m_new);
         float psum = 0.f;
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
+        for (int nt = 0; nt < DNT; ++nt)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const float p = exp_f(sc[nt][i] - m_new);
@@ -669,12 +678,12 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc_o[dt][i] *= alpha;
 #pragma unroll
-        for (int pp = 0; pp < NTP; ++pp) {
+        for (int pp = 0; pp < DNTP; ++pp) {
             Frag pf;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 pf.v[i] = from_f32<elem_t>(sc[2 * pp][i]);
-                pf.v[4 + i] = from_f32<elem_t>((2 * pp + 1 < NT) ? sc[(2 * pp + 1) % NT][i] : 0.f);
+                pf.v[4 + i] = from_f32<elem_t>((2 * pp + 1 < DNT) ? sc[(2 * pp + 1) % DNT][i] : 0.f);
             }
 #pragma unroll
             for (int dt = 0; dt < ND; ++dt) mma_16x16x32(acc_o[dt], cur.vf[pp][dt], pf);
@@ -851,12 +860,12 @@ extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
     // key groups per block by the longest context the block tables allow (the lengths themselves
     // are on the device): short contexts have no chain worth cutting
     const long span = window > 0 ? (long)window + BKV : (long)table_stride * ps;
-    int groups = MAX_KEY_GROUPS;
+    // measured at 512 to 8,192 keys: two groups beat one by a quarter, four gain nothing over two
+    int groups = 2;
     if (max_key_groups > 0) {
         groups = max_key_groups < MAX_KEY_GROUPS ? max_key_groups : MAX_KEY_GROUPS;
-    } else {
-        if (span < 16 * BKV && groups > 2) groups = 2;
-        if (span < 4 * BKV) groups = 1;
+    } else if (span < 4 * BKV) {
+        groups = 1;
     }
     const dim3 grid((unsigned)n_work, (unsigned)KV);
     if (groups >= 4 && MAX_KEY_GROUPS >= 4) {
@@ -919,4 +928,4 @@ extern "C" int MS_CAT(ms_decode_attention_fused_nd, MS_ATTN_ND)(
     return check_launch("decode_merge");
 }
 
-extern "C" int MS_CAT(ms_attention_key_tile_nd, MS_ATTN_ND)() { return BKV; }
+extern "C" int MS_CAT(ms_attention_key_tile_nd, MS_ATTN_ND)() { return DBKV; }  // of the decode kernel
