@@ -92,17 +92,27 @@ __device__ __forceinline__ float exp2_f(float x) {
 // index is kg modulo KG, with its own staging buffers, and the groups' running (max, sum, output)
 // are merged through LDS at the end.  A block's time is the length of its serial chain of tiles,
 // and a causal prompt's last rows see every key: more groups cut that chain.
+// Waves per SIMD the compiler has to leave room for: with the small bfloat16 tiles two blocks of a CU
+// overlap one's LDS traffic with the other's arithmetic, if the registers allow them.
+#ifdef MS_ELEM_BF16
+template <int KG> constexpr int attention_waves_per_simd() { return ND <= 4 ? (KG == 1 ? 3 : 4) : 1; }
+#else
+template <int KG> constexpr int attention_waves_per_simd() { return 1; }
+#endif
+
 template <int KG>
-__global__ __launch_bounds__(256 * KG) void paged_attention_kernel(AttnArgs a) {
+__global__ __launch_bounds__(256 * KG, attention_waves_per_simd<KG>()) void paged_attention_kernel(AttnArgs a) {
     constexpr int KS_ELEMS = BKV * K_LD, VS_ELEMS = HDT * V_LD;
     constexpr int STAGE_BYTES = (KS_ELEMS + VS_ELEMS) * (int)sizeof(elem_t);
     constexpr int MERGE_FLOATS = 4 * 64 * (4 * ND + 2);  // per group: four waves, per lane the output and (max, sum)
-    constexpr int SMEM_BYTES = KG * STAGE_BYTES > (KG - 1) * MERGE_FLOATS * 4 ? KG * STAGE_BYTES : (KG - 1) * MERGE_FLOATS * 4;
+    // two stages per group: a tile is multiplied out of one while the next is written into the other
+    constexpr int SMEM_BYTES = 2 * KG * STAGE_BYTES > (KG - 1) * MERGE_FLOATS * 4 ? 2 * KG * STAGE_BYTES : (KG - 1) * MERGE_FLOATS * 4;
+    static_assert(SMEM_BYTES <= 160 * 1024, "the tiles of a block exceed the LDS of a CU");
     __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
 
     const int kg = threadIdx.x >> 8, tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
-    elem_t* Ks = reinterpret_cast<elem_t*>(smem + kg * STAGE_BYTES);
-    elem_t* Vs = Ks + KS_ELEMS;
+    auto stage_k = [&](int b) { return reinterpret_cast<elem_t*>(smem + (2 * kg + b) * STAGE_BYTES); };
+    auto stage_v = [&](int b) { return stage_k(b) + KS_ELEMS; };
     const int r16 = lane & 15, grp = lane >> 4;
     const int s = a.work[blockIdx.x * 2], r0 = a.work[blockIdx.x * 2 + 1];
     const int kvh = blockIdx.y;
@@ -227,22 +237,37 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_kernel(AttnArgs a) {
         }
         live[slot] = bits;
     };
-    auto store_tile = [&](int slot, const u32x4* pk, const u32x4* pv) {
+    auto store_tile = [&](int slot, int b, const u32x4* pk, const u32x4* pv) {
+        elem_t* Ks = stage_k(b);
+        elem_t* Vs = stage_v(b);
         const unsigned bits = live[slot];
-        const bool all = bits == (1u << (NCK + NCV)) - 1;  // nearly always: the masks cost nothing then
+        // nearly always every chunk of every thread was really read: then nothing is masked
+        if (__all(bits == (1u << (NCK + NCV)) - 1)) {
+#pragma unroll
+            for (int i = 0; i < NCK; ++i) {
+                const int c = tid + i * 256;
+                if (c < BKV * CPRK) *reinterpret_cast<u32x4*>(&Ks[(c / CPRK) * K_LD + (c % CPRK) * EPC]) = pk[i];
+            }
+#pragma unroll
+            for (int i = 0; i < NCV; ++i) {
+                const int c = tid + i * 256;
+                if (c < HDT * CPRV) *reinterpret_cast<u32x4*>(&Vs[(c / CPRV) * V_LD + (c % CPRV) * EPC]) = pv[i];
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < NCK; ++i) {
             const int c = tid + i * 256;
-            const unsigned keep = (all || (bits >> i & 1)) ? 0xffffffffu : 0u;
+            const unsigned keep = (bits >> i & 1) ? 0xffffffffu : 0u;
             if (c < BKV * CPRK)
-                *reinterpret_cast<u32x4*>(&Ks[(c / CPRK) * K_LD + (c % CPRK) * EPC]) = all ? pk[i] : pk[i] & (u32x4){keep, keep, keep, keep};
+                *reinterpret_cast<u32x4*>(&Ks[(c / CPRK) * K_LD + (c % CPRK) * EPC]) = pk[i] & (u32x4){keep, keep, keep, keep};
         }
 #pragma unroll
         for (int i = 0; i < NCV; ++i) {
             const int c = tid + i * 256;
-            const unsigned keep = (all || (bits >> (NCK + i) & 1)) ? 0xffffffffu : 0u;
+            const unsigned keep = (bits >> (NCK + i) & 1) ? 0xffffffffu : 0u;
             if (c < HDT * CPRV)
-                *reinterpret_cast<u32x4*>(&Vs[(c / CPRV) * V_LD + (c % CPRV) * EPC]) = all ? pv[i] : pv[i] & (u32x4){keep, keep, keep, keep};
+                *reinterpret_cast<u32x4*>(&Vs[(c / CPRV) * V_LD + (c % CPRV) * EPC]) = pv[i] & (u32x4){keep, keep, keep, keep};
         }
     };
     // rows of this wave: the first and the last position decide which tiles need no mask at all
@@ -250,7 +275,9 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_kernel(AttnArgs a) {
     const int pos_last = pos0 + min(r0 + wave * 16 + 15, max(R - 1, 0)) / g;
     const int lo_last = a.window > 0 ? pos_last - a.window + 1 : 0;
 
-    // round r, slot j: group kg has the tile of absolute index (round_first + r * PF + j) * KG + kg
+    // Round r: group kg has the tile of absolute index round_first * KG + r * KG + kg.  Its loads are
+    // asked for PF rounds ahead into register slot r % PF, it is written into LDS stage r % 2 while
+    // round r - 1 is multiplied out of the other stage, and one barrier a round separates the two.
     const int kt_first = (kv_lo / ROUND) * ROUND;
     start_lookup(kt_first + kg * BKV);
 #pragma unroll
@@ -259,31 +286,44 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_kernel(AttnArgs a) {
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < PF; ++j) load_tile(j, rk[j], rv[j]);
-    for (int kt_base = kt_first; kt_base < kv_hi; kt_base += PF * ROUND) {
+    __syncthreads();  // slot 0's offsets have been read by everyone
+    fill_offsets(0, ahead);  // of round PF, which the first round asks for
+    ahead = lookup();
+    store_tile(0, 0, rk[0], rv[0]);
+    __syncthreads();
+    constexpr int UNROLL = PF > 2 ? PF : 2;
+    for (int kt_base = kt_first; kt_base < kv_hi; kt_base += UNROLL * ROUND) {
 #pragma unroll
-      for (int j = 0; j < PF; ++j) {
-        if (kt_base + j * ROUND >= kv_hi) break;  // the same for every thread of the block
-        const int kt0 = kt_base + j * ROUND + kg * BKV;
-        __syncthreads();  // the previous tiles have been consumed
-        store_tile(j, rk[j], rv[j]);
-        fill_offsets(j, ahead);
-        ahead = lookup();
-        __syncthreads();
-        load_tile(j, rk[j], rv[j]);
-        if (!wave_active || kt0 >= kv_hi) continue;
+      for (int u = 0; u < UNROLL; ++u) {
+        if (kt_base + u * ROUND >= kv_hi) break;  // the same for every thread of the block
+        const int j = u % PF, jn = (u + 1) % PF, b = u & 1;
+        const int kt0 = kt_base + u * ROUND + kg * BKV;
+        const elem_t* Ks = stage_k(b);
+        const elem_t* Vs = stage_v(b);
+        load_tile(j, rk[j], rv[j]);  // round r + PF into the slot that round r left
+        const bool busy = wave_active && kt0 < kv_hi;
 
         // S^T = K Q^T: lane holds keys grp * 4 + i of tile nt for query row r16
         f32x4 sc[NT];
+        if (busy) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            sc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int nt = 0; nt < NT; ++nt) {
+                sc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) {
-                const int d0 = ks * 32 + grp * 8;
-                Frag kf = (d0 < HDT) ? frag_load(&Ks[(nt * 16 + r16) * K_LD + d0]) : frag_zero();
-                mma_16x16x32(sc[nt], kf, qf[ks]);
+                for (int ks = 0; ks < NKS; ++ks) {
+                    const int d0 = ks * 32 + grp * 8;
+                    Frag kf = (d0 < HDT) ? frag_load(&Ks[(nt * 16 + r16) * K_LD + d0]) : frag_zero();
+                    mma_16x16x32(sc[nt], kf, qf[ks]);
+                }
             }
         }
+        // the next round's tile goes into the other stage, which the round before this one has left
+        if (kt_base + (u + 1) * ROUND < kv_hi) {
+            store_tile(jn, b ^ 1, rk[jn], rv[jn]);
+            fill_offsets(jn, ahead);
+            ahead = lookup();
+        }
+        if (busy) {
         // a tile that every row of the wave sees whole needs no mask
         const bool whole = kt0 + BKV - 1 <= pos_first && kt0 >= lo_last;
         float tmax = NEG_BIG;
@@ -356,12 +396,14 @@ __global__ __launch_bounds__(256 * KG) void paged_attention_kernel(AttnArgs a) {
                 mma_16x16x32(acc_o[dt], vf, pf);
             }
         }
+        }
+        __syncthreads();  // this round's stage has been read, the next round's written
       }
     }
 
     if constexpr (KG > 1) {
         // groups 1.. hand (output, max, sum) to group 0 through LDS, which adds them in group order
-        __syncthreads();  // the staging buffers are free
+        // (the rounds end with a barrier: the stages are free)
         float* mg = reinterpret_cast<float*>(smem);
         if (kg > 0) {
             float* mine = mg + ((size_t)(kg - 1) * 4 + wave) * 64 * (4 * ND + 2);
