@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--dtype bf16|f32]
+                    [--shape 0.5b|1.5b|7b] [--batch B] [--context C] [--page-size P]
 
 Default run: Qwen2.5-0.5B layer sizes with random weights (synthetic token ids), 8 requests
 that each hold a 2,048-token context, K decode steps through the whole engine (scheduler,
@@ -30,6 +31,14 @@ QWEN25_05B = {
 }
 
 
+# the two larger configurations of the same architecture (random weights, same distribution)
+QWEN25_15B = dict(QWEN25_05B, hidden_size=1536, num_hidden_layers=28, num_attention_heads=12, num_key_value_heads=2,
+                  intermediate_size=8960)
+QWEN25_7B = dict(QWEN25_05B, hidden_size=3584, num_hidden_layers=28, num_attention_heads=28, num_key_value_heads=4,
+                 intermediate_size=18944, vocab_size=152064, tie_word_embeddings=False)
+SHAPES = {"0.5b": ("Qwen2.5-0.5B", QWEN25_05B), "1.5b": ("Qwen2.5-1.5B", QWEN25_15B), "7b": ("Qwen2.5-7B", QWEN25_7B)}
+
+
 def model_numbers(cfg, elem_bytes):
     d, L, H, KV, hd = cfg.hidden_size, cfg.num_hidden_layers, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
     I, V = cfg.intermediate_size, cfg.vocab_size
@@ -56,6 +65,8 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=2048)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (named in config)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
+    ap.add_argument("--shape", default="0.5b", choices=sorted(SHAPES), help="layer sizes (default: the 0.5B configuration)")
+    ap.add_argument("--page-size", type=int, default=64)
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiles)")
     args = ap.parse_args()
@@ -69,14 +80,15 @@ def main() -> int:
     from machserve_amd.sampling import SamplingParams
     from machserve_amd.weights import random_tensor_dict
 
-    raw = dict(QWEN25_05B)
+    shape_name, shape = SHAPES[args.shape]
+    raw = dict(shape)
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
     cfg = config_from_dict(raw)
     dt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     tensors = random_tensor_dict(cfg, 0, dt, device="cuda:0")
-    ctx, page = args.context, 64
+    ctx, page = args.context, args.page_size
     gen = torch.Generator().manual_seed(1)
 
     def prompts(n, length):
@@ -132,12 +144,12 @@ def main() -> int:
     step_bytes = nums["weight_bytes"] + args.batch * (ctx + args.warmup + args.steps / 2) * nums["kv_bytes_per_token"]
     achieved = step_bytes / (ms * 1e-3) / 1e9
     out = {
-        "metric": "decode tok/s at batch 8, 2048-token contexts (Qwen2.5-0.5B shape)",
+        "metric": f"decode tok/s at batch {args.batch}, {ctx}-token contexts ({shape_name} shape)",
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic: random weights N(0,0.02) seed 0, uniform random token ids",
         "config": {
-            "model": "Qwen2.5-0.5B shape (Qwen2ForCausalLM)", "global_batch": args.batch, "seq_len": ctx,
+            "model": f"{shape_name} shape (Qwen2ForCausalLM)", "global_batch": args.batch, "seq_len": ctx,
             "parallelism": "single GPU", "layers": cfg.num_hidden_layers, "layers_of_configuration": full_layers,
             "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
@@ -155,7 +167,7 @@ def main() -> int:
         b1, _ = decode_run(1)
         b64, _ = decode_run(64)
         out["points"] = {"decode_b1": round(b1, 1), "decode_b64": round(b64, 1)}
-        if args.dtype == "bf16" and cfg.num_hidden_layers == full_layers:
+        if args.dtype == "bf16" and cfg.num_hidden_layers == full_layers and args.shape == "0.5b" and ctx == 2048:
             out["vs_reference"] = {"decode_b64_ctx2048": round(b64 / REF_DECODE_B64_CTX2048, 2),
                                    "prefill_2048": round(ctx / t / REF_PREFILL_2048, 2)}
     print(json.dumps(out))

@@ -259,6 +259,23 @@ extern "C" int ms_linear_swiglu(const void* a, const void* w, void* out, int M, 
 // Number of partial sums ms_linear_split_tiled writes for this problem (1 = the complete product).
 extern "C" int ms_tiled_partials(int M, int N, int K) { return plan_tiled_splits(M, N, K); }
 
+// Whether a product of M rows is better served by the tiled kernel than by the few-rows kernel (which
+// takes at most 64 rows).  The few-rows kernel reads its rows again for every 32 or 64 columns; with
+// many rows and a large weight that traffic outweighs the weight itself, and the tiled kernel, which
+// shares the rows of a block through LDS, streams the weight faster (measured at the 0.5B, 1.5B and 7B
+// layer sizes, 8 to 64 rows).  The choice changes the order of the sums, so results differ in rounding.
+extern "C" int ms_prefers_tiled(int M, int N, int K) {
+    if (M > 64) return 1;
+#ifdef MS_ELEM_BF16
+    if (N < 2048) return 0;
+    const double nk = (double)N * (double)K;
+    if (M >= 8 && nk >= 100e6) return 1;  // a vocabulary-sized product
+    return M >= 16 && nk * M >= 280e6;
+#else
+    return 0;
+#endif
+}
+
 // out[ks, M, N] (float) = partial sums of a w^T over ms_tiled_partials(M, N, K) slices of K.
 extern "C" int ms_linear_split_tiled(const void* a, const void* w, float* out, int M, int N, int K, hipStream_t stream) {
     EpiArgs ep{out, nullptr, N, N, 0, 0};

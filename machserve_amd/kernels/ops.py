@@ -136,12 +136,18 @@ class HipOps:
 
     SKINNY_ROWS = 64  # at most this many rows: the weight-streaming kernels
 
+    def _tiled(self, M: int, N: int, K: int) -> bool:
+        """Whether the tiled kernel takes this product (always above SKINNY_ROWS rows; below, when the
+        weight is large enough that the few-rows kernel's repeated reads of the rows cost more)."""
+        return M > self.SKINNY_ROWS or bool(self._core.ms_prefers_tiled(_c_int(M), _c_int(N), _c_int(K)))
+
     def linear_split(self, a: torch.Tensor, w: torch.Tensor, allow_partials: bool = True) -> torch.Tensor:
-        """Float32 ``[P, M, N]`` whose sum over P is ``a @ w.T``.  P depends on N and K only (1 for
-        more than 64 rows), so the consumer that adds the parts sees the same sums for a row
-        whatever else is in the batch."""
+        """Float32 ``[P, M, N]`` whose sum over P is ``a @ w.T``.  Within one kernel family the cut
+        of K depends on N and K only, so the consumer that adds the parts sees the same sums for a row
+        whatever else is in the batch; which family runs depends on the number of rows (see
+        :meth:`_tiled`), and the two differ in rounding."""
         M, N, K = self._mm_operands(a, w, "linear_split")
-        if M > self.SKINNY_ROWS:
+        if self._tiled(M, N, K):
             P = self._core.ms_tiled_partials(_c_int(M), _c_int(N), _c_int(K)) if allow_partials else 1
             if P == 1:
                 return self.linear(a, w, None, out_f32=True).unsqueeze(0)
@@ -159,7 +165,7 @@ class HipOps:
                out_f32: bool = False) -> torch.Tensor:
         """``a @ w.T (+ bias)``; 32-bit output on request (logits)."""
         M, N, K = self._mm_operands(a, w, "linear")
-        if M <= self.SKINNY_ROWS and out_f32 and bias is None:
+        if not self._tiled(M, N, K) and out_f32 and bias is None:
             return self.linear_split(a, w, allow_partials=False)[0]
         if bias is not None:
             self._want(bias, torch.float32, "linear bias", N)
@@ -174,7 +180,7 @@ class HipOps:
         ``[P, M, N]`` are returned for the consumer (the next norm) to fold in; otherwise None."""
         M, N, K = self._mm_operands(a, w, "linear_residual")
         self._want(x, torch.float32, "residual stream", M, N)
-        if M <= self.SKINNY_ROWS or self._core.ms_tiled_partials(_c_int(M), _c_int(N), _c_int(K)) > 1:
+        if not self._tiled(M, N, K) or self._core.ms_tiled_partials(_c_int(M), _c_int(N), _c_int(K)) > 1:
             return self.linear_split(a, w)
         self._check(self._core, self._core.ms_linear_residual(_ptr(a), _ptr(w), _ptr(x), _c_int(M), _c_int(N), _c_int(K),
                                                               _stream()))
@@ -187,7 +193,7 @@ class HipOps:
         if N != 2 * ((intermediate + 15) // 16) * 16:
             raise KernelError(f"linear_swiglu: interleaved weight has {N} rows for intermediate size {intermediate}")
         out = torch.empty((M, intermediate), dtype=self.dtype, device=a.device)
-        fn = self._core.ms_linear_swiglu_skinny if M <= self.SKINNY_ROWS else self._core.ms_linear_swiglu
+        fn = self._core.ms_linear_swiglu if self._tiled(M, N, K) else self._core.ms_linear_swiglu_skinny
         self._check(self._core, fn(_ptr(a), _ptr(w_gate_up), _ptr(out), _c_int(M), _c_int(intermediate), _c_int(K),
                                    _stream()))
         return out
