@@ -43,8 +43,10 @@ def test_real_layer_sizes(name, dtype):
     lm = load_model(config=cfg, tensors=tensors, dtype=dtype, device=DEV, page_size=64, num_pages=5, max_requests=2)
     sa, sb = lm.cache.admit(), lm.cache.admit()
     got_a, got_b = [], []
-    # a: a long portion, then portions beside b's prompt, then both decode side by side
-    got_a.append(lm.step([StepEntry(sa, a[:100], list(range(100)))]))
+    # a: a long portion, a short one, then portions beside b's prompt, then both decode side by side
+    got_a.append(lm.step([StepEntry(sa, a[:80], list(range(80)))]))
+    # twenty rows: few enough for the few-rows kernels, but the large products go to the tiled kernel
+    got_a.append(lm.step([StepEntry(sa, a[80:100], list(range(20)))]))
     out = lm.step([StepEntry(sa, a[100:130], list(range(30))), StepEntry(sb, b[:66], list(range(66)))])
     got_a.append(out[:30]), got_b.append(out[30:])
     out = lm.step([StepEntry(sa, a[130:132], [0, 1]), StepEntry(sb, b[66:67], [0])])
