@@ -305,3 +305,85 @@ def test_attention_part_alone(dtype, window, shared):
     ref = P.attention_block(h.float(), w, "p.", torch.arange(T), sizes, window)
     for o in outs:
         assert_close(o, ref, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_block_arrangement_alone(dtype):
+    """The pre-norm arrangement around the stream, built from the registries with parts of its own
+    sizes: x += mixer(norm(x)); x += feed_forward(norm(x))
+    (crates/mach-model/src/batched.rs:3180-3200).  A portion and single tokens against the plain parts."""
+    from machserve_amd.cache import CacheManager, DeviceCache
+    from machserve_amd.config import AttentionSpec, GatedMlpSpec, NormSpec, RotarySpec
+    from machserve_amd.engine.step import StepEntry, StepFunction
+    from machserve_amd.parts import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, ResidualStream
+    rt = _runtime(dtype)
+    H, KV, hd, d, I, T, eps = 3, 1, 48, 112, 136, 40, 1e-5
+    names = {k: k for k in ("q.weight", "k.weight", "v.weight", "o.weight", "q.bias", "k.bias", "v.bias")}
+    mixer = MIXERS.build(AttentionSpec("attention", d, H, KV, hd, RotarySpec("rotary", hd, 5e4), tensors=names), rt)
+    ff = FEED_FORWARDS.build(GatedMlpSpec("gated_mlp", d, I), rt)
+    n1, n2 = NORMS.build(NormSpec("rmsnorm", d, eps), rt), NORMS.build(NormSpec("rmsnorm", d, eps), rt)
+    block = BLOCKS.get("prenorm")(mixer, ff, n1, n2)
+    assert block.parts() == [n1, mixer, n2, ff]
+    g = torch.Generator().manual_seed(11)
+    r = lambda *s: torch.randn(*s, generator=g) * 0.1
+    t = {"q.weight": r(H * hd, d), "k.weight": r(KV * hd, d), "v.weight": r(KV * hd, d), "o.weight": r(d, H * hd),
+         "q.bias": r(H * hd), "k.bias": None, "v.bias": r(KV * hd),
+         "gate.weight": r(I, d), "up.weight": r(I, d), "down.weight": r(d, I), "n1": 1 + r(d), "n2": 1 + r(d)}
+    t = {k: (v.to(dtype) if v is not None and v.dim() == 2 else v) for k, v in t.items()}
+    dev = {k: (v.to(DEV) if v is not None else None) for k, v in t.items()}
+    mixer.load(dev), ff.load(dev), n1.load({"weight": dev["n1"]}), n2.load({"weight": dev["n2"]})
+    cache = CacheManager([mixer.cache_request()], 16, 4, 1)
+    dc = DeviceCache(cache, dtype, rt.device)
+    mixer.bind_cache(dc.binding(0))
+
+    class OneLayer:
+        vocab = 100
+        class spec:
+            max_positions = 1000
+        def attention_rows_per_token(self):
+            return [H // KV]
+    sf = StepFunction(OneLayer(), cache, rt)
+    x = torch.randn(T, d, generator=g)
+    slot = cache.admit()
+    out = torch.zeros(T, d)
+    i = 0
+    for c in [17, 1, 2, 1, 19]:
+        cache.extend(slot, c)
+        ctx = sf.build_context([StepEntry(slot, [0] * c, [])])
+        stream = ResidualStream(x[i:i + c].to(DEV).clone(), rt.ops)
+        block.forward(stream, ctx)
+        out[i:i + c] = stream.value().cpu()
+        cache.commit(slot, c)
+        i += c
+    f = {k: (v.float() if v is not None else None) for k, v in t.items()}
+    w = {"p.q_proj.weight": f["q.weight"], "p.k_proj.weight": f["k.weight"], "p.v_proj.weight": f["v.weight"],
+         "p.o_proj.weight": f["o.weight"], "p.q_proj.bias": f["q.bias"], "p.v_proj.bias": f["v.bias"]}
+    sizes = {"heads": H, "kv_heads": KV, "head_dim": hd, "theta": 5e4}
+    y = x + P.attention_block(P.rms_norm(x, f["n1"], eps), w, "p.", torch.arange(T), sizes)
+    y = y + P.swiglu(P.rms_norm(y, f["n2"], eps), f["gate.weight"], f["up.weight"], f["down.weight"])
+    assert_close(out, y, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("tied", [True, False, None])
+def test_embedding_and_head_parts_alone(dtype, tied):
+    """Rows of the table in 32-bit, and logits from the head tensor or, tied, from the table
+    (crates/mach-model/src/loader.rs:1025-1033); a vocabulary and a width that are no powers of two."""
+    from machserve_amd.config import EmbeddingSpec, HeadSpec
+    from machserve_amd.parts.model import Embedding, Head
+    rt = _runtime(dtype)
+    V, d = 333, 88
+    table, head_w = (torch.randn(V, d) * 0.3).to(dtype), (torch.randn(V, d) * 0.3).to(dtype)
+    emb = Embedding(EmbeddingSpec(V, d), rt)
+    emb.load({"weight": table.to(DEV)})
+    head = Head(HeadSpec(V, d, tied), rt, emb)
+    assert [dd.name for dd in head.tensor_decls()] == ([] if tied is True else ["weight"])
+    head.load({"weight": head_w.to(DEV)} if tied is False else {"weight": None} if tied is None else {})
+    toks = torch.tensor([0, 332, 17, 17, 200], dtype=torch.int32)
+    x = emb.forward(toks.to(DEV))
+    assert x.dtype == torch.float32 and torch.equal(x.cpu(), table.float()[toks.long()])
+    h = (torch.randn(5, d)).to(dtype)
+    logits = head.forward(h.to(DEV))
+    used = head_w if tied is False else table
+    assert logits.dtype == torch.float32
+    assert_close(logits, P.linear(h.float(), used.float()), dtype)
