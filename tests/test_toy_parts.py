@@ -1,7 +1,8 @@
-"""Generality of the parts: a toy mixer with state of its own, a toy position encoding and a
-toy architecture are defined *here*, registered, built and stepped without a change to the
-framework's files.  The toy model mixes kinds of layers, runs one layer twice and lets one
-layer read another layer's cache.  It is nobody's model."""
+"""Generality of the parts: a toy mixer with state of its own, a toy feed-forward that routes
+each row to one of a few experts, a toy position encoding and a toy architecture are defined
+*here*, registered, built and stepped without a change to the framework's files.  The toy model
+mixes kinds of layers, runs one layer twice and lets one layer read another layer's cache.  It
+is nobody's model."""
 from dataclasses import dataclass, field
 from typing import Mapping
 
@@ -13,10 +14,11 @@ from plain import qwen2_plain as P
 
 from machserve_amd.config import (AttentionSpec, EmbeddingSpec, GatedMlpSpec, HeadSpec, LayerSpec, ModelSpec, NormSpec,
                                   RotarySpec, register_architecture)
-from machserve_amd.parts import (Mixer, PositionEncoding, StateRequest, TensorDecl, register_mixer,
-                                 register_position_encoding)
+from machserve_amd.parts import (FeedForward, Mixer, PositionEncoding, StateRequest, TensorDecl, register_feed_forward,
+                                 register_mixer, register_position_encoding)
 
 WIDTH, HEADS, KV, HD, INTER, VOCAB = 48, 3, 1, 16, 80, 90
+EXPERTS, EXPERT_INTER = 3, 24
 
 
 @dataclass(frozen=True)
@@ -54,6 +56,38 @@ class RunningMean(Mixer):
         stream.add(out @ self.w.float().t())
 
 
+@dataclass(frozen=True)
+class RoutedSpec:
+    kind: str
+    width: int
+    experts: int
+    inter: int
+    tensors: Mapping[str, str] = field(default_factory=dict)
+
+
+@register_feed_forward("toy_routed")
+class Routed(FeedForward):
+    """Every row goes to the one expert its router logit (32-bit) is largest for; an expert is
+    w2 relu(w1 h).  The router and the experts are the part's own business."""
+
+    def tensor_decls(self):
+        sp = self.spec
+        return [TensorDecl("router", (sp.experts, sp.width), "vector"), TensorDecl("w1", (sp.experts, sp.inter, sp.width)),
+                TensorDecl("w2", (sp.experts, sp.width, sp.inter))]
+
+    def load(self, t):
+        self.router, self.w1, self.w2 = t["router"], t["w1"], t["w2"]
+
+    def forward(self, h, stream, ctx):
+        x = h.float()
+        choice = (x @ self.router.float().t()).argmax(-1)
+        out = torch.zeros_like(x)
+        for e in range(self.spec.experts):
+            rows = choice == e
+            out[rows] = torch.relu(x[rows] @ self.w1[e].float().t()) @ self.w2[e].float().t()
+        stream.add(out)
+
+
 @register_position_encoding("toy_position_scale")
 class PositionScale(PositionEncoding):
     """q and k of the row at position p are multiplied by 1 + p / 64: not a rotation, so the
@@ -85,6 +119,8 @@ class ToyConfig:
 
         def layer(i, mixer):
             ff = GatedMlpSpec("gated_mlp", WIDTH, INTER, "silu", {k: f"l{i}.ff.{k}" for k in ("gate.weight", "up.weight", "down.weight")})
+            if i == 2:
+                ff = RoutedSpec("toy_routed", WIDTH, EXPERTS, EXPERT_INTER, {k: f"l2.moe.{k}" for k in ("router", "w1", "w2")})
             return LayerSpec("prenorm", mixer, ff, norm(f"l{i}.n1"), norm(f"l{i}.n2"))
 
         layers = [
@@ -103,10 +139,12 @@ register_architecture("ToyForCausalLM", ToyConfig)
 def toy_tensors(seed=0):
     g = torch.Generator().manual_seed(seed)
     r = lambda *s: torch.randn(*s, generator=g) * 0.2
-    t = {"emb": r(VOCAB, WIDTH), "nf": 1 + r(WIDTH) * 0.2, "l1.mean.w": r(WIDTH, WIDTH)}
+    t = {"emb": r(VOCAB, WIDTH), "nf": 1 + r(WIDTH) * 0.2, "l1.mean.w": r(WIDTH, WIDTH),
+         "l2.moe.router": r(EXPERTS, WIDTH) * 5, "l2.moe.w1": r(EXPERTS, EXPERT_INTER, WIDTH), "l2.moe.w2": r(EXPERTS, WIDTH, EXPERT_INTER)}
     for i in range(4):
         t[f"l{i}.n1"], t[f"l{i}.n2"] = 1 + r(WIDTH) * 0.2, 1 + r(WIDTH) * 0.2
-        t[f"l{i}.ff.gate.weight"], t[f"l{i}.ff.up.weight"], t[f"l{i}.ff.down.weight"] = r(INTER, WIDTH), r(INTER, WIDTH), r(WIDTH, INTER)
+        if i != 2:  # layer 2 has the routed feed-forward
+            t[f"l{i}.ff.gate.weight"], t[f"l{i}.ff.up.weight"], t[f"l{i}.ff.down.weight"] = r(INTER, WIDTH), r(INTER, WIDTH), r(WIDTH, INTER)
     for i in (0, 2, 3):
         t[f"l{i}.att.q.weight"], t[f"l{i}.att.o.weight"], t[f"l{i}.att.q.bias"] = r(HEADS * HD, WIDTH), r(WIDTH, HEADS * HD), r(HEADS * HD)
         if i != 3:
@@ -149,6 +187,11 @@ def plain_toy(t, toks):
         else:
             x = x + attention(i, xn, "rotary" if i != 2 else "scale")
         xn = P.rms_norm(x, t[f"l{i}.n2"], 1e-5)
+        if i == 2:  # one expert a row
+            choice = (xn @ t["l2.moe.router"].t()).argmax(-1)
+            y = torch.stack([torch.relu(t["l2.moe.w1"][e] @ row) for row, e in zip(xn, choice)])
+            x = x + torch.stack([t["l2.moe.w2"][e] @ row for row, e in zip(y, choice)])
+            continue
         x = x + P.swiglu(xn, t[f"l{i}.ff.gate.weight"], t[f"l{i}.ff.up.weight"], t[f"l{i}.ff.down.weight"])
     return P.linear(P.rms_norm(x, t["nf"], 1e-5), t["emb"])
 
