@@ -19,12 +19,12 @@ namespace ms {
 constexpr int KSTEP = 128;  // K elements per wave iteration: four fragments per lane; fragment c of the wave is the
                             // contiguous chunk c of 32 elements (the four key groups side by side: 64 bytes a row in bf16)
 
-enum SkinnyEpi { SK_STORE_F32 = 0, SK_SWIGLU = 1 };
+enum SkinnyEpi { SK_STORE_F32 = 0, SK_SWIGLU = 1, SK_RESIDUAL = 2 };
 
 struct SkinnyArgs {
     const elem_t* A;  // [M, K]
     const elem_t* W;  // [N, K]
-    void* out;        // SK_STORE_F32: float [gridDim.y, M, N]; SK_SWIGLU: elem [M, n_out]
+    void* out;        // SK_STORE_F32: float [gridDim.y, M, N]; SK_SWIGLU: elem [M, n_out]; SK_RESIDUAL: float [M, N], added to
     int M, N, K;
     int k_per_wave;   // multiple of 32
     int n_out;        // SK_SWIGLU: intermediate size
@@ -54,6 +54,21 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
 #pragma unroll
         for (int j = 0; j < NT; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
+    // SK_RESIDUAL: the stream's values are asked for now, with everything else, not after the sums
+    constexpr bool PRIOR_EARLY = EPI == SK_RESIDUAL && MT <= 2;  // with more row tiles the registers are needed elsewhere
+    float prior[PRIOR_EARLY ? MT : 1][NT][4];
+    if constexpr (PRIOR_EARLY) {
+        const float* xs = reinterpret_cast<const float*>(a.out);
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int row = min(i * 16 + grp * 4 + e, a.M - 1), col = min(n0 + j * 16 + r16, a.N - 1);
+                    prior[i][j][e] = xs[(size_t)row * a.N + col];
+                }
+    }
     if (n0 < a.N) {
         // Every load is unconditional, so that all of a slice's fragments are in flight at once and
         // one wait serves them: a row or column beyond the matrix reads row 0 instead (what it adds
@@ -99,7 +114,9 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
 #pragma unroll
                     for (int j = 0; j < NT; ++j) mma_16x16x32(acc[i][j], fa[i][c], fw[j][c]);
         };
-        constexpr bool PREFETCH = MT * NT <= 8;  // a second set of fragments fits the registers
+        // a second set of fragments, if it fits the registers of a wave in a block of eight
+        constexpr int FRAG_REGS = (int)sizeof(Frag) / 4;
+        constexpr bool PREFETCH = 2 * (MT + NT) * 4 * FRAG_REGS + MT * NT * 4 <= 176;
         Frag fw0[NT][4], fa0[MT][4];
         if (!PREFETCH || k1 - k0 <= KSTEP) {
             for (int kk = k0; kk < k1; kk += KSTEP) {
@@ -168,6 +185,7 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
             }
     } else {
         if (owner) {
+            // SK_RESIDUAL: all of K lies in this block (gridDim.y == 1), so every element has one writer
             float* out = reinterpret_cast<float*>(a.out) + (size_t)blockIdx.y * a.M * a.N;
 #pragma unroll
             for (int i = 0; i < MT; ++i)
@@ -178,9 +196,162 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const int row = i * 16 + grp * 4 + e;
-                        if (row < a.M) out[(size_t)row * a.N + col] = acc[i][j][e];
+                        if (row >= a.M) continue;
+                        if constexpr (PRIOR_EARLY) out[(size_t)row * a.N + col] = prior[i][j][e] + acc[i][j][e];
+                        else if constexpr (EPI == SK_RESIDUAL) out[(size_t)row * a.N + col] += acc[i][j][e];
+                        else out[(size_t)row * a.N + col] = acc[i][j][e];
                     }
                 }
+        }
+    }
+}
+
+// The same product for at most 16 rows with the RMS norm of the residual stream folded in:
+//   v = x + sum_p partials[p] (in order);  out = ((v * norm_w) W^T) / sqrt(mean(v^2) + eps).
+// The norm's factor is one number a row, so it is applied to the finished sums instead of to the
+// rows: a wave builds its A fragments from v * norm_w (rounded to the element type as a norm kernel's
+// output would be), sums v^2 over its slice of K, and the slices' sums of squares ride along with
+// the reduction of the products through LDS.  The whole of K lies inside one block.  The blocks of
+// the first columns also write v to x_out (another buffer than x, which other blocks still read):
+// the stream with its pending sums added.  This saves the norm's own launch, a memory round trip
+// on the critical path of a decode step.
+struct SkinnyNormArgs {
+    const float* x;         // [M, K] residual stream
+    const float* partials;  // [NP, M, K] pending sums
+    size_t partial_stride;
+    const float* norm_w;    // [K]
+    float* x_out;           // [M, K] or null (nothing pending)
+    const elem_t* W;        // [N, K]
+    void* out;              // SK_STORE_F32: float [M, N]; SK_SWIGLU: elem [M, n_out]
+    int M, N, K, k_per_wave, n_out;
+    float eps;
+};
+
+template <int NT, int KSI, int EPI, int NP>
+__global__ __launch_bounds__(64 * KSI) void gemm_skinny_norm_kernel(SkinnyNormArgs a) {
+    static_assert(KSI > 1, "the slices of K are waves of one block");
+    __shared__ float red[(KSI - 1) * NT * 4 * 64];
+    __shared__ float ss_part[KSI][16];
+    const int lane = threadIdx.x & 63, wk = threadIdx.x >> 6;
+    const int r16 = lane & 15, grp = lane >> 4;
+    const int n0 = blockIdx.x * 16 * NT;
+    const int k0 = wk * a.k_per_wave, k1 = min(a.K, k0 + a.k_per_wave);
+    const bool row_on = r16 < a.M;
+    const size_t row = row_on ? r16 : 0;
+    const float* xrow = a.x + row * a.K;
+    const float* prow = a.partials + row * a.K;
+    float* orow = a.x_out + row * a.K;
+    const bool writer = blockIdx.x == 0 && a.x_out != nullptr && row_on;
+    const elem_t* wrow[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int n = n0 + j * 16 + r16;
+        wrow[j] = a.W + (size_t)(n < a.N ? n : 0) * a.K;
+    }
+    f32x4 acc[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) acc[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float ss = 0.f;
+    for (int kk = k0; kk < k1; kk += KSTEP) {
+        // Every load first (unconditional, clamped as in the plain kernel), then the sums.  With many
+        // pending sums the registers hold only half a step's loads at a time.
+        constexpr int HALVES = NP >= 3 ? 2 : 1, CPH = 4 / HALVES;
+#pragma unroll
+        for (int half = 0; half < HALVES; ++half) {
+            Frag fw[NT][CPH];
+            f32x4 xv[CPH][2], wn[CPH][2], pv[NP > 0 ? NP : 1][CPH][2];
+#pragma unroll
+            for (int cc = 0; cc < CPH; ++cc) {
+                const int c = half * CPH + cc;
+                const int k = min(kk + (c * 4 + grp) * 8, a.K - 8);
+#pragma unroll
+                for (int j = 0; j < NT; ++j) fw[j][cc] = frag_load(wrow[j] + k);
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    xv[cc][h] = *reinterpret_cast<const f32x4*>(xrow + k + 4 * h);
+                    wn[cc][h] = *reinterpret_cast<const f32x4*>(a.norm_w + k + 4 * h);
+#pragma unroll
+                    for (int p = 0; p < NP; ++p)
+                        pv[p][cc][h] = *reinterpret_cast<const f32x4*>(prow + p * a.partial_stride + k + 4 * h);
+                }
+            }
+#pragma unroll
+            for (int cc = 0; cc < CPH; ++cc) {
+                const int k = kk + ((half * CPH + cc) * 4 + grp) * 8;
+                const bool on = k < k1;  // beyond the slice: nothing (K is a multiple of 8, so a chunk is in or out)
+                Frag fa;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    f32x4 v = xv[cc][h];
+#pragma unroll
+                    for (int p = 0; p < NP; ++p) v += pv[p][cc][h];
+                    if (!on) v = (f32x4){0.f, 0.f, 0.f, 0.f};
+                    if (writer && on && NP > 0) *reinterpret_cast<f32x4*>(orow + k + 4 * h) = v;
+                    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+                    const f32x4 t = v * wn[cc][h];
+                    fa.v[4 * h + 0] = from_f32<elem_t>(t.x);
+                    fa.v[4 * h + 1] = from_f32<elem_t>(t.y);
+                    fa.v[4 * h + 2] = from_f32<elem_t>(t.z);
+                    fa.v[4 * h + 3] = from_f32<elem_t>(t.w);
+                }
+#pragma unroll
+                for (int j = 0; j < NT; ++j) mma_16x16x32(acc[j], fa, fw[j][cc]);
+            }
+        }
+    }
+    // the row's sum of squares over this wave's slice: the four key groups of a row, then the slices
+    ss += __shfl_xor(ss, 16, WAVE);
+    ss += __shfl_xor(ss, 32, WAVE);
+    if (grp == 0) ss_part[wk][r16] = ss;
+    if (wk > 0) {
+        float* dst = red + ((size_t)(wk - 1) * NT * 4) * 64;
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dst[(j * 4 + e) * 64 + lane] = acc[j][e];
+    }
+    __syncthreads();
+    if (wk > 0 || n0 >= a.N) return;
+#pragma unroll
+    for (int s = 1; s < KSI; ++s) {
+        const float* src = red + ((size_t)(s - 1) * NT * 4) * 64;
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[j][e] += src[(j * 4 + e) * 64 + lane];
+    }
+    float total = 0.f;
+#pragma unroll
+    for (int s = 0; s < KSI; ++s) total += ss_part[s][r16];  // in slice order
+    const float inv_own = 1.0f / sqrtf(total / (float)a.K + a.eps);  // of row r16
+    float inv[4];  // of the rows this lane holds: grp * 4 + e
+#pragma unroll
+    for (int e = 0; e < 4; ++e) inv[e] = __shfl(inv_own, grp * 4 + e, WAVE);
+
+    if constexpr (EPI == SK_SWIGLU) {
+        static_assert(NT % 2 == 0, "gate and up tiles come in pairs");
+        elem_t* out = reinterpret_cast<elem_t*>(a.out);
+#pragma unroll
+        for (int j = 0; j < NT; j += 2) {
+            const int col = (n0 + j * 16) / 2 + r16;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int r = grp * 4 + e;
+                if (r < a.M && col < a.n_out)
+                    out[(size_t)r * a.n_out + col] = from_f32<elem_t>(silu_sk(acc[j][e] * inv[e]) * (acc[j + 1][e] * inv[e]));
+            }
+        }
+    } else {
+        float* out = reinterpret_cast<float*>(a.out);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const int col = n0 + j * 16 + r16;
+            if (col >= a.N) continue;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int r = grp * 4 + e;
+                if (r < a.M) out[(size_t)r * a.N + col] = acc[j][e] * inv[e];
+            }
         }
     }
 }
@@ -192,7 +363,7 @@ struct SkinnyPlan { int wn, ksi, ksb, k_per_wave; };
 // Columns per wave in units of 16: with more than 32 rows and enough columns to keep every CU busy,
 // a wave takes 64 columns, so that the rows it re-reads (from L2, they are shared by all waves)
 // weigh no more than the weights it streams.
-static int skinny_nt(int M, int N) { return (M > 32 && N >= 4096) ? 4 : 2; }
+static int skinny_nt(int M, int N) { return (kBf16 && M > 32 && N >= 4096) ? 4 : 2; }  // 32-bit fragments are twice as large
 
 static int g_force_ksi = 0;  // measurements only: waves along K inside a block (1 = four column waves)
 static int g_max_ksb = 0;    // measurements only: most blocks along K
@@ -238,12 +409,56 @@ static int launch_skinny(const SkinnyArgs& a, const SkinnyPlan& p, hipStream_t s
     MS_REQUIRE(a.K % 8 == 0, "skinny product: the reduction size K=%d must be a multiple of 8", a.K);
     if (a.M <= 16) return launch_skinny_mt<1, 2, EPI>(a, p, stream);
     if (a.M <= 32) return launch_skinny_mt<2, 2, EPI>(a, p, stream);
-    if (skinny_nt(a.M, a.N) == 4) {
-        if (a.M <= 48) return launch_skinny_mt<3, 4, EPI>(a, p, stream);
-        return launch_skinny_mt<4, 4, EPI>(a, p, stream);
+    if constexpr (kBf16) {
+        if (skinny_nt(a.M, a.N) == 4) {
+            if (a.M <= 48) return launch_skinny_mt<3, 4, EPI>(a, p, stream);
+            return launch_skinny_mt<4, 4, EPI>(a, p, stream);
+        }
     }
     if (a.M <= 48) return launch_skinny_mt<3, 2, EPI>(a, p, stream);
     return launch_skinny_mt<4, 2, EPI>(a, p, stream);
+}
+
+
+// Waves along K for the product with the norm folded in (all of K inside a block), or 0 if this
+// shape is not taken: more than 16 rows, so few columns that one wave would do all of K, or more
+// pending sums than the kernel has variants for.
+static int plan_skinny_norm(int M, int N, int K, int n_partials) {
+    if (M > 16 || n_partials > 6 || K % 8) return 0;
+    const int col_waves = ceil_div(N, 32);
+    const int slices = ceil_div(K, KSTEP);
+    const int want = max(1, min(ceil_div(4096, col_waves), slices));
+    if (want == 1) return 0;
+    return want > 4 ? 8 : (want > 2 ? 4 : 2);
+}
+
+template <int EPI>
+static int launch_skinny_norm(SkinnyNormArgs a, int n_partials, hipStream_t stream) {
+    const int ksi = plan_skinny_norm(a.M, a.N, a.K, n_partials);
+    MS_REQUIRE(ksi > 0, "product with the norm folded in: M=%d N=%d K=%d with %d pending sums is not taken", a.M, a.N, a.K, n_partials);
+    MS_REQUIRE(((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.partials) | reinterpret_cast<uintptr_t>(a.norm_w) |
+                 reinterpret_cast<uintptr_t>(a.x_out)) & 15) == 0, "product with the norm folded in: operands must be 16-byte aligned");
+    MS_REQUIRE(n_partials == 0 || (a.x_out && a.x_out != a.x), "product with the norm folded in: pending sums need another buffer for the stream");
+    a.k_per_wave = ceil_div(ceil_div(a.K, KSTEP), ksi) * KSTEP;
+    const dim3 grid((unsigned)ceil_div(a.N, 32));
+#define MS_SKN(KSI_, NP_)                                                                                     \
+    hipLaunchKernelGGL((gemm_skinny_norm_kernel<2, KSI_, EPI, NP_>), grid, dim3(64 * KSI_), 0, stream, a); \
+    return check_launch("gemm_skinny_norm")
+#define MS_SKN_NP(KSI_)                          \
+    switch (n_partials) {                        \
+        case 0: MS_SKN(KSI_, 0);                 \
+        case 1: MS_SKN(KSI_, 1);                 \
+        case 2: MS_SKN(KSI_, 2);                 \
+        case 3: MS_SKN(KSI_, 3);                 \
+        case 4: MS_SKN(KSI_, 4);                 \
+        case 5: MS_SKN(KSI_, 5);                 \
+        default: MS_SKN(KSI_, 6);                \
+    }
+    if (ksi == 8) { MS_SKN_NP(8) }
+    if (ksi == 4) { MS_SKN_NP(4) }
+    MS_SKN_NP(2)
+#undef MS_SKN_NP
+#undef MS_SKN
 }
 
 }  // namespace ms
@@ -268,4 +483,38 @@ extern "C" int ms_linear_swiglu_skinny(const void* a, const void* w, void* out, 
     const int n = 2 * ceil_div(I, 16) * 16;
     SkinnyArgs args{(const elem_t*)a, (const elem_t*)w, out, M, n, K, 0, I};
     return launch_skinny<SK_SWIGLU>(args, plan_skinny(M, n, K, false), stream);
+}
+
+// Whether ms_linear_norm_skinny / ms_linear_swiglu_norm_skinny should be given this shape.
+// Every block reads the stream and its pending sums for itself, which pays only while there is little
+// to read (measured: with nothing pending it saves a microsecond or two over the norm's own launch;
+// with one pending sum it breaks even at four rows; with five it costs twice as much).
+extern "C" int ms_skinny_norm_takes(int M, int N, int K, int n_partials) {
+    if (n_partials > 1 || (n_partials == 1 && M > 4)) return 0;
+    return plan_skinny_norm(M, N, K, n_partials) > 0;
+}
+
+// out[M, N] (float) = rmsnorm(x + sum partials; norm_w, eps) w^T, and x_out = x + sum partials (if any are pending).
+extern "C" int ms_linear_norm_skinny(const float* x, const float* partials, int n_partials, int T, const float* norm_w, float eps,
+                                     float* x_out, const void* w, float* out, int M, int N, int K, hipStream_t stream) {
+    SkinnyNormArgs a{x, partials ? partials : x, (size_t)T * K, norm_w, n_partials ? x_out : nullptr, (const elem_t*)w, out, M, N, K, 0, 0, eps};
+    return launch_skinny_norm<SK_STORE_F32>(a, n_partials, stream);
+}
+
+// out[M, I] = silu(h g^T) * (h u^T) with h = rmsnorm(x + sum partials), gate and up rows interleaved in blocks of 16.
+extern "C" int ms_linear_swiglu_norm_skinny(const float* x, const float* partials, int n_partials, int T, const float* norm_w,
+                                            float eps, float* x_out, const void* w, void* out, int M, int I, int K,
+                                            hipStream_t stream) {
+    const int n = 2 * ceil_div(I, 16) * 16;
+    SkinnyNormArgs a{x, partials ? partials : x, (size_t)T * K, norm_w, n_partials ? x_out : nullptr, (const elem_t*)w, out, M, n, K, 0, I, eps};
+    return launch_skinny_norm<SK_SWIGLU>(a, n_partials, stream);
+}
+
+// x[M, N] += a w^T for a product whose K lies inside one block (ms_skinny_partials(..., 1) == 1): the
+// stream takes the sum in the product's epilogue and nothing stays pending.
+extern "C" int ms_linear_residual_skinny(const void* a, const void* w, float* x, int M, int N, int K, hipStream_t stream) {
+    const SkinnyPlan p = plan_skinny(M, N, K, true);
+    MS_REQUIRE(p.ksb == 1, "few-rows product into the stream: K=%d is cut over %d blocks", K, p.ksb);
+    SkinnyArgs args{(const elem_t*)a, (const elem_t*)w, x, M, N, K, 0, 0};
+    return launch_skinny<SK_RESIDUAL>(args, p, stream);
 }

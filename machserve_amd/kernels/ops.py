@@ -183,12 +183,21 @@ class HipOps:
         return out
 
     def linear_residual(self, a: torch.Tensor, w: torch.Tensor, x: torch.Tensor) -> Optional[torch.Tensor]:
-        """``x += a @ w.T`` in the 32-bit residual stream.  When the product is cut along K (few rows,
-        or too few tiles to fill the chip) the sum is not added here: the float32 partial sums
-        ``[P, M, N]`` are returned for the consumer (the next norm) to fold in; otherwise None."""
+        """``x += a @ w.T`` in the 32-bit residual stream.  When the product is cut along K over several
+        blocks (a long K under few rows, or too few tiles to fill the chip) the sum is not added here:
+        the float32 partial sums ``[P, M, N]`` are returned for the consumer (the next norm) to fold
+        in; otherwise None."""
         M, N, K = self._mm_operands(a, w, "linear_residual")
         self._want(x, torch.float32, "residual stream", M, N)
-        if not self._tiled(M, N, K) or self._core.ms_tiled_partials(_c_int(M), _c_int(N), _c_int(K)) > 1:
+        if not self._tiled(M, N, K):
+            if M > 32 or self._core.ms_skinny_partials(_c_int(M), _c_int(N), _c_int(K), _c_int(1)) > 1:
+                return self.linear_split(a, w)
+            # all of K inside one block: one writer an element, added in the epilogue (up to 32 rows the
+            # kernel has registers to ask for the stream's values ahead; beyond, the next norm adds the sum)
+            self._check(self._core, self._core.ms_linear_residual_skinny(_ptr(a), _ptr(w), _ptr(x), _c_int(M), _c_int(N),
+                                                                         _c_int(K), _stream()))
+            return None
+        if self._core.ms_tiled_partials(_c_int(M), _c_int(N), _c_int(K)) > 1:
             return self.linear_split(a, w)
         self._check(self._core, self._core.ms_linear_residual(_ptr(a), _ptr(w), _ptr(x), _c_int(M), _c_int(N), _c_int(K),
                                                               _stream()))
@@ -205,6 +214,51 @@ class HipOps:
         self._check(self._core, fn(_ptr(a), _ptr(w_gate_up), _ptr(out), _c_int(M), _c_int(intermediate), _c_int(K),
                                    _stream()))
         return out
+
+    # ------------------------------------------------------------------ products with the norm folded in
+    def norm_folds_into(self, M: int, N: int, K: int, n_partials: int) -> bool:
+        """Whether a few-rows product over the stream can apply the stream's RMS norm itself (at most
+        16 rows, and a shape the few-rows kernel would take anyway)."""
+        return (not self._tiled(M, N, K)
+                and bool(self._core.ms_skinny_norm_takes(_c_int(M), _c_int(N), _c_int(K), _c_int(n_partials))))
+
+    def _normed_operands(self, x, partials, norm_w, w, what):
+        M, K = x.shape
+        self._want(x, torch.float32, f"{what} stream", M, K)
+        self._want(norm_w, torch.float32, f"{what} norm weight", K)
+        self._want(w, self.dtype, f"{what} weight")
+        if w.dim() != 2 or w.shape[1] != K:
+            raise KernelError(f"{what}: weight {tuple(w.shape)} for a stream of width {K}")
+        P = 0
+        if partials is not None:
+            P = partials.shape[0]
+            self._want(partials, torch.float32, f"{what} pending sums", P, M, K)
+        x_new = torch.empty_like(x) if P else None
+        return M, w.shape[0], K, P, x_new
+
+    def linear_split_normed(self, x: torch.Tensor, partials: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float,
+                            w: torch.Tensor):
+        """``rmsnorm(x + sum(partials)) @ w.T`` as float32 ``[1, M, N]``, and the stream with the
+        pending sums added (a new tensor; None if nothing was pending)."""
+        M, N, K, P, x_new = self._normed_operands(x, partials, norm_w, w, "linear_split_normed")
+        out = torch.empty((1, M, N), dtype=torch.float32, device=x.device)
+        self._check(self._core, self._core.ms_linear_norm_skinny(
+            _ptr(x), _ptr(partials), _c_int(P), _c_int(M), _ptr(norm_w), _c_float(eps), _ptr(x_new), _ptr(w), _ptr(out),
+            _c_int(M), _c_int(N), _c_int(K), _stream()))
+        return out, x_new
+
+    def linear_swiglu_normed(self, x: torch.Tensor, partials: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float,
+                             w_gate_up: torch.Tensor, intermediate: int):
+        """``silu(h @ gate.T) * (h @ up.T)`` for ``h = rmsnorm(x + sum(partials))`` (see
+        :meth:`linear_swiglu`), and the stream with the pending sums added (or None)."""
+        M, N, K, P, x_new = self._normed_operands(x, partials, norm_w, w_gate_up, "linear_swiglu_normed")
+        if N != 2 * ((intermediate + 15) // 16) * 16:
+            raise KernelError(f"linear_swiglu_normed: interleaved weight has {N} rows for intermediate size {intermediate}")
+        out = torch.empty((M, intermediate), dtype=self.dtype, device=x.device)
+        self._check(self._core, self._core.ms_linear_swiglu_norm_skinny(
+            _ptr(x), _ptr(partials), _c_int(P), _c_int(M), _ptr(norm_w), _c_float(eps), _ptr(x_new), _ptr(w_gate_up), _ptr(out),
+            _c_int(M), _c_int(intermediate), _c_int(K), _stream()))
+        return out, x_new
 
     # ------------------------------------------------------------------ attention
     def _attention_lib(self, hd: int):

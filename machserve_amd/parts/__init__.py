@@ -1,11 +1,11 @@
-from .base import (Block, FeedForward, GroupView, Mixer, Norm, PagedKVRequest, Part, PositionEncoding, ResidualStream, Runtime,
+from .base import (Block, FeedForward, GroupView, Mixer, Norm, PagedKVRequest, Part, PendingNorm, PositionEncoding, ResidualStream, Runtime,
                    SharedKVRequest, StateRequest, StepContext, TensorDecl)
 from .registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, register_block, register_feed_forward,
                        register_mixer, register_norm, register_position_encoding)
 from . import norm, rotary, attention, feed_forward, block  # noqa: F401  (registers the built-in parts)
 from .model import DecoderModel, Embedding, Head
 
-__all__ = ["Block", "FeedForward", "GroupView", "Mixer", "Norm", "PagedKVRequest", "Part", "PositionEncoding",
+__all__ = ["Block", "FeedForward", "GroupView", "Mixer", "Norm", "PagedKVRequest", "Part", "PendingNorm", "PositionEncoding",
            "ResidualStream", "Runtime", "SharedKVRequest", "StateRequest", "StepContext", "TensorDecl", "BLOCKS", "FEED_FORWARDS",
            "MIXERS", "NORMS", "POSITION_ENCODINGS", "register_block", "register_feed_forward", "register_mixer",
            "register_norm", "register_position_encoding", "DecoderModel", "Embedding", "Head"]

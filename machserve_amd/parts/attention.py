@@ -10,13 +10,14 @@ from __future__ import annotations
 
 import torch
 
-from .base import Mixer, PagedKVRequest, SharedKVRequest, TensorDecl
+from .base import Mixer, PagedKVRequest, PendingNorm, SharedKVRequest, TensorDecl
 from .registry import POSITION_ENCODINGS, register_mixer
 
 
 @register_mixer("attention")
 class Attention(Mixer):
     graph_safe = True  # reads positions and addresses from device memory only
+    takes_pending_norm = True  # its first product can apply the norm of the stream itself
 
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
@@ -70,7 +71,8 @@ class Attention(Mixer):
     def forward(self, h, stream, ctx):
         s, ops = self.spec, self.rt.ops
         view = ctx.groups[self.group]
-        qkv = ops.linear_split(h, self.w_qkv)  # [P, T, nq (+ 2 nkv)] partial sums, bias not yet added
+        # [P, T, nq (+ 2 nkv)] partial sums, bias not yet added
+        qkv = h.linear_split(self.w_qkv) if isinstance(h, PendingNorm) else ops.linear_split(h, self.w_qkv)
         inv_freq = self.position.rotary_inv_freq() if self.position is not None else None
         bias = self.b_qkv
         if self.position is not None and inv_freq is None:

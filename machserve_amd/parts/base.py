@@ -129,6 +129,31 @@ class ResidualStream:
         self.flush()
         return self.x
 
+    def normed_linear_split(self, weight: torch.Tensor, eps: float, w: torch.Tensor) -> torch.Tensor:
+        """``rmsnorm(x) @ w.T`` as float32 ``[P, T, N]`` partial sums, the norm folded into the product
+        where the kernels take the shape."""
+        self._launch_deferred()
+        T, K = self.x.shape
+        P = 0 if self.pending is None else self.pending.shape[0]
+        if self.ops.norm_folds_into(T, w.shape[0], K, P):
+            out, x_new = self.ops.linear_split_normed(self.x, self.pending, weight, eps, w)
+            if x_new is not None:
+                self.x, self.pending = x_new, None
+            return out
+        return self.ops.linear_split(self.normed(weight, eps), w)
+
+    def normed_linear_swiglu(self, weight: torch.Tensor, eps: float, w_gate_up: torch.Tensor, intermediate: int) -> torch.Tensor:
+        """``silu(h @ gate.T) * (h @ up.T)`` for ``h = rmsnorm(x)``, the norm folded in where possible."""
+        self._launch_deferred()
+        T, K = self.x.shape
+        P = 0 if self.pending is None else self.pending.shape[0]
+        if self.ops.norm_folds_into(T, w_gate_up.shape[0], K, P):
+            out, x_new = self.ops.linear_swiglu_normed(self.x, self.pending, weight, eps, w_gate_up, intermediate)
+            if x_new is not None:
+                self.x, self.pending = x_new, None
+            return out
+        return self.ops.linear_swiglu(self.normed(weight, eps), w_gate_up, intermediate)
+
     def normed(self, weight: torch.Tensor, eps: float, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``rmsnorm(x) * weight`` of the stream with everything added (of its ``rows`` if given),
         in the element type."""
@@ -139,7 +164,27 @@ class ResidualStream:
         return h
 
 
+class PendingNorm:
+    """The normalised stream, not yet computed: a part that starts with a product over it (``takes_pending_norm``)
+    gets this instead of a tensor and lets the product's kernel apply the norm; ``tensor()`` runs
+    the norm by itself."""
+
+    def __init__(self, stream: ResidualStream, weight: torch.Tensor, eps: float):
+        self.stream, self.weight, self.eps = stream, weight, eps
+
+    def tensor(self) -> torch.Tensor:
+        return self.stream.normed(self.weight, self.eps)
+
+    def linear_split(self, w: torch.Tensor) -> torch.Tensor:
+        return self.stream.normed_linear_split(self.weight, self.eps, w)
+
+    def linear_swiglu(self, w_gate_up: torch.Tensor, intermediate: int) -> torch.Tensor:
+        return self.stream.normed_linear_swiglu(self.weight, self.eps, w_gate_up, intermediate)
+
+
 class Part:
+    takes_pending_norm = False  # True: forward's normalised input may be a PendingNorm
+
     def __init__(self, spec, rt: Runtime):
         self.spec = spec
         self.rt = rt
@@ -157,6 +202,10 @@ class Norm(Part):
         """Normalised copy of the stream (of its ``rows`` if given), in the element type.  Pending
         sums of the stream are folded in."""
         raise NotImplementedError
+
+    def pending(self, stream: ResidualStream) -> Optional[PendingNorm]:
+        """The same, left to the reader's first product, if this norm can be folded into one."""
+        return None
 
 
 class PositionEncoding(Part):

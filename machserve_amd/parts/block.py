@@ -9,5 +9,15 @@ from .registry import register_block
 @register_block("prenorm")
 class PreNormBlock(Block):
     def forward(self, stream, ctx):
-        self.mixer.forward(self.mixer_norm.forward(stream), stream, ctx)
-        self.feed_forward.forward(self.feed_forward_norm.forward(stream), stream, ctx)
+        self.mixer.forward(self._input(self.mixer_norm, self.mixer, stream), stream, ctx)
+        self.feed_forward.forward(self._input(self.feed_forward_norm, self.feed_forward, stream), stream, ctx)
+
+    @staticmethod
+    def _input(norm, reader, stream):
+        """The reader's normalised input: a tensor, or for a reader that starts with a product over it
+        the norm left pending, so that the product's kernel can apply it."""
+        if reader.takes_pending_norm:
+            pending = norm.pending(stream)
+            if pending is not None:
+                return pending
+        return norm.forward(stream)

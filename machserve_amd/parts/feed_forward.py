@@ -5,12 +5,14 @@ the 32-bit stream."""
 from __future__ import annotations
 
 from ..kernels.ops import interleave_gate_up
-from .base import FeedForward, TensorDecl
+from .base import FeedForward, PendingNorm, TensorDecl
 from .registry import register_feed_forward
 
 
 @register_feed_forward("gated_mlp")
 class GatedMlp(FeedForward):
+    takes_pending_norm = True  # its first product can apply the norm of the stream itself
+
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
         if spec.activation != "silu":
@@ -26,5 +28,8 @@ class GatedMlp(FeedForward):
         self.w_down = t["down.weight"]
 
     def forward(self, h, stream, ctx):
-        a = self.rt.ops.linear_swiglu(h, self.w_gate_up, self.spec.intermediate)
+        if isinstance(h, PendingNorm):
+            a = h.linear_swiglu(self.w_gate_up, self.spec.intermediate)
+        else:
+            a = self.rt.ops.linear_swiglu(h, self.w_gate_up, self.spec.intermediate)
         stream.add_linear(a, self.w_down)

@@ -2,7 +2,7 @@
 (``crates/mach-model/src/kernels.rs:63-80``)."""
 from __future__ import annotations
 
-from .base import Norm, TensorDecl
+from .base import Norm, PendingNorm, TensorDecl
 from .registry import register_norm
 
 
@@ -16,3 +16,6 @@ class RMSNorm(Norm):
 
     def forward(self, stream, rows=None):
         return stream.normed(self.weight, self.spec.eps, rows)
+
+    def pending(self, stream):
+        return PendingNorm(stream, self.weight, self.spec.eps)

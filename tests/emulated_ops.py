@@ -54,6 +54,26 @@ class EmulatedOps:
             return torch.stack([y - r, r])
         return y.unsqueeze(0)
 
+    def norm_folds_into(self, M, N, K, n_partials):
+        return M <= 16 and N >= 64
+
+    def _normed(self, x, partials, norm_w, eps):
+        full = x if partials is None else x + partials.sum(0)
+        inv = 1.0 / torch.sqrt((full * full).sum(-1, keepdim=True) / full.shape[-1] + eps)
+        return self._r(full * norm_w), inv, (full if partials is not None else None)
+
+    def linear_split_normed(self, x, partials, norm_w, eps, w):
+        a, inv, x_new = self._normed(x, partials, norm_w, eps)
+        return ((a.float() @ w.float().t()) * inv).unsqueeze(0), x_new
+
+    def linear_swiglu_normed(self, x, partials, norm_w, eps, w_gate_up, intermediate):
+        a, inv, x_new = self._normed(x, partials, norm_w, eps)
+        Ip = w_gate_up.shape[0] // 2
+        w = w_gate_up.float().view(Ip // 16, 2, 16, -1)
+        gate = (a.float() @ w[:, 0].reshape(Ip, -1).t()) * inv
+        up = (a.float() @ w[:, 1].reshape(Ip, -1).t()) * inv
+        return self._r((gate / (1.0 + torch.exp(-gate)) * up)[:, :intermediate]), x_new
+
     def linear_residual(self, a, w, x):
         if a.shape[0] <= self.SKINNY_ROWS:
             return self.linear_split(a, w)

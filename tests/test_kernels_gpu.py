@@ -71,8 +71,8 @@ def test_linear(dtype, M, N, K):
     assert_close(ops.linear(a.to(DEV), w.to(DEV), None), P.linear(a.double(), w.double()), dtype, "linear")
     x = rnd((M, N), torch.float32, 8)
     xd = x.to(DEV).clone()
-    pending = ops.linear_residual(a.to(DEV), w.to(DEV), xd)  # few rows, or few tiles and a long K: partial sums
-    assert pending is not None or M > 64
+    # K cut over several blocks (a long K under few rows, or few tiles): partial sums; else added in the epilogue
+    pending = ops.linear_residual(a.to(DEV), w.to(DEV), xd)
     if pending is not None:
         ops.add_partials(xd, pending)
     assert_close(xd, x.double() + P.linear(a.double(), w.double()), torch.float32 if dtype == torch.float32 else dtype, "linear_residual")
@@ -113,11 +113,48 @@ def test_linear_few_rows(dtype, M, N, K):
     x0 = rnd((M, N), torch.float32, 23)
     x = x0.to(DEV)
     pend = ops.linear_residual(a.to(DEV), w.to(DEV), x)
-    if pend is None:  # a large weight under many rows goes to the tiled kernel, which adds in its epilogue
-        assert ops._tiled(M, N, K)
+    if pend is None:  # K inside one block, or a large weight under many rows (tiled kernel): added in the epilogue
+        assert (parts.shape[0] == 1 and M <= 32) or ops._tiled(M, N, K)
         assert_close(x.cpu() - x0, ref, torch.float32 if dtype == torch.float32 else dtype, "added in place")
     else:
         assert torch.equal(pend, parts) and torch.equal(x.cpu(), x0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K,NP", [(1, 1152, 896, 0), (8, 1152, 896, 5), (16, 300, 264, 1), (3, 2048, 1536, 2),
+                                      (5, 130, 1000, 3), (16, 4608, 3584, 6), (2, 64, 4864, 4)])
+def test_products_with_the_norm_folded_in(dtype, M, N, K, NP):
+    """rmsnorm(x + pending sums) times a weight in one kernel: the norm's factor applied to the
+    finished sums, the stream with the sums added written to another buffer (the same bits as adding
+    them in order), and the same with the gated activation."""
+    from machserve_amd.kernels import interleave_gate_up
+    ops = ops_for(dtype)
+    # the engine folds the norm in only while there is little to read; the kernels take up to six pending sums
+    assert ops.norm_folds_into(M, N, K, NP) == (NP == 0 or (NP == 1 and M <= 4))
+    assert not ops.norm_folds_into(17, N, K, 0)
+    eps = 1e-5
+    x = rnd((M, K), torch.float32, 31, 2.0)
+    parts = rnd((NP, M, K), torch.float32, 32) if NP else None
+    nw = 1 + rnd((K,), torch.float32, 33, 0.1)
+    w = rnd((N, K), dtype, 34, K ** -0.5)
+    total = x.clone()
+    for p in range(NP):
+        total += parts[p]
+    h = P.rms_norm(total, nw, eps)
+    ref = P.linear(h.double(), w.double())
+    dev = lambda t: None if t is None else t.to(DEV)
+    out, x_new = ops.linear_split_normed(dev(x), dev(parts), dev(nw), eps, dev(w))
+    assert out.shape == (1, M, N) and (x_new is None) == (NP == 0)
+    assert_close(out[0], ref, torch.float32 if dtype == torch.float32 else dtype, "product of the normed stream")
+    if NP:
+        assert torch.equal(x_new.cpu(), total), "the stream with its pending sums, added in order"
+    I = N // 2 - 3
+    g, u = rnd((I, K), dtype, 35, K ** -0.5 * 3), rnd((I, K), dtype, 36, K ** -0.5)
+    ref = P.silu(P.linear(h.double(), g.double())) * P.linear(h.double(), u.double())
+    got, x_new = ops.linear_swiglu_normed(dev(x), dev(parts), dev(nw), eps, interleave_gate_up(g, u).to(DEV), I)
+    assert_close(got, ref, dtype, "gated product of the normed stream")
+    if NP:
+        assert torch.equal(x_new.cpu(), total)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
