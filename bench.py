@@ -68,6 +68,7 @@ def main() -> int:
     ap.add_argument("--shape", default="0.5b", choices=sorted(SHAPES), help="layer sizes (default: the 0.5B configuration)")
     ap.add_argument("--page-size", type=int, default=64)
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--sync-steps", action="store_true", help="wait for each decode step's tokens before the next is launched")
     ap.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiles)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -106,15 +107,21 @@ def main() -> int:
             eng.add(p, args.warmup + args.steps + 2 * batch + 64, SamplingParams())  # early ones decode while later ones prefill
         while any(not r.decoding for r in eng.scheduler.running) or eng.scheduler.waiting:
             eng.step()
+        # the engine's own loop (Engine.run): a step is launched while the tokens of the step before
+        # are on their way to the host, so the tokens a call returns are those of the launch before it
+        step = eng.step if args.sync_steps else eng.step_pipelined
         for _ in range(args.warmup):
-            eng.step()
+            step()
         torch.cuda.synchronize()
+        before, seen = eng.steps, 0
         t0 = time.perf_counter()
         for _ in range(args.steps):
-            em, _ = eng.step()
-            assert len(em) == batch
+            em, _ = step()
+            seen += len(em)
         torch.cuda.synchronize()
         dt_s = time.perf_counter() - t0
+        assert eng.steps - before == args.steps, "exactly the timed steps ran on the device"
+        assert batch * (args.steps - 1) <= seen <= batch * args.steps  # the first call may have had nothing before it
         del eng
         torch.cuda.empty_cache()
         return batch * args.steps / dt_s, dt_s / args.steps * 1e3
@@ -155,6 +162,7 @@ def main() -> int:
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
             "tied_head": bool(cfg.tie_word_embeddings), "rope_theta": cfg.rope_theta, "rms_eps": cfg.rms_norm_eps,
             "page_size": page, "prefill_tokens": ctx, "sampling": "greedy",
+            "stepping": "one at a time" if args.sync_steps else "launched one step ahead",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},

@@ -23,6 +23,7 @@ class Engine:
         self.sampler = Sampler(loaded.rt.ops, loaded.rt.device)
         self.steps = 0
         self.tokens_run = 0
+        self._inflight = None  # (plan, launched step) of step_pipelined
         # Every step makes a few hundred short-lived objects; with the interpreter's whole heap in the
         # collector's oldest generation its full passes cost more than the scheduling itself.  What
         # exists now (modules, the model) is taken out of the collector's reach.
@@ -46,12 +47,80 @@ class Engine:
         return self.scheduler.add(prompt, max_new, params, eos, stop_seqs)
 
     def has_work(self) -> bool:
-        return self.scheduler.has_work()
+        return self.scheduler.has_work() or self._inflight is not None
 
     def step(self):
         """One scheduled batch.  Returns ``(emitted, finished)``: the (request id, token) pairs
         produced and the requests that ended."""
+        if self._inflight is not None:
+            return self._drain()
         plan: StepPlan = self.scheduler.schedule()
+        return self._run_plan(plan)
+
+    def step_pipelined(self):
+        """Like :meth:`step`, but a step of decoded tokens is launched before the tokens of the step
+        before it have come back: it takes them on the device, and the host's share of a step (the
+        scheduler, the step's buffers, reading the samples) runs while the device works.  What is
+        returned is what has become known by now, which lags the launches by one step; what would
+        end a request is seen one step late, and the token computed for it in between is dropped.
+        Steps that are not plain decoding of the same requests (a prompt portion, an arrival, an
+        end, sampling with penalties) are run as :meth:`step` runs them, after what is in flight."""
+        sched = self.scheduler
+        if self._inflight is None:
+            plan = sched.schedule()
+            launched = self._launch(plan, None)
+            if launched is None:
+                return self._run_plan(plan)
+            self._inflight = (plan, launched)
+            return [], []
+        prev_plan, prev = self._inflight
+        plan = sched.schedule()
+        launched = self._launch(plan, prev) if self._continues(prev_plan, plan) else None
+        emitted, done = sched.complete(prev_plan, *self.loaded.step.collect(prev))
+        if launched is not None:
+            self._inflight = (plan, launched)
+            return emitted, done
+        self._inflight = None
+        # the plan was made before these tokens were known: what has ended meanwhile drops out of it
+        plan.items = [it for it in plan.items if it.request.closing is None or it.request.pending > 0]
+        plan.native = [n for n in plan.native if n.id in sched.requests]
+        em2, done2 = self._run_plan(plan)
+        return emitted + em2, done + done2
+
+    def _continues(self, before: StepPlan, plan: StepPlan) -> bool:
+        """Whether ``plan`` decodes one token for exactly the requests of ``before``, in its order."""
+        return (not plan.preempted and not plan.admitted and len(plan.items) == len(before.items)
+                and all(a.request is b.request and a.sample and a.count == 1 for a, b in zip(plan.items, before.items)))
+
+    def _launch(self, plan: StepPlan, after):
+        """Launch ``plan`` without waiting if it is plain decoding; None (nothing done) if it is not."""
+        if not plan.items or not all(it.sample and it.count == 1 and it.request.params.plain() for it in plan.items):
+            return None
+        if after is None and any(it.request.pending for it in plan.items):
+            return None
+        reqs = [it.request for it in plan.items]
+        # after another launch the tokens are taken on the device; the entries' own are placeholders
+        entries = [StepEntry(r.slot, [0] if after is not None else [r.tokens[it.start]], [0]) for r, it in zip(reqs, plan.items)]
+        launched = self.loaded.step.launch_decode(
+            entries, [r.params.temperature for r in reqs], [r.params.top_k for r in reqs], [r.params.top_p for r in reqs],
+            [r.rng_state for r in reqs], after)
+        if launched is None:
+            return None
+        from ..sampling import advance
+        for r in reqs:
+            r.rng_state = advance(r.rng_state)  # one draw a sampled row, whatever the token
+        self.scheduler.begin(plan)
+        self.steps += 1
+        self.tokens_run += plan.n_tokens
+        return launched
+
+    def _drain(self):
+        """Wait for the step in flight and take its tokens."""
+        plan, launched = self._inflight
+        self._inflight = None
+        return self.scheduler.complete(plan, *self.loaded.step.collect(launched))
+
+    def _run_plan(self, plan: StepPlan):
         if not plan.items:
             return [], []
         entries, sampled_items = [], []
@@ -84,7 +153,7 @@ class Engine:
     def run(self) -> Dict[int, Request]:
         """Step until every queued request has finished."""
         while self.has_work():
-            self.step()
+            self.step_pipelined()
         return self.scheduler.finished
 
     def generate(self, prompts: Sequence[Sequence[int]], max_new: int, temperature: float = 0.0, seed: int = 0,

@@ -47,6 +47,8 @@ class Request:
     top_logprobs: List[list] = field(default_factory=list)  # per generated token: [(token, logprob), ...]
     finish_reason: Optional[str] = None
     preemptions: int = 0
+    pending: int = 0                  # tokens sampled on the device that the host has not seen yet
+    closing: Optional[str] = None     # it has left the queues for this reason; finished once its tokens are in
 
     @property
     def generated(self) -> List[int]:
@@ -54,7 +56,8 @@ class Request:
 
     @property
     def decoding(self) -> bool:
-        return self.fed == len(self.tokens) - 1 and len(self.tokens) > len(self.prompt)
+        n = len(self.tokens) + self.pending
+        return self.fed == n - 1 and n > len(self.prompt)
 
 
 @dataclass
@@ -150,44 +153,80 @@ class Scheduler:
         return plan
 
     # ------------------------------------------------------------------ after the step
+    def _close(self, r: Request, reason: str) -> None:
+        """The request leaves the queues: its pages and slot go back now (work already launched on them
+        runs before anything that is launched later).  It is finished once its last token is in."""
+        if r.closing is None:
+            r.closing = reason
+            self.core.finish(r.id)
+            r.slot = None
+            del self.requests[r.id]
+
     def _finish(self, r: Request, reason: str) -> None:
-        r.finish_reason = reason
-        self.core.finish(r.id)  # its pages and slot go back
-        r.slot = None
-        del self.requests[r.id]
+        self._close(r, reason)
+        r.finish_reason = r.closing
         self.finished[r.id] = r
 
-    def update(self, plan: StepPlan, sampled: Sequence[int], logprobs: Optional[Sequence[float]] = None,
-               new_states: Optional[Sequence[int]] = None):
-        """The step ran: ``sampled[i]`` is the token of the i-th item with ``sample`` set.
-        Returns the list of (request id, token) emitted and the requests that finished."""
-        emitted, done = [], []
+    def begin(self, plan: StepPlan) -> None:
+        """The step has been launched: its tokens are in the cache, a sampled row will yield one
+        token more.  What follows from counts alone is decided here, before the tokens are known:
+        a request whose next token is its last leaves the queues."""
         self.core.advance(plan.native)
-        k = 0
         for it in plan.items:
             r = it.request
             r.fed += it.count
             if not it.sample:
                 continue
+            r.pending += 1
+            n = len(r.tokens) + r.pending
+            if n - len(r.prompt) >= r.max_new or (self.max_positions is not None and n > self.max_positions):
+                self._close(r, "length")
+
+    def complete(self, plan: StepPlan, sampled: Sequence[int], logprobs: Optional[Sequence[float]] = None,
+                 new_states: Optional[Sequence[int]] = None):
+        """The sampled tokens of a launched step have arrived: ``sampled[i]`` is the token of the i-th
+        item with ``sample`` set.  Returns the (request id, token) pairs emitted and the requests that
+        finished.  A token that arrives for a request already stopped (its end was only seen after
+        the next step had been launched) is dropped."""
+        emitted, done = [], []
+        k = 0
+        for it in plan.items:
+            if not it.sample:
+                continue
+            r = it.request
             tok = int(sampled[k])
-            if logprobs is not None:
-                r.logprobs.append(float(logprobs[k]))
+            lp = float(logprobs[k]) if logprobs is not None else None
             if new_states is not None:
                 r.rng_state = new_states[k]
             k += 1
+            r.pending -= 1
+            if r.finish_reason is not None:
+                continue
             r.tokens.append(tok)
+            if lp is not None:
+                r.logprobs.append(lp)
             emitted.append((r.id, tok))
             n_gen = len(r.tokens) - len(r.prompt)
-            reason = None
             if r.eos is not None and tok == r.eos:
-                reason = "stop"
+                r.closing = None if r.closing == "length" else r.closing  # the token itself decides
+                self._stop(r)
             elif any(n_gen >= len(s) and r.tokens[-len(s):] == s for s in r.stop_seqs):
-                reason = "stop"
-            elif n_gen >= r.max_new:
-                reason = "length"
-            elif self.max_positions is not None and len(r.tokens) > self.max_positions:
-                reason = "length"
-            if reason:
-                self._finish(r, reason)
+                r.closing = None if r.closing == "length" else r.closing
+                self._stop(r)
+            if r.closing is not None and (r.closing == "stop" or r.pending == 0):
+                r.finish_reason = r.closing
+                self.finished[r.id] = r
                 done.append(r)
         return emitted, done
+
+    def _stop(self, r: Request) -> None:
+        if r.id in self.requests:
+            self._close(r, "stop")
+        else:
+            r.closing = "stop"  # it had left the queues for its length already
+
+    def update(self, plan: StepPlan, sampled: Sequence[int], logprobs: Optional[Sequence[float]] = None,
+               new_states: Optional[Sequence[int]] = None):
+        """``begin`` and ``complete`` at once, for a step whose tokens are known when it returns."""
+        self.begin(plan)
+        return self.complete(plan, sampled, logprobs, new_states)

@@ -43,6 +43,17 @@ class _DecodeGraph:
         self.copied = torch.cuda.Event()  # the last upload of `pinned` has finished
 
 
+@dataclass
+class LaunchedDecode:
+    """A decode step that runs on the device: its requests' slots, the device tensor that will hold
+    its samples (int32 ``[2, B]``: tokens, bits of the logprobs), the pinned copy of it, and the
+    event after that copy."""
+    slots: List[int]
+    sampled: torch.Tensor
+    result: torch.Tensor
+    done: object
+
+
 class StepFunction:
     TABLE_BUCKET = 8  # captured block tables are this many pages wide, or a multiple
 
@@ -55,6 +66,8 @@ class StepFunction:
         self.use_graphs = (use_graphs and rt.device.type == "cuda"
                            and all(getattr(b.mixer, "graph_safe", False) for b in getattr(model, "blocks", [])))
         self._graphs: Dict[tuple, _DecodeGraph] = {}
+        self._results: Dict[int, list] = {}  # pinned buffers for the samples, three per batch size, in turn
+        self._launches = 0
 
     # ------------------------------------------------------------------ context
     def _check_entries(self, entries: Sequence[StepEntry]):
@@ -113,10 +126,12 @@ class StepFunction:
         return self._context_from(dev, offsets, widths, lists)
 
     # ------------------------------------------------------------------ captured decode steps
-    def _run_decode_graph(self, entries: Sequence[StepEntry], sampling=None):
+    def _run_decode_graph(self, entries: Sequence[StepEntry], sampling=None, device_tokens: Optional[torch.Tensor] = None):
         """Replay (or first capture) the graph of this batch size.  ``sampling`` = (temperatures,
         top_ks, top_ps, states) makes sampling part of the graph; the result is then the int32
-        ``[2, B]`` tensor of :meth:`HipOps.sample_packed`, else the logits."""
+        ``[2, B]`` tensor of :meth:`HipOps.sample_packed`, else the logits.  With ``device_tokens``
+        (int32, one per entry, on the device) the step's tokens are taken from there and the
+        entries' own tokens are placeholders."""
         slots, counts, tokens, _ = self._check_entries(entries)
         B = len(slots)
         host, offsets, widths = self.cache.build_step(slots, counts, tokens, list(range(B)), self.heads_per_kv,
@@ -148,6 +163,9 @@ class StepFunction:
             staged[dg.offsets[k][0]:dg.offsets[k][0] + a.size] = a
         dg.dev.copy_(dg.pinned, non_blocking=True)
         dg.copied.record()
+        if device_tokens is not None:
+            start, size = dg.offsets["tokens"]
+            dg.dev[start:start + size].copy_(device_tokens)
         if dg.graph is None:
             ctx = self._context_from(dg.dev, dg.offsets, widths)
             side = torch.cuda.Stream(device=self.rt.device)
@@ -173,9 +191,21 @@ class StepFunction:
         """A decode-only step (one token per request) with sampling inside the captured graph: one
         upload, one replay, one copy back.  Returns ``(tokens, logprobs)`` as host lists, or None
         if this step cannot take that path (the caller then uses ``__call__`` and the sampler)."""
+        launched = self.launch_decode(entries, temperatures, top_ks, top_ps, states)
+        return None if launched is None else self.collect(launched)
+
+    def launch_decode(self, entries: Sequence[StepEntry], temperatures, top_ks, top_ps, states,
+                      after: Optional["LaunchedDecode"] = None) -> Optional["LaunchedDecode"]:
+        """The same step, launched and not waited for.  With ``after`` - the launched step before
+        this one, of the same requests in the same order - the tokens are that step's samples,
+        taken on the device: the host need not have seen them.  None if the step cannot take this
+        path; ``OutOfPages`` before anything ran if the pages are not there."""
         if not (self.use_graphs and all(len(e.tokens) == 1 for e in entries)
                 and len({e.slot for e in entries}) == len(entries)):
             return None
+        slots = [e.slot for e in entries]
+        if after is not None and after.slots != slots:
+            raise StepError("a step fed from the device must hold the requests of the step before, in the same order")
         cache = self.cache
         reserved: Dict[str, int] = {}
         for e in entries:
@@ -186,10 +216,25 @@ class StepFunction:
                 raise OutOfPages(f"group {k}: the step needs {v} new pages, {cache.free_pages(k)} are free")
         for e in entries:
             cache.extend(e.slot, 1)
-        both = self._run_decode_graph(entries, (temperatures, top_ks, top_ps, states)).cpu()  # the step's one sync
+        sampled = self._run_decode_graph(entries, (temperatures, top_ks, top_ps, states),
+                                         None if after is None else after.sampled[0])
         for e in entries:
             cache.commit(e.slot, 1)
-        return both[0].tolist(), both[1].view(torch.float32).tolist()
+        # the samples go to a pinned buffer of their own (the graph's is overwritten by its next replay)
+        ring = self._results.get(len(slots))
+        if ring is None:
+            ring = self._results[len(slots)] = [torch.empty((2, len(slots)), dtype=torch.int32, pin_memory=True) for _ in range(3)]
+        result = ring[self._launches % 3]  # at most two steps are in flight: a buffer is read before its next turn
+        self._launches += 1
+        result.copy_(sampled, non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+        return LaunchedDecode(slots, sampled, result, done)
+
+    def collect(self, launched: "LaunchedDecode"):
+        """``(tokens, logprobs)`` of a launched step as host lists; waits for them."""
+        launched.done.synchronize()
+        return launched.result[0].tolist(), launched.result[1].view(torch.float32).tolist()
 
     # ------------------------------------------------------------------ the step
     def __call__(self, entries: Sequence[StepEntry], borrow_logits: bool = False) -> Optional[torch.Tensor]:

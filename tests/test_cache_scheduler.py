@@ -294,3 +294,78 @@ def test_engine_reports_logprobs_and_top_logprobs(tmp_path):
         seq.append(tok)
     with pytest.raises(ValueError, match="top_logprobs"):
         eng.add(p, 1, SamplingParams(top_logprobs=21))
+
+
+class _LaggedDecode:
+    """Stand-in on the CPU for the launched decode step of the device: what it samples stays out of
+    the engine's sight until ``collect``, and a step launched after another takes that step's tokens
+    from it directly, as the device does."""
+
+    def __init__(self, eng):
+        self.eng, self.fed_from_device = eng, 0
+        eng.loaded.step.launch_decode = self.launch_decode
+        eng.loaded.step.collect = lambda launched: (launched["tokens"], launched["logprobs"])
+
+    def launch_decode(self, entries, temperatures, top_ks, top_ps, states, after=None):
+        from machserve_amd.engine.step import StepEntry
+        from machserve_amd.sampling import SamplingParams
+        if not all(len(e.tokens) == 1 for e in entries):
+            return None
+        if after is not None:
+            assert after["slots"] == [e.slot for e in entries]
+            entries = [StepEntry(e.slot, [t], e.want) for e, t in zip(entries, after["tokens"])]
+            self.fed_from_device += 1
+        logits = self.eng.loaded.step(entries)
+        params = [SamplingParams(temperature=t, top_k=k, top_p=p) for t, k, p in zip(temperatures, top_ks, top_ps)]
+        tokens, logprobs, _, _ = self.eng.sampler.sample(logits, params, list(states), [[] for _ in entries])
+        return {"slots": [e.slot for e in entries], "tokens": [int(t) for t in tokens], "logprobs": list(logprobs)}
+
+
+@pytest.mark.parametrize("pages", [16, 4])
+def test_pipelined_steps_give_what_synchronous_steps_give(tmp_path, pages):
+    """Steps launched before the tokens of the step before are known: the same tokens, log
+    probabilities and reasons to finish as with one step at a time, although an end-of-sequence
+    token or a stop sequence is seen one step late, requests end at different steps, one arrives in
+    the middle, and (with few pages) one is preempted."""
+    from machserve_amd.engine import Engine, load_model
+    from machserve_amd.sampling import SamplingParams
+    d = make_model_dir(tmp_path, "A")
+    prompts = [random_prompt(n, 512, 80 + n) for n in (7, 19, 12, 5)]
+    max_new = [14, 6, 11, 9]
+
+    def run(pipelined, eos=None, stop=()):
+        lm = load_model(d, dtype="float32", device="cpu", page_size=16, num_pages=pages, max_requests=3, ops=EmulatedOps())
+        eng = Engine(lm, max_batch_tokens=32)
+        lag = _LaggedDecode(eng)
+        ids = [eng.add(p, m, SamplingParams(temperature=0.9, top_k=40, seed=3 + i), eos=eos, stop_seqs=stop)
+               for i, (p, m) in enumerate(zip(prompts[:3], max_new))]
+        emitted, n = [], 0
+        while eng.has_work():
+            em, _ = eng.step_pipelined() if pipelined else eng.step()
+            emitted += em
+            n += 1
+            if n == 5:
+                ids.append(eng.add(prompts[3], max_new[3], SamplingParams(temperature=0.7, seed=9), eos=eos, stop_seqs=stop))
+            lm.cache.check()
+            assert n < 500
+        assert all(g.pool.available() == g.pool.num_pages for g in lm.cache.groups.values())
+        done = eng.scheduler.finished
+        per_request = {i: [t for j, t in emitted if j == i] for i in ids}
+        assert all(per_request[i] == done[i].generated for i in ids)
+        return ([(done[i].generated, done[i].finish_reason, [round(x, 5) for x in done[i].logprobs]) for i in ids],
+                lag.fed_from_device, sum(done[i].preemptions for i in ids))
+
+    plain, _, _ = run(False)
+    piped, from_device, preempted = run(True)
+    assert piped == plain and from_device > 3
+    assert (preempted > 0) == (pages == 4)
+    assert [r for _, r, _ in plain] == ["length"] * 4
+    # an end-of-sequence token and a stop sequence taken from the middle of what request 0 generates
+    first = plain[0][0]
+    eos = first[5]
+    stop = [first[3:5]]
+    for kw in ({"eos": eos}, {"stop": stop}, {"eos": plain[1][0][-1]}):
+        a, _, _ = run(False, **kw)
+        b, n_dev, _ = run(True, **kw)
+        assert a == b and n_dev > 0
+        assert "stop" in [r for _, r, _ in a]

@@ -61,6 +61,48 @@ def test_generation_under_page_pressure_equals_roomy_generation(dirs):
     assert n0 == 0 and n1 > 0 and roomy == tight
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_launched_ahead_give_what_steps_one_at_a_time_give(dirs, dtype):
+    """Engine.run launches a decode step before the samples of the step before have reached the
+    host (they are taken on the device).  Same tokens and log probabilities as with one step at a
+    time, with requests that end at different steps, one that arrives in the middle, and an
+    end-of-sequence token that is only seen one step late."""
+    from machserve_amd.engine import Engine
+    from machserve_amd.sampling import SamplingParams
+    prompts = [random_prompt(n, 1000, 20 + n) for n in (37, 8, 21, 14)]
+    max_new = [40, 17, 29, 23]
+
+    def run(pipelined, eos=None):
+        eng = Engine.from_dir(dirs["B"], dtype=dtype, page_size=32, num_pages=16, capacity=4, max_batch_tokens=48)
+        fed_from_device = [0]
+        launch = eng.loaded.step.launch_decode
+
+        def counted(*a, **kw):
+            fed_from_device[0] += (len(a) > 5 and a[5] is not None) or kw.get("after") is not None
+            return launch(*a, **kw)
+        eng.loaded.step.launch_decode = counted
+        ids = [eng.add(p, m, SamplingParams(temperature=0.8, top_k=60, top_p=0.9, seed=2 + i), eos=eos)
+               for i, (p, m) in enumerate(zip(prompts[:3], max_new))]
+        n = 0
+        while eng.has_work():
+            eng.step_pipelined() if pipelined else eng.step()
+            n += 1
+            if n == 9:
+                ids.append(eng.add(prompts[3], max_new[3], SamplingParams(seed=1), eos=eos))
+        eng.loaded.cache.check()
+        done = eng.scheduler.finished
+        return [(done[i].generated, done[i].finish_reason, done[i].logprobs) for i in ids], fed_from_device[0]
+
+    one_by_one, n0 = run(False)
+    ahead, n1 = run(True)
+    assert n0 == 0 and n1 > 20
+    assert ahead == one_by_one
+    eos = one_by_one[0][0][11]
+    a, _ = run(False, eos)
+    b, n2 = run(True, eos)
+    assert a == b and n2 > 0 and a[0][1] == "stop" and len(a[0][0]) <= 12
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_long_decoding(dirs, dtype):
     """One step of 8 tokens, then 400 single tokens across many pages: every position against
