@@ -74,12 +74,6 @@ __device__ __forceinline__ float exp_f(float x) {
 #endif
 }
 
-// The value unchanged, but of unknown origin to the optimiser.
-__device__ __forceinline__ int opaque(int x) {
-    asm volatile("" : "+v"(x));
-    return x;
-}
-
 __device__ __forceinline__ float exp2_f(float x) {
 #ifdef MS_ELEM_BF16
     return __builtin_amdgcn_exp2f(x);

@@ -96,6 +96,18 @@ __device__ __forceinline__ void mma_16x16x32(f32x4& acc, const Frag& a, const Fr
 #endif
 }
 
+// The value unchanged, but of unknown origin to the optimiser: a mask made this way is applied
+// to a loaded value as it stands, where a visible condition would be turned into a branch round
+// the load.
+__device__ __forceinline__ int opaque(int x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
+__device__ __forceinline__ uint32_t opaque(uint32_t x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
+
 // ---- reductions -----------------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

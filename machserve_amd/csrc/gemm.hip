@@ -11,6 +11,8 @@
 // Two LDS buffers, one barrier per K step.
 // Every output element is the sum over K in steps of 32 in ascending order whatever the
 // tile shape or the number of rows, so a row's result does not depend on its batch.
+#include <type_traits>
+
 #include "common.cuh"
 
 namespace ms {
@@ -61,22 +63,43 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
     const int m0 = (blockIdx.x % tiles_m) * BM, n0 = (blockIdx.x / tiles_m) * BN;
     const int r16 = lane & 15, grp = lane >> 4;
 
-    const int k_end = min(K, (int)(blockIdx.y + 1) * ep.k_per_split);
+    const int split = blockIdx.y;
+    const int k_end = min(K, (split + 1) * ep.k_per_split);
+    // Loads are unconditional, on one straight path: a row beyond the operand reads the last row
+    // (its results are never stored), and only the last K step of a slice, if it is a partial one,
+    // masks what lies beyond the slice.
     u32x4 ra[A_CHUNKS], rw[W_CHUNKS];
+    const elem_t* pa[A_CHUNKS];
+    const elem_t* pw[W_CHUNKS];
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+        const int c = tid + i * 256;
+        pa[i] = A + (size_t)min(m0 + c / CPR, M - 1) * K + (c % CPR) * EPC;
+    }
+#pragma unroll
+    for (int i = 0; i < W_CHUNKS; ++i) {
+        const int c = tid + i * 256;
+        pw[i] = W + (size_t)min(n0 + c / CPR, N - 1) * K + (c % CPR) * EPC;
+    }
     auto load_global = [&](int k0) {
 #pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) ra[i] = *reinterpret_cast<const u32x4*>(pa[i] + k0);
+#pragma unroll
+        for (int i = 0; i < W_CHUNKS; ++i) rw[i] = *reinterpret_cast<const u32x4*>(pw[i] + k0);
+    };
+    auto load_global_tail = [&](int k0) {
+        const int kk = k0 + (tid % CPR) * EPC;  // 256 % CPR == 0: the same K chunk for all of a thread's loads
+        const bool in = kk < k_end;
+        const uint32_t keep = opaque(in ? 0xffffffffu : 0u);
+#pragma unroll
         for (int i = 0; i < A_CHUNKS; ++i) {
-            const int c = tid + i * 256, row = c / CPR, kk = k0 + (c % CPR) * EPC;
-            u32x4 v = {0, 0, 0, 0};
-            if (m0 + row < M && kk < k_end) v = *reinterpret_cast<const u32x4*>(A + (size_t)(m0 + row) * K + kk);
-            ra[i] = v;
+            u32x4 v = *reinterpret_cast<const u32x4*>(in ? pa[i] + k0 : A);  // the operand's start when beyond the slice
+            ra[i] = (u32x4){v[0] & keep, v[1] & keep, v[2] & keep, v[3] & keep};
         }
 #pragma unroll
         for (int i = 0; i < W_CHUNKS; ++i) {
-            const int c = tid + i * 256, row = c / CPR, kk = k0 + (c % CPR) * EPC;
-            u32x4 v = {0, 0, 0, 0};
-            if (n0 + row < N && kk < k_end) v = *reinterpret_cast<const u32x4*>(W + (size_t)(n0 + row) * K + kk);
-            rw[i] = v;
+            u32x4 v = *reinterpret_cast<const u32x4*>(in ? pw[i] + k0 : W);
+            rw[i] = (u32x4){v[0] & keep, v[1] & keep, v[2] & keep, v[3] & keep};
         }
     };
     auto store_lds = [&](int buf) {
@@ -99,14 +122,17 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
         for (int j = 0; j < TN; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     // a slice of K per blockIdx.y: partial sums that the consumer adds in slice order
-    const int k_begin = blockIdx.y * ep.k_per_split;
+    const int k_begin = split * ep.k_per_split;
     const int nk = ceil_div(k_end - k_begin, BK);
-    load_global(k_begin);
+    const bool partial = (k_end - k_begin) % BK != 0;  // the last step is a partial one
+    if (nk == 1 && partial) load_global_tail(k_begin);
+    else load_global(k_begin);
     store_lds(0);
     __syncthreads();
     for (int kt = 0; kt < nk; ++kt) {
         const int buf = kt & 1;
-        if (kt + 1 < nk) load_global(k_begin + (kt + 1) * BK);
+        if (kt + 2 < nk || (kt + 2 == nk && !partial)) load_global(k_begin + (kt + 1) * BK);
+        else if (kt + 1 < nk) load_global_tail(k_begin + (kt + 1) * BK);
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 32) {
             Frag fa[TM], fb[TN];
@@ -123,44 +149,53 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
         __syncthreads();
     }
 
-    // Epilogue.  Lane holds rows grp * 4 + i of column r16 in each 16x16 tile.
+    // Epilogue.  Lane holds rows grp * 4 + e of column r16 in each 16x16 tile: sixteen lanes write
+    // sixteen consecutive elements of a row.  (Four consecutive columns a lane - transposed tiles,
+    // one 8-byte store - measured slower: neighbouring lanes then write to different rows, which
+    // the memory pipeline does not merge.)  A tile wholly inside the output stores without checks:
+    // sixty-four guarded stores cost a third of a whole 2,048 x 9,728 x 896 product.
     const int row_base = m0 + wm * (BM / WM) + grp * 4;
     const int col_base = n0 + wn * (BN / WN) + r16;
-    if constexpr (EPI == EPI_SWIGLU) {
-        static_assert(TN % 2 == 0, "gate and up tiles come in pairs");
-        elem_t* out = reinterpret_cast<elem_t*>(ep.out);
+    const bool whole = m0 + BM <= M && n0 + BN <= N && (EPI != EPI_SWIGLU || (n0 + BN) / 2 <= ep.n_out);
+    auto emit = [&](auto checked) {
+        constexpr bool CHECKED = decltype(checked)::value;
+        if constexpr (EPI == EPI_SWIGLU) {
+            static_assert(TN % 2 == 0, "gate and up tiles come in pairs");
+            elem_t* out = reinterpret_cast<elem_t*>(ep.out);
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; j += 2) {
-                const int col = (col_base + j * 16 - r16) / 2 + r16;  // tiles 2t, 2t+1 -> output tile t
+                for (int j = 0; j < TN; j += 2) {
+                    const int col = (col_base + j * 16 - r16) / 2 + r16;  // tiles 2t, 2t+1 -> output tile t
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int row = row_base + i * 16 + e;
-                    if (row < M && col < ep.n_out)
+                    for (int e = 0; e < 4; ++e) {
+                        const int row = row_base + i * 16 + e;
+                        if (CHECKED && !(row < M && col < ep.n_out)) continue;
                         out[(size_t)row * ep.ldo + col] = from_f32<elem_t>(silu_f(acc[i][j][e]) * acc[i][j + 1][e]);
+                    }
                 }
-            }
-    } else {
+        } else {
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const int col = col_base + j * 16;
-                if (col >= N) continue;
-                const float b = ep.bias ? ep.bias[col] : 0.f;
+                for (int j = 0; j < TN; ++j) {
+                    const int col = col_base + j * 16;
+                    const float b = ep.bias ? ep.bias[min(col, N - 1)] : 0.f;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int row = row_base + i * 16 + e;
-                    if (row >= M) continue;
-                    const size_t o = (size_t)row * ep.ldo + col;
-                    const float v = acc[i][j][e] + b;
-                    if constexpr (EPI == EPI_STORE_F32) reinterpret_cast<float*>(ep.out)[blockIdx.y * ep.split_stride + o] = v;
-                    else if constexpr (EPI == EPI_STORE_ELEM) reinterpret_cast<elem_t*>(ep.out)[o] = from_f32<elem_t>(v);
-                    else reinterpret_cast<float*>(ep.out)[o] += v;  // residual stream, 32-bit
+                    for (int e = 0; e < 4; ++e) {
+                        const int row = row_base + i * 16 + e;
+                        if (CHECKED && !(row < M && col < N)) continue;
+                        const size_t o = (size_t)row * ep.ldo + col;
+                        const float v = acc[i][j][e] + b;
+                        if constexpr (EPI == EPI_STORE_F32) reinterpret_cast<float*>(ep.out)[split * ep.split_stride + o] = v;
+                        else if constexpr (EPI == EPI_STORE_ELEM) reinterpret_cast<elem_t*>(ep.out)[o] = from_f32<elem_t>(v);
+                        else reinterpret_cast<float*>(ep.out)[o] += v;  // residual stream, 32-bit
+                    }
                 }
-            }
-    }
+        }
+    };
+    if (whole) emit(std::false_type{});
+    else emit(std::true_type{});
 }
 
 static int g_gemm_config = 0;  // 0: chosen by shape; else a fixed tile (measurements only)
@@ -191,16 +226,19 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
     if (forced == 2) MS_GEMM(128, 128, 2, 2, 64);
     if (forced == 5) MS_GEMM(128, 64, 2, 2, 64);
     if (forced == 6) MS_GEMM(64, 64, 2, 2, 64);
-    // The largest tile that still gives every CU of the chip a block or two; a K step of 64 (half
-    // the barriers) where the K loop is long enough to pay for the larger tiles in LDS.  Measured
-    // on M = 512..8192 of the 0.5B shapes; larger wave tiles (256x128) lose to register pressure.
+    // The largest tile that still gives every CU of the chip a block or two, with K steps of 64 (half
+    // the barriers of steps of 32).  Measured on M = 512..8192 of the 0.5B shapes; larger wave tiles
+    // (256x128) lose: their accumulators no longer fit the registers of two blocks a CU.
     if (M > 64) {
         const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128), b12864 = (long)ceil_div(M, 128) * ceil_div(N, 64);
         if (b128 * ns >= 300) {
-            if (ep.k_per_split >= 1024) MS_GEMM(128, 128, 2, 2, 64);
+            if (ep.k_per_split >= 128) MS_GEMM(128, 128, 2, 2, 64);
             MS_GEMM(128, 128, 2, 2, 32);
         }
-        if (b12864 * ns >= 300) MS_GEMM(128, 64, 2, 2, 32);
+        if (b12864 * ns >= 300) {
+            if (ep.k_per_split >= 128) MS_GEMM(128, 64, 2, 2, 64);
+            MS_GEMM(128, 64, 2, 2, 32);
+        }
     }
     MS_GEMM(64, 64, 2, 2, 64);
 #else
