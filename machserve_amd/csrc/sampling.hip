@@ -36,6 +36,7 @@ struct SampleArgs {
     // per-row partial maxima of ARGMAX_CHUNKS chunks of the row, or null: a greedy row scans itself
     const float* part_val;
     const int* part_idx;
+    int* also_token;  // [W] or null: a second place for the tokens (the next step's input, on the device)
 };
 
 constexpr int ARGMAX_CHUNKS = 64;
@@ -115,6 +116,7 @@ __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs a) {
             }
             if (tid == 0) {
                 a.out_token[r] = bi;
+                if (a.also_token) a.also_token[r] = bi;
                 a.out_logprob[r] = 0.0f;
             }
         }
@@ -145,6 +147,7 @@ __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs a) {
                 }
             }
             a.out_token[r] = bi;
+            if (a.also_token) a.also_token[r] = bi;
             a.out_logprob[r] = 0.0f;
         }
         return;
@@ -238,6 +241,7 @@ __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs a) {
             if (found < 0) found = 0;
         }
         a.out_token[r] = found;
+        if (a.also_token) a.also_token[r] = found;
         a.out_logprob[r] = (row[found] - maxv) * inv_t - logf(tot);
     }
 }
@@ -332,7 +336,7 @@ extern "C" int ms_sample_chunks() { return ARGMAX_CHUNKS; }
 
 extern "C" int ms_sample(const float* logits, const float* temperature, const int* top_k, const float* top_p,
                          unsigned long long* state, int* out_token, float* out_logprob, float* part_val, int* part_idx,
-                         int rows, int vocab, hipStream_t stream) {
+                         int* also_token, int rows, int vocab, hipStream_t stream) {
     MS_REQUIRE(rows > 0 && vocab > 0, "sample: empty problem rows=%d vocab=%d", rows, vocab);
     static_assert(ARGMAX_CHUNKS <= WAVE, "stage two is one wave");
     if (part_val && part_idx) {
@@ -343,7 +347,7 @@ extern "C" int ms_sample(const float* logits, const float* temperature, const in
         part_val = nullptr;
         part_idx = nullptr;
     }
-    SampleArgs a{logits, temperature, top_k, top_p, state, out_token, out_logprob, vocab, part_val, part_idx};
+    SampleArgs a{logits, temperature, top_k, top_p, state, out_token, out_logprob, vocab, part_val, part_idx, also_token};
     hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(ST), 0, stream, a);
     return check_launch("sample");
 }

@@ -46,12 +46,14 @@ class _DecodeGraph:
 @dataclass
 class LaunchedDecode:
     """A decode step that runs on the device: its requests' slots, the device tensor that will hold
-    its samples (int32 ``[2, B]``: tokens, bits of the logprobs), the pinned copy of it, and the
-    event after that copy."""
+    its samples (int32 ``[2, B]``: tokens, bits of the logprobs), the pinned copy of it, the
+    event after that copy, and the captured graph that ran it (whose token section holds the
+    sampled tokens as well)."""
     slots: List[int]
     sampled: torch.Tensor
     result: torch.Tensor
     done: object
+    graph: object
 
 
 class StepFunction:
@@ -126,12 +128,13 @@ class StepFunction:
         return self._context_from(dev, offsets, widths, lists)
 
     # ------------------------------------------------------------------ captured decode steps
-    def _run_decode_graph(self, entries: Sequence[StepEntry], sampling=None, device_tokens: Optional[torch.Tensor] = None):
+    def _run_decode_graph(self, entries: Sequence[StepEntry], sampling=None, after: Optional["LaunchedDecode"] = None):
         """Replay (or first capture) the graph of this batch size.  ``sampling`` = (temperatures,
         top_ks, top_ps, states) makes sampling part of the graph; the result is then the int32
-        ``[2, B]`` tensor of :meth:`HipOps.sample_packed`, else the logits.  With ``device_tokens``
-        (int32, one per entry, on the device) the step's tokens are taken from there and the
-        entries' own tokens are placeholders."""
+        ``[2, B]`` tensor of :meth:`HipOps.sample_packed`, else the logits.  With ``after`` (the
+        launched step before this one, of the same requests) the step's tokens are that step's
+        samples, on the device, and the entries' own tokens are placeholders.  Returns the result
+        and the graph."""
         slots, counts, tokens, _ = self._check_entries(entries)
         B = len(slots)
         host, offsets, widths = self.cache.build_step(slots, counts, tokens, list(range(B)), self.heads_per_kv,
@@ -161,11 +164,18 @@ class StepFunction:
         staged[:host.size] = host
         for k, a in extra.items():
             staged[dg.offsets[k][0]:dg.offsets[k][0] + a.size] = a
-        dg.dev.copy_(dg.pinned, non_blocking=True)
+        start, size = dg.offsets["tokens"]
+        if after is not None and after.graph is dg:
+            # the sampling kernel of this graph's last replay left its tokens in the graph's own
+            # token section: everything but that section is uploaded
+            if start:
+                dg.dev[:start].copy_(dg.pinned[:start], non_blocking=True)
+            dg.dev[start + size:].copy_(dg.pinned[start + size:], non_blocking=True)
+        else:
+            dg.dev.copy_(dg.pinned, non_blocking=True)
+            if after is not None:  # another graph ran that step (the block tables have grown a bucket)
+                dg.dev[start:start + size].copy_(after.sampled[0])
         dg.copied.record()
-        if device_tokens is not None:
-            start, size = dg.offsets["tokens"]
-            dg.dev[start:start + size].copy_(device_tokens)
         if dg.graph is None:
             ctx = self._context_from(dg.dev, dg.offsets, widths)
             side = torch.cuda.Stream(device=self.rt.device)
@@ -181,11 +191,12 @@ class StepFunction:
                 if sampling is not None:
                     dg.sampled = self.rt.ops.sample_packed(
                         dg.logits, sec("sample/temperature").view(torch.float32), sec("sample/top_k"),
-                        sec("sample/top_p").view(torch.float32), sec("sample/state").view(torch.int64), True)
+                        sec("sample/top_p").view(torch.float32), sec("sample/state").view(torch.int64), True,
+                        also_tokens=sec("tokens"))
             dg.graph = graph
             self._graphs[key] = dg
         dg.graph.replay()
-        return dg.sampled if sampling is not None else dg.logits
+        return (dg.sampled if sampling is not None else dg.logits), dg
 
     def decode_and_sample(self, entries: Sequence[StepEntry], temperatures, top_ks, top_ps, states):
         """A decode-only step (one token per request) with sampling inside the captured graph: one
@@ -216,8 +227,7 @@ class StepFunction:
                 raise OutOfPages(f"group {k}: the step needs {v} new pages, {cache.free_pages(k)} are free")
         for e in entries:
             cache.extend(e.slot, 1)
-        sampled = self._run_decode_graph(entries, (temperatures, top_ks, top_ps, states),
-                                         None if after is None else after.sampled[0])
+        sampled, graph = self._run_decode_graph(entries, (temperatures, top_ks, top_ps, states), after)
         for e in entries:
             cache.commit(e.slot, 1)
         # the samples go to a pinned buffer of their own (the graph's is overwritten by its next replay)
@@ -229,7 +239,7 @@ class StepFunction:
         result.copy_(sampled, non_blocking=True)
         done = torch.cuda.Event()
         done.record()
-        return LaunchedDecode(slots, sampled, result, done)
+        return LaunchedDecode(slots, sampled, result, done, graph)
 
     def collect(self, launched: "LaunchedDecode"):
         """``(tokens, logprobs)`` of a launched step as host lists; waits for them."""
@@ -255,7 +265,7 @@ class StepFunction:
         for e in entries:
             cache.extend(e.slot, len(e.tokens))
         if self.use_graphs and all(len(e.tokens) == 1 for e in entries) and len({e.slot for e in entries}) == len(entries):
-            logits = self._run_decode_graph(entries)
+            logits, _ = self._run_decode_graph(entries)
             wanted = [i for i, e in enumerate(entries) if len(e.want)]
             if not wanted:
                 logits = None

@@ -384,17 +384,20 @@ class HipOps:
         return both[0], both[1].view(torch.float32)
 
     def sample_packed(self, logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-                      state: torch.Tensor, any_greedy: bool = True) -> torch.Tensor:
+                      state: torch.Tensor, any_greedy: bool = True, also_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         """:meth:`sample` with both results in one int32 tensor ``[2, W]`` (tokens, then the bits of
         the logprobs) so that one copy brings them to the host.  With ``any_greedy`` a first
         launch finds the maxima of 64 chunks of every row, so that a greedy row is not one
-        block's serial scan."""
+        block's serial scan.  ``also_tokens`` (int32 ``[W]``) receives the tokens as well: the
+        place where a following step reads its input."""
         W, V = logits.shape
         self._want(logits, torch.float32, "sample logits")
         self._want(temperature, torch.float32, "sample temperature", W)
         self._want(top_k, torch.int32, "sample top_k", W)
         self._want(top_p, torch.float32, "sample top_p", W)
         self._want(state, torch.int64, "sample state", W)
+        if also_tokens is not None:
+            self._want(also_tokens, torch.int32, "sample also_tokens", W)
         both = torch.empty((2, W), dtype=torch.int32, device=logits.device)  # tokens, then logprob bits
         tok, lp = both[0], both[1].view(torch.float32)
         pv = pi = None
@@ -403,8 +406,8 @@ class HipOps:
             pv = torch.empty((W, chunks), dtype=torch.float32, device=logits.device)
             pi = torch.empty((W, chunks), dtype=torch.int32, device=logits.device)
         self._check(self._core, self._core.ms_sample(_ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p),
-                                                     _ptr(state), _ptr(tok), _ptr(lp), _ptr(pv), _ptr(pi), _c_int(W),
-                                                     _c_int(V), _stream()))
+                                                     _ptr(state), _ptr(tok), _ptr(lp), _ptr(pv), _ptr(pi),
+                                                     _ptr(also_tokens), _c_int(W), _c_int(V), _stream()))
         return both
 
     def top_logprobs(self, logits: torch.Tensor, inv_t: torch.Tensor, k: int):
