@@ -361,6 +361,49 @@ def test_decode_attention_fused(dtype, H, KV, hd, ps, window, P_):
         assert_close(vd, vp, dtype, "value pages")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,KV,hd,ps,window", [(14, 2, 64, 64, None), (4, 1, 128, 16, None), (6, 2, 64, 32, 4000)])
+def test_attention_long_contexts(dtype, H, KV, hd, ps, window):
+    """Contexts of nine and twenty thousand keys: a decoded row (many splits, merged in batches) and
+    a portion of a prompt far into its request, with a key near the start (or at the window's
+    edge) that towers over the rest, so that a range of keys that went missing would show."""
+    ops, emu = ops_for(dtype), EmulatedOps(dtype)
+    lens = [20011, 9000, 5]
+    S = len(lens)
+    gen = torch.Generator().manual_seed(700 + hd)
+    n_pages = sum(-(-(c + 1) // ps) for c in lens) + 2
+    order = torch.randperm(n_pages, generator=gen).tolist()
+    kp, vp = rnd((n_pages, KV, ps, hd), dtype, 701), rnd((n_pages, KV, hd, ps), dtype, 702)
+    width = max(-(-(c + 1) // ps) for c in lens)
+    table = torch.full((S, width), -1, dtype=torch.int32)
+    for i, c in enumerate(lens):
+        for p in range(-(-(c + 1) // ps)):
+            table[i, p] = order.pop()
+    q = rnd((S, H * hd), dtype, 703)
+    for i in (0, 1):
+        far = 2 if not window else lens[i] - window + 1
+        qv = q[i, (H - 1) * hd:].float()
+        kp[int(table[i, far // ps]), KV - 1, far % ps, :] = (qv / qv.norm() * 8.0).to(dtype)
+        q[i, (H - 1) * hd:] = (qv / qv.norm() * 8.0 * math.sqrt(hd) / 4).to(dtype)
+    pos0 = torch.tensor(lens, dtype=torch.int32)
+    ref = emu.decode_attention(q, kp, vp, table, pos0, H, KV, hd, ps, window, hd ** -0.5)
+    got = ops.decode_attention(q.to(DEV), kp.to(DEV), vp.to(DEV), table.to(DEV), pos0.to(DEV), H, KV, hd, ps, window, hd ** -0.5)
+    assert_close(got, ref, dtype, "decode attention over long contexts")
+    # the last 150 positions of the 9,000-key request as one portion
+    n, c = 150, lens[1] + 1 - 150
+    g = H // KV
+    qq = rnd((n, H * hd), dtype, 704)
+    qq[n - 1] = q[1]
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32)
+    args = (i32([0]), i32([n]), i32([c]), i32([(0, r0) for r0 in range(0, n * g, 64)]).view(-1, 2))
+    tab = table[1:2].contiguous()
+    ref2 = emu.paged_attention(qq, kp, vp, tab, *args, H, KV, hd, ps, window, hd ** -0.5)
+    got2 = ops.paged_attention(qq.to(DEV), kp.to(DEV), vp.to(DEV), tab.to(DEV), *[a.to(DEV) for a in args], H, KV, hd, ps,
+                               window, hd ** -0.5)
+    assert_close(got2, ref2, dtype, "a portion far into a long request")
+    assert_close(got2[n - 1:].float().cpu(), got[1:2].float().cpu(), dtype, "its last row against the decode kernel")
+
+
 def test_attention_equals_library_attention_without_rotation_or_paging():
     """One request, whole prompt, pages in order: the kernel is plain causal attention."""
     dtype = torch.float32
