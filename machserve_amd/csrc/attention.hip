@@ -61,9 +61,11 @@ struct AttnArgs {
     const int* seq_q_start;  // [S] first row of the request in this step
     const int* seq_q_len;    // [S] rows of the request in this step
     const int* seq_pos0;     // [S] position of its first row
-    const int* work;         // [W, 2] (request index, first flat row)
+    const int* work;         // [W, 2] (request index, first flat row), best with the longest contexts first
     int table_stride, H, KV, hd, ps, window;
     float scale;
+    int n_work;     // W
+    int pair_span;  // work items per round of blocks over the chip when two blocks share a CU, else 0
 };
 
 __device__ __forceinline__ float exp_f(float x) {
@@ -108,8 +110,15 @@ __global__ __launch_bounds__(256 * KG, attention_waves_per_simd<KG>()) void page
     auto stage_k = [&](int b) { return reinterpret_cast<elem_t*>(smem + (2 * kg + b) * STAGE_BYTES); };
     auto stage_v = [&](int b) { return stage_k(b) + KS_ELEMS; };
     const int r16 = lane & 15, grp = lane >> 4;
-    const int s = a.work[blockIdx.x * 2], r0 = a.work[blockIdx.x * 2 + 1];
-    const int kvh = blockIdx.y;
+    // Blocks are numbered item by item, the KV heads of an item side by side.  A block's work grows
+    // with its context, and blocks go to the CUs in turn: with two blocks a CU, block b shares its
+    // CU with block b + (number of CUs).  So the list's heaviest `pair_span` items come first, then
+    // its lightest ones, lightest first (each beside one of the heaviest), then the middle.
+    const int kvh = blockIdx.x % a.KV, turn = blockIdx.x / a.KV;
+    int item = turn;
+    if (a.pair_span > 0 && turn >= a.pair_span)
+        item = turn < 2 * a.pair_span ? a.n_work - 1 - (turn - a.pair_span) : turn - a.pair_span;
+    const int s = a.work[item * 2], r0 = a.work[item * 2 + 1];
     const int g = a.H / a.KV;
     const int q_start = a.seq_q_start[s], q_len = a.seq_q_len[s], pos0 = a.seq_pos0[s];
     const int R = q_len * g;
@@ -892,7 +901,7 @@ extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
     MS_REQUIRE(window >= 0, "attention: window %d", window);
     MS_REQUIRE((double)n_pages * KV * ps * hd < 68719476736.0, "attention: a pool of %d pages exceeds 2^36 elements", n_pages);
     AttnArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, (elem_t*)out, block_table, seq_q_start,
-               seq_q_len, seq_pos0, work, table_stride, H, KV, hd, ps, window, scale};
+               seq_q_len, seq_pos0, work, table_stride, H, KV, hd, ps, window, scale, n_work, 0};
     // key groups per block by the longest context the block tables allow (the lengths themselves
     // are on the device): short contexts have no chain worth cutting
     const long span = window > 0 ? (long)window + BKV : (long)table_stride * ps;
@@ -903,13 +912,32 @@ extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
     } else if (span < 4 * BKV) {
         groups = 1;
     }
-    const dim3 grid((unsigned)n_work, (unsigned)KV);
+    MS_REQUIRE((long)n_work * KV < 2147483647L, "attention: %d blocks of rows times %d key/value heads", n_work, KV);
+    const dim3 grid((unsigned)(n_work * KV));
+    // how many blocks of each variant a CU holds, and how many CUs there are: asked once
+    static int cus = 0, resident[3] = {0, 0, 0};
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1)
+            n = 256;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident[0], paged_attention_kernel<1>, 256, 0) != hipSuccess) resident[0] = 1;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident[1], paged_attention_kernel<2>, 512, 0) != hipSuccess) resident[1] = 1;
+        if constexpr (MAX_KEY_GROUPS >= 4) {
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident[2], paged_attention_kernel<4>, 1024, 0) != hipSuccess) resident[2] = 1;
+        }
+        (void)hipGetLastError();
+        cus = n;
+    }
+    auto span_for = [&](int variant) { return resident[variant] == 2 ? (cus / KV > 0 ? cus / KV : 1) : 0; };
     if (groups >= 4 && MAX_KEY_GROUPS >= 4) {
         // sixteen waves leave each 128 registers, which only the small bfloat16 tiles fit into
+        a.pair_span = span_for(2);
         if constexpr (MAX_KEY_GROUPS >= 4) hipLaunchKernelGGL(paged_attention_kernel<4>, grid, dim3(1024), 0, stream, a);
     } else if (groups >= 2) {
+        a.pair_span = span_for(1);
         hipLaunchKernelGGL(paged_attention_kernel<2>, grid, dim3(512), 0, stream, a);
     } else {
+        a.pair_span = span_for(0);
         hipLaunchKernelGGL(paged_attention_kernel<1>, grid, dim3(256), 0, stream, a);
     }
     return check_launch("paged_attention");

@@ -289,13 +289,22 @@ public:
             add("slot_map/" + g.name, std::move(slot_map));
             widths[py::str(g.name)] = width;
         }
+        // Blocks of rows for the attention kernels, those with the longest contexts first: a block's
+        // work grows with the keys its last row sees, and the kernel spreads the blocks over the chip
+        // by their place in this order.
         for (int hk : heads_per_kv) {
-            std::vector<int32_t> work;
+            struct Item { int keys, seq, r0; };
+            std::vector<Item> items;
             for (int i = 0; i < S; ++i)
-                for (int r0 = 0; r0 < counts[i] * hk; r0 += rows_per_block) {
-                    work.push_back(i);
-                    work.push_back(r0);
-                }
+                for (int r0 = 0; r0 < counts[i] * hk; r0 += rows_per_block)
+                    items.push_back({pos0[i] + std::min(counts[i], (r0 + rows_per_block + hk - 1) / hk), i, r0});
+            std::stable_sort(items.begin(), items.end(), [](const Item& a, const Item& b) { return a.keys > b.keys; });
+            std::vector<int32_t> work;
+            work.reserve(items.size() * 2);
+            for (const Item& it : items) {
+                work.push_back(it.seq);
+                work.push_back(it.r0);
+            }
             add("work/" + std::to_string(hk), std::move(work));
         }
         size_t total = 0;
