@@ -46,6 +46,12 @@ class Engine:
                 raise ValueError(f"token {t} is outside the vocabulary of {vocab}")
         return self.scheduler.add(prompt, max_new, params, eos, stop_seqs)
 
+    def cancel(self, rid: int) -> bool:
+        """End a request now (reason ``"cancelled"``); its pages and slot go back at once.  A token that
+        a step in flight still computes for it is dropped.  False if the request is not live
+        (``continuous.rs:1266-1292``)."""
+        return self.scheduler.cancel(rid)
+
     def has_work(self) -> bool:
         return self.scheduler.has_work() or self._inflight is not None
 

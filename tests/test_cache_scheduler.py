@@ -369,3 +369,34 @@ def test_pipelined_steps_give_what_synchronous_steps_give(tmp_path, pages):
         b, n_dev, _ = run(True, **kw)
         assert a == b and n_dev > 0
         assert "stop" in [r for _, r, _ in a]
+
+
+def test_cancel_while_a_step_is_in_flight(tmp_path):
+    """A request cancelled between two launches: the token the step in flight computes for it is
+    dropped, the others go on as if it had never been there, and its pages are back at once."""
+    from machserve_amd.engine import Engine, load_model
+    from machserve_amd.sampling import SamplingParams
+    d = make_model_dir(tmp_path, "A")
+    prompts = [random_prompt(n, 512, 30 + n) for n in (6, 11)]
+
+    def run(cancel_at):
+        lm = load_model(d, dtype="float32", device="cpu", page_size=16, num_pages=8, max_requests=2, ops=EmulatedOps())
+        eng = Engine(lm, max_batch_tokens=32)
+        _LaggedDecode(eng)
+        ids = [eng.add(p, 12, SamplingParams(temperature=0.9, seed=4 + i)) for i, p in enumerate(prompts)]
+        n = 0
+        while eng.has_work():
+            eng.step_pipelined()
+            n += 1
+            if n == cancel_at:
+                assert eng._inflight is not None, "the cancellation is meant to meet a step in flight"
+                free = lm.cache.groups["full"].pool.available()
+                assert eng.cancel(ids[1]) and not eng.cancel(ids[1])
+                assert lm.cache.groups["full"].pool.available() > free
+            lm.cache.check()
+        done = eng.scheduler.finished
+        return [(done[i].generated, done[i].finish_reason) for i in ids]
+
+    whole, cut = run(None), run(5)
+    assert cut[0] == whole[0] and whole[0][1] == "length"
+    assert cut[1][1] == "cancelled" and 0 < len(cut[1][0]) < 12 and cut[1][0] == whole[1][0][:len(cut[1][0])]
