@@ -66,6 +66,11 @@ struct AttnArgs {
     float scale;
     int n_work;     // W
     int pair_span;  // work items per round of blocks over the chip when two blocks share a CU, else 0
+    // the keys of a block cut over gridDim.y blocks (few blocks of rows, long contexts): each writes
+    // its unnormalised output and (max, sum) per row, and decode_merge_kernel adds them up
+    int nsplit;
+    float* part_o;   // [T, H, nsplit, hd]
+    float* part_ml;  // [T, H, nsplit, 2]
 };
 
 __device__ __forceinline__ float exp_f(float x) {
@@ -133,12 +138,44 @@ __global__ __launch_bounds__(256 * KG, attention_waves_per_simd<KG>()) void page
     const int pos = pos0 + tok;
     const bool wave_active = r0 + wave * 16 < R;
 
-    // keys any row of the block may see
+    // keys any row of the block may see, and of those the rounds of tiles that are this split's
+    constexpr int ROUND = KG * BKV;  // keys per round of the block
     const int last_row = min(r0 + ROWS_PER_BLOCK, R) - 1;
-    const int kv_hi = pos0 + last_row / g + 1;
+    int kv_hi = pos0 + last_row / g + 1;
     int kv_lo = 0;
     if (a.window > 0) kv_lo = max(0, pos0 + r0 / g - a.window + 1);
     const int lo_key = a.window > 0 ? pos - a.window + 1 : 0;
+    const int sp = blockIdx.y;
+    if (a.nsplit > 1) {
+        const int first = (kv_lo / ROUND) * ROUND;
+        const int per = ceil_div(ceil_div(kv_hi - first, ROUND), a.nsplit) * ROUND;
+        kv_lo = max(kv_lo, first + sp * per);
+        kv_hi = min(kv_hi, first + (sp + 1) * per);
+    }
+    // a row's partial result of this split (group 0 writes, after the groups have been merged)
+    auto write_partial = [&](const f32x4* o, float m, float l) {
+        const size_t base = (((size_t)(q_start + tok)) * a.H + head) * a.nsplit + sp;
+        float* po = a.part_o + base * hd;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) {
+            const int d0 = dt * 16 + grp * 4;
+            if (d0 < hd) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) po[d0 + i] = o[dt][i];
+            }
+        }
+        // the merge takes maxima in natural-logarithm units of the scaled scores
+        if (grp == 0) { a.part_ml[base * 2] = m * a.scale; a.part_ml[base * 2 + 1] = l; }
+    };
+    if (kv_lo >= kv_hi) {  // nothing for this split (the same for every thread of the block)
+        if (a.nsplit > 1 && threadIdx.x < 256 && valid) {
+            f32x4 zero[ND];
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt) zero[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            write_partial(zero, NEG_BIG, 0.f);
+        }
+        return;
+    }
 
     Frag qf[NKS];
     {
@@ -191,7 +228,6 @@ __global__ __launch_bounds__(256 * KG, attention_waves_per_simd<KG>()) void page
     // is about to use, and the younger tiles stay in flight.  The page of a tile's 16-key group is
     // read one round before its offsets are needed; which logical page that is, is stepped from
     // round to round rather than divided out.
-    constexpr int ROUND = KG * BKV;  // keys per round of the block
     const int tsub = tid % NT;
     const int round_pages = ROUND / ps, round_rem = ROUND % ps;
     int key_next, lp_next, off_next;  // this thread's 16-key group of the next tile to look up
@@ -434,7 +470,9 @@ __global__ __launch_bounds__(256 * KG, attention_waves_per_simd<KG>()) void page
         }
     }
 
-    if (valid) {
+    if (valid && a.nsplit > 1) {
+        write_partial(acc_o, m_run, l_run);
+    } else if (valid) {
         const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
         elem_t* orow = a.out + ((size_t)(q_start + tok) * a.H + head) * hd;
 #pragma unroll
@@ -889,19 +927,25 @@ using namespace ms;
 // Attention of a mixed batch.  `work` lists (request index, first flat row) for every block
 // of 64 flat rows; see the file comment.  window = 0 means all keys.  max_key_groups = 0 lets the
 // launcher choose how many key groups share a block (1, 2 or 4) from the width of the block tables;
-// a positive value asks for that many (as far as this tile has them).
+// a positive value asks for that many (as far as this tile has them).  nsplit > 1 cuts every block's
+// keys over that many blocks (few blocks of rows over long contexts would leave most of the chip idle
+// and run as long as their chain of tiles); T is the number of rows, part_o [T, H, nsplit, hd] and
+// part_ml [T, H, nsplit, 2] are float workspaces.
 extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
     const void* q, const void* kpool, const void* vpool, void* out, const int* block_table, int table_stride,
     const int* seq_q_start, const int* seq_q_len, const int* seq_pos0, const int* work, int n_work, int H, int KV,
-    int hd, int ps, int n_pages, int window, float scale, int max_key_groups, hipStream_t stream) {
+    int hd, int ps, int n_pages, int window, float scale, int max_key_groups, int T, int nsplit, float* part_o,
+    float* part_ml, hipStream_t stream) {
     MS_REQUIRE(n_work > 0, "attention: no work");
+    MS_REQUIRE(nsplit >= 1 && nsplit <= MAX_SPLITS && (nsplit == 1 || (part_o && part_ml && T > 0)),
+               "attention: %d key splits (at most %d, with their workspaces)", nsplit, MAX_SPLITS);
     MS_REQUIRE(hd % 16 == 0 && hd > 0 && hd <= HDT, "attention: head size %d does not fit this tile of %d", hd, HDT);
     MS_REQUIRE(KV > 0 && H % KV == 0, "attention: %d heads are not a multiple of %d key/value heads", H, KV);
     MS_REQUIRE(ps % 16 == 0 && ps > 0, "attention: page size %d must be a multiple of 16", ps);
     MS_REQUIRE(window >= 0, "attention: window %d", window);
     MS_REQUIRE((double)n_pages * KV * ps * hd < 68719476736.0, "attention: a pool of %d pages exceeds 2^36 elements", n_pages);
     AttnArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, (elem_t*)out, block_table, seq_q_start,
-               seq_q_len, seq_pos0, work, table_stride, H, KV, hd, ps, window, scale, n_work, 0};
+               seq_q_len, seq_pos0, work, table_stride, H, KV, hd, ps, window, scale, n_work, 0, nsplit, part_o, part_ml};
     // key groups per block by the longest context the block tables allow (the lengths themselves
     // are on the device): short contexts have no chain worth cutting
     const long span = window > 0 ? (long)window + BKV : (long)table_stride * ps;
@@ -913,7 +957,7 @@ extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
         groups = 1;
     }
     MS_REQUIRE((long)n_work * KV < 2147483647L, "attention: %d blocks of rows times %d key/value heads", n_work, KV);
-    const dim3 grid((unsigned)(n_work * KV));
+    const dim3 grid((unsigned)(n_work * KV), (unsigned)nsplit);
     // how many blocks of each variant a CU holds, and how many CUs there are: asked once
     static int cus = 0, resident[3] = {0, 0, 0};
     if (cus == 0) {
@@ -940,7 +984,10 @@ extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
         a.pair_span = span_for(0);
         hipLaunchKernelGGL(paged_attention_kernel<1>, grid, dim3(256), 0, stream, a);
     }
-    return check_launch("paged_attention");
+    int rc = check_launch("paged_attention");
+    if (rc || nsplit == 1) return rc;
+    hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)((size_t)T * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit);
+    return check_launch("attention_merge");
 }
 
 extern "C" int MS_CAT(ms_attention_rows_per_block_nd, MS_ATTN_ND)() { return ROWS_PER_BLOCK; }

@@ -12,6 +12,7 @@ device once; everything after that is kernel launches on one stream.
 """
 from __future__ import annotations
 
+from collections import OrderedDict
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence
 
@@ -34,8 +35,9 @@ class StepEntry:
 
 
 class _DecodeGraph:
-    """One captured decode step for a fixed number of requests and fixed block-table widths:
-    a static int32 buffer the host refills before every replay, and the logits it produces."""
+    """One captured step for fixed numbers of tokens per request, of wanted rows and fixed
+    block-table widths: a static int32 buffer the host refills before every replay, and the
+    logits it produces."""
 
     def __init__(self, graph, dev, pinned, offsets, widths, logits):
         self.graph, self.dev, self.pinned, self.offsets, self.widths, self.logits = graph, dev, pinned, offsets, widths, logits
@@ -57,17 +59,25 @@ class LaunchedDecode:
 
 
 class StepFunction:
-    TABLE_BUCKET = 8  # captured block tables are this many pages wide, or a multiple
+    TABLE_BUCKET = 8        # captured block tables are this many pages wide, or a multiple
+    MAX_GRAPHS = 48         # captured steps kept; the one unused longest goes first
+    CAPTURE_MAX_ROWS = 128  # a step of more rows keeps the device busy longer than the host needs to launch it
+    CAPTURE_AFTER = 3       # a shape other than plain decoding is captured when it has come this often before
 
     def __init__(self, model, cache: CacheManager, rt, attention_rows_per_block: int = 64, use_graphs: bool = True):
         self.model, self.cache, self.rt = model, cache, rt
         self.rows_per_block = attention_rows_per_block
         self.heads_per_kv = model.attention_rows_per_token()
-        # a decode step is launch-bound; it is captured once per batch size into a HIP graph and
-        # replayed.  Only for models whose parts read nothing but device memory from the context.
+        # A step of few tokens is bound by its launches: it is captured into a HIP graph and replayed.
+        # A decode step (one token a request) at its first occurrence; any other step of few rows
+        # when its shape (tokens per request, wanted rows, table widths) keeps coming, as it does
+        # while a long prompt is fed in small portions beside the same decoding requests (a
+        # capture costs as much as a few dozen launched steps, so a shape must earn it).  Only for
+        # models whose parts read nothing but device memory from the context.
         self.use_graphs = (use_graphs and rt.device.type == "cuda"
                            and all(getattr(b.mixer, "graph_safe", False) for b in getattr(model, "blocks", [])))
-        self._graphs: Dict[tuple, _DecodeGraph] = {}
+        self._graphs: "OrderedDict[tuple, _DecodeGraph]" = OrderedDict()
+        self._seen: Dict[tuple, int] = {}
         self._results: Dict[int, list] = {}  # pinned buffers for the samples, three per batch size, in turn
         self._launches = 0
 
@@ -129,18 +139,24 @@ class StepFunction:
 
     # ------------------------------------------------------------------ captured decode steps
     def _run_decode_graph(self, entries: Sequence[StepEntry], sampling=None, after: Optional["LaunchedDecode"] = None):
-        """Replay (or first capture) the graph of this batch size.  ``sampling`` = (temperatures,
-        top_ks, top_ps, states) makes sampling part of the graph; the result is then the int32
-        ``[2, B]`` tensor of :meth:`HipOps.sample_packed`, else the logits.  With ``after`` (the
-        launched step before this one, of the same requests) the step's tokens are that step's
-        samples, on the device, and the entries' own tokens are placeholders.  Returns the result
-        and the graph."""
+        """Replay (or first capture) the graph of a decode step; every row's logits are computed.
+        ``sampling`` = (temperatures, top_ks, top_ps, states) makes sampling part of the graph;
+        the result is then the int32 ``[2, B]`` tensor of :meth:`HipOps.sample_packed`, else the
+        logits.  With ``after`` (the launched step before this one, of the same requests) the
+        step's tokens are that step's samples, on the device, and the entries' own tokens are
+        placeholders.  Returns the result and the graph."""
         slots, counts, tokens, _ = self._check_entries(entries)
-        B = len(slots)
-        host, offsets, widths = self.cache.build_step(slots, counts, tokens, list(range(B)), self.heads_per_kv,
-                                                      self.rows_per_block, self.TABLE_BUCKET)
-        # for a given number of requests and given table widths the layout is always the same
-        key = (B, tuple(sorted(widths.items())), sampling is not None)
+        built = self.cache.build_step(slots, counts, tokens, list(range(len(slots))), self.heads_per_kv,
+                                      self.rows_per_block, self.TABLE_BUCKET)
+        return self._run_graph(self._graph_key(counts, len(slots), built[2], sampling is not None), built, sampling, after)
+
+    @staticmethod
+    def _graph_key(counts, n_want: int, widths, sampled: bool) -> tuple:
+        # for given tokens per request, wanted rows and table widths the buffer's layout is always the same
+        return (tuple(counts), n_want, tuple(sorted(widths.items())), sampled)
+
+    def _run_graph(self, key: tuple, built, sampling=None, after: Optional["LaunchedDecode"] = None):
+        host, offsets, widths = built
         extra: Dict[str, np.ndarray] = {}
         if sampling is not None:
             temps, top_ks, top_ps, states = sampling
@@ -149,6 +165,8 @@ class StepFunction:
             extra["sample/top_k"] = np.asarray(top_ks, dtype=np.int32)
             extra["sample/state"] = np.asarray(states, dtype=np.uint64).view(np.int32)
         dg = self._graphs.get(key)
+        if dg is not None:
+            self._graphs.move_to_end(key)
         if dg is None:
             offsets = dict(offsets)
             total = host.size
@@ -195,6 +213,8 @@ class StepFunction:
                         also_tokens=sec("tokens"))
             dg.graph = graph
             self._graphs[key] = dg
+            while len(self._graphs) > self.MAX_GRAPHS:
+                self._graphs.popitem(last=False)
         dg.graph.replay()
         return (dg.sampled if sampling is not None else dg.logits), dg
 
@@ -273,6 +293,29 @@ class StepFunction:
                 logits = logits[torch.tensor(wanted, device=logits.device)]
             elif not borrow_logits:
                 logits = logits.clone()  # the graph's own buffer is overwritten by its next replay
+        elif self.use_graphs:
+            slots, counts, tokens, want = self._check_entries(entries)
+            # block tables as wide as the next power of two of pages: a prompt that grows by a
+            # portion a step keeps its shape for many steps
+            pages = max(-(-(cache.length(sl) + n) // cache.page_size) for sl, n in zip(slots, counts))
+            width = self.TABLE_BUCKET
+            while width < pages:
+                width *= 2
+            try:
+                built = cache.build_step(slots, counts, tokens, want, self.heads_per_kv, self.rows_per_block, width)
+            except CacheError as e:
+                raise StepError(str(e)) from e
+            key = self._graph_key(counts, len(want), built[2], False)
+            if len(tokens) <= self.CAPTURE_MAX_ROWS and (key in self._graphs or self._seen.get(key, 0) >= self.CAPTURE_AFTER):
+                logits, _ = self._run_graph(key, built)
+                if logits is not None and not borrow_logits:
+                    logits = logits.clone()
+            else:  # a shape seen for the first time runs as it is: most shapes never come again
+                if len(self._seen) > 4096:
+                    self._seen.clear()
+                self._seen[key] = self._seen.get(key, 0) + 1
+                host, offsets, widths = built
+                logits = self.model.forward(self._context_from(torch.from_numpy(host).to(self.rt.device), offsets, widths))
         else:
             logits = self.model.forward(self.build_context(entries))
         for e in entries:

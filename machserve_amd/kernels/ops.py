@@ -277,8 +277,10 @@ class HipOps:
     def paged_attention(self, q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
                         seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_pos0: torch.Tensor,
                         work: torch.Tensor, H: int, KV: int, hd: int, page_size: int, window: Optional[int],
-                        scale: float, max_key_groups: int = 0) -> torch.Tensor:
-        """``max_key_groups`` asks for that many groups of waves sharing a block's keys (0: the kernel's choice)."""
+                        scale: float, max_key_groups: int = 0, key_splits: int = 0) -> torch.Tensor:
+        """``max_key_groups`` asks for that many groups of waves sharing a block's keys (0: the kernel's
+        choice); ``key_splits`` for that many blocks sharing them (0: by the number of blocks of rows
+        and the width of the block tables), merged by a second kernel."""
         lib, fn = self._attention_lib(hd)[:2]
         T = q.shape[0]
         self._want(q, self.dtype, "attention q", T, H * hd)
@@ -295,11 +297,29 @@ class HipOps:
         if work.dim() != 2 or work.shape[1] != 2 or work.shape[0] == 0:
             raise KernelError(f"attention: work list of shape {tuple(work.shape)}")
         out = torch.empty((T, H * hd), dtype=self.dtype, device=q.device)
+        nsplit = key_splits or self._portion_splits(work.shape[0] * KV, block_table.shape[1] * page_size, window)
+        part_o = part_ml = None
+        if nsplit > 1:
+            part_o = torch.empty((T, H, nsplit, hd), dtype=torch.float32, device=q.device)
+            part_ml = torch.empty((T, H, nsplit, 2), dtype=torch.float32, device=q.device)
         self._check(lib, fn(_ptr(q), _ptr(kpool), _ptr(vpool), _ptr(out), _ptr(block_table), _c_int(block_table.shape[1]),
                             _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_pos0), _ptr(work), _c_int(work.shape[0]),
                             _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), _c_int(pages), _c_int(window or 0),
-                            _c_float(scale), _c_int(max_key_groups), _stream()))
+                            _c_float(scale), _c_int(max_key_groups), _c_int(T), _c_int(nsplit), _ptr(part_o), _ptr(part_ml),
+                            _stream()))
         return out
+
+    @staticmethod
+    def _portion_splits(blocks: int, span: int, window: Optional[int]) -> int:
+        """Blocks sharing the keys of one block of rows.  Few blocks of rows (a short portion of a
+        prompt, or single rows) over long contexts leave most of the chip idle and take as long
+        as their chain of tiles; cutting the chain fills the chip.  One split has at least 512
+        keys; the cut depends on the batch, so results differ in rounding between batches."""
+        if blocks >= 192:
+            return 1
+        if window:
+            span = min(span, window + 64)
+        return max(1, min(-(-384 // blocks), span // 512, 64))
 
     DECODE_MAX_GROUP = 16  # query heads per key/value head the decode kernel takes
 

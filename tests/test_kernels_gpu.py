@@ -206,7 +206,7 @@ def test_rope_kv_write(dtype, H, KV, hd, ps, theta):
     assert_close(vd, vp2, dtype, "value pages from partial sums")
 
 
-def _attention_case(dtype, H, KV, hd, ps, window, seqs, seed, peak=False, groups=0):
+def _attention_case(dtype, H, KV, hd, ps, window, seqs, seed, peak=False, groups=0, splits=0):
     """seqs: list of (cached length, rows in this step).  Builds scattered pages holding random
     keys and values for positions < cached + rows and queries for the step's rows."""
     ops, emu = ops_for(dtype), EmulatedOps(dtype)
@@ -239,11 +239,11 @@ def _attention_case(dtype, H, KV, hd, ps, window, seqs, seed, peak=False, groups
         q[row, head * hd:(head + 1) * hd] = (qv / qv.norm() * 8.0 * math.sqrt(hd) / 4).to(dtype)
     i32 = lambda x: torch.tensor(x, dtype=torch.int32)
     args = (i32(q_start), i32(q_len), i32(pos0), i32(work).view(-1, 2))
-    if groups:
+    if groups or splits:
         emu = EmulatedOps(torch.float32)  # the reference unrounded: the tolerance allows the output's one rounding
     ref = emu.paged_attention(q, kp, vp, table, *args, H, KV, hd, ps, window, hd ** -0.5)
     got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV), table.to(DEV), *[a.to(DEV) for a in args], H, KV, hd,
-                              ps, window, hd ** -0.5, groups)
+                              ps, window, hd ** -0.5, groups, splits)
     return got, ref
 
 
@@ -266,6 +266,18 @@ def test_attention_key_groups(dtype, groups, H, KV, hd, ps, window):
     seqs = [(0, 1), (0, 300), (517, 1), (700, 37), (3, 2), (1023, 1), (64 * groups, 1), (64 * groups - 1, 2)]
     got, ref = _attention_case(dtype, H, KV, hd, ps, window, seqs, 300 + hd + groups, peak=True, groups=groups)
     assert_close(got, ref, dtype, f"attention with {groups} key groups")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("splits", [2, 5, 64])
+@pytest.mark.parametrize("H,KV,hd,ps,window", [(4, 2, 16, 16, None), (14, 2, 64, 64, None), (6, 3, 128, 32, None),
+                                               (6, 2, 64, 16, 100), (3, 1, 48, 32, 333)])
+def test_attention_key_splits(dtype, splits, H, KV, hd, ps, window):
+    """The keys of a block of rows cut over several blocks and merged: short and long requests in
+    one launch (most splits of the short ones are empty), and a far key that must not be missed."""
+    seqs = [(0, 1), (0, 300), (517, 1), (1500, 37), (3, 2), (1023, 1), (128, 1), (127, 2)]
+    got, ref = _attention_case(dtype, H, KV, hd, ps, window, seqs, 400 + hd + splits, peak=True, splits=splits)
+    assert_close(got, ref, dtype, f"attention with the keys cut over {splits} blocks")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -171,3 +171,68 @@ def test_mixed_with_page_reuse(models, which, dtype):
     assert total_pages > pages, "the trace must need more pages than the pool has"
     for r in range(len(seqs)):
         check(torch.cat(got[r]), refs[r], dtype, f"{which} request {r} mixed")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("which", ["B", "C"])
+def test_a_step_shape_that_recurs_is_replayed_from_its_graph(models, which, dtype):
+    """A long prompt fed in equal portions beside two requests that decode: once the step's shape
+    has come a few times it runs from a captured graph.  Every replay is compared with
+    the plain model, with other steps (another shape, run as it is) in between; and so is the
+    same trace with capturing switched off (it differs in rounding only: the captured tables
+    are wider, which changes how the keys are cut among waves)."""
+    from machserve_amd.engine import StepEntry
+    d, w, sizes, prompts, _ = models[which]
+    long_i = max(range(len(prompts)), key=lambda i: len(prompts[i]))
+    others = [i for i in range(len(prompts)) if i != long_i and len(prompts[i]) >= 9][:2]
+    assert len(others) == 2
+
+    def run(use_graphs):
+        lm = engine(models, which, dtype, 24)
+        if not use_graphs:
+            lm.step.use_graphs = False
+        replays = [0]
+        inner = lm.step._run_graph
+
+        def counted(key, *a, **kw):
+            replays[0] += key in lm.step._graphs
+            return inner(key, *a, **kw)
+        lm.step._run_graph = counted
+        slots = {i: lm.cache.admit() for i in [long_i] + others}
+        fed = {i: 0 for i in slots}
+        got = {i: [] for i in slots}
+        # the two short ones: all but their last eight tokens at once
+        for i in others:
+            n = len(prompts[i]) - 8
+            got[i].append(lm.step([StepEntry(slots[i], prompts[i][:n], list(range(n)))]))
+            fed[i] = n
+        portion, step = 7, 0
+        while fed[long_i] < len(prompts[long_i]):
+            entries, order = [], []
+            for i in others:
+                if fed[i] < len(prompts[i]):
+                    entries.append(StepEntry(slots[i], prompts[i][fed[i]:fed[i] + 1], [0]))
+                    order.append((i, 1))
+            n = min(portion, len(prompts[long_i]) - fed[long_i])
+            entries.append(StepEntry(slots[long_i], prompts[long_i][fed[long_i]:fed[long_i] + n], list(range(n))))
+            order.append((long_i, n))
+            logits = lm.step(entries)
+            k = 0
+            for i, m in order:
+                got[i].append(logits[k:k + m])
+                k += m
+                fed[i] += m
+            step += 1
+        for i in others:  # what is left of the short ones, one by one
+            while fed[i] < len(prompts[i]):
+                got[i].append(lm.step([StepEntry(slots[i], prompts[i][fed[i]:fed[i] + 1], [0])]))
+                fed[i] += 1
+        lm.cache.check()
+        return {i: torch.cat(got[i]) for i in slots}, replays[0]
+
+    captured, n_replays = run(True)
+    plain_run, none = run(False)
+    assert n_replays >= 2 and none == 0, "the recurring shape must have been replayed"
+    for i in captured:
+        check(captured[i], plain_logits(models, which, dtype, i), dtype, f"{which} request {i} with captured steps")
+        check(plain_run[i], plain_logits(models, which, dtype, i), dtype, f"{which} request {i} without captured steps")
