@@ -256,7 +256,8 @@ static int plan_tiled_splits(int M, int N, int K) {
     const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
     if (b128 >= 300 && g_force_splits == 0) return 1;
     // about 1.75 blocks a CU; more than six slices cost more in the consumer's sums than they gain here
-    int want = max(1, min(min((int)ceil_div(448, b128), K / 512), 6));
+    // (with very few tiles - a portion of a few hundred rows - slices of 256 still pay)
+    int want = max(1, min(min((int)ceil_div(448, b128), K / (b128 <= 32 ? 256 : 512)), 6));
     if (g_force_splits > 0) want = g_force_splits;
     // what the launcher's rounding of a slice to a multiple of 64 really yields
     const int k_per_split = ceil_div(ceil_div(K, want), 64) * 64;

@@ -61,7 +61,7 @@ class LaunchedDecode:
 class StepFunction:
     TABLE_BUCKET = 8        # captured block tables are this many pages wide, or a multiple
     MAX_GRAPHS = 48         # captured steps kept; the one unused longest goes first
-    CAPTURE_MAX_ROWS = 128  # a step of more rows keeps the device busy longer than the host needs to launch it
+    CAPTURE_MAX_ROWS = 320  # a larger step keeps the device busy longer than the host needs to launch it (and replays slower)
     CAPTURE_AFTER = 3       # a shape other than plain decoding is captured when it has come this often before
 
     def __init__(self, model, cache: CacheManager, rt, attention_rows_per_block: int = 64, use_graphs: bool = True):
