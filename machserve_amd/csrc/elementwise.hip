@@ -168,6 +168,76 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(RopeArgs a) {
     }
 }
 
+// The same in quads: head sizes that are multiples of 8, rows whose stride is a multiple of 4 and
+// 16-byte aligned buffers.  A thread takes four neighbouring pairs (j .. j + 3, j + half .. + 3) of one
+// head: two 16-byte loads per partial sum, all asked for before the first is used, and two 8-byte
+// (bfloat16) or 16-byte stores.  Nothing is staged in LDS but the row's cosines and sines.
+template <int NP>
+__global__ __launch_bounds__(256) void rope_kv_write_quads_kernel(RopeArgs a) {
+    __shared__ float cs[128], sn[128];
+    const int t = blockIdx.x, half = a.hd / 2, hq = half / 4;
+    if (threadIdx.x < half) {
+        float c = 1.f, s = 0.f;
+        if (a.inv_freq) {
+            const float ang = (float)a.positions[t] * a.inv_freq[threadIdx.x];
+            sincosf(ang, &s, &c);
+        }
+        cs[threadIdx.x] = c;
+        sn[threadIdx.x] = s;
+    }
+    const bool writes = a.slot_map != nullptr;
+    const int slot = writes ? a.slot_map[t] : -1;
+    const int page = slot >= 0 ? slot / a.ps : 0, off = slot >= 0 ? slot % a.ps : 0;
+    const float* rowp = a.qkv + (size_t)t * a.stride;
+    auto summed = [&](int c) {  // bias + the partial sums of columns c .. c + 3, in order
+        f32x4 v[NP];
+#pragma unroll
+        for (int p = 0; p < NP; ++p) v[p] = *reinterpret_cast<const f32x4*>(rowp + p * a.partial_stride + c);
+        f32x4 r = a.bias ? *reinterpret_cast<const f32x4*>(a.bias + c) : (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int p = 0; p < NP; ++p) r += v[p];
+        return r;
+    };
+    auto store_quad = [](elem_t* o, const f32x4& v) {
+#ifdef MS_ELEM_BF16
+        bf16x4_t b = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+        *reinterpret_cast<bf16x4_t*>(o) = b;
+#else
+        *reinterpret_cast<f32x4*>(o) = v;
+#endif
+    };
+    // q heads, then k heads: pairs (j, j + half)
+    const int rot_heads = a.H + (writes ? a.KV : 0);
+    const int n_rot = rot_heads * hq;
+    // v heads: quads of the head's elements
+    const int n_v = writes ? a.KV * (a.hd / 4) : 0;
+    __syncthreads();
+    for (int it = threadIdx.x; it < n_rot + n_v; it += 256) {
+        if (it < n_rot) {
+            const int h = it / hq, j = (it % hq) * 4;
+            const f32x4 x0 = summed(h * a.hd + j), x1 = summed(h * a.hd + half + j);
+            f32x4 lo, hi;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                lo[e] = x0[e] * cs[j + e] - x1[e] * sn[j + e];
+                hi[e] = x0[e] * sn[j + e] + x1[e] * cs[j + e];
+            }
+            elem_t* o;
+            if (h < a.H) o = a.q_out + ((size_t)t * a.H + h) * a.hd;
+            else if (slot >= 0) o = a.kpool + (((size_t)page * a.KV + (h - a.H)) * a.ps + off) * a.hd;
+            else continue;
+            store_quad(o + j, lo);
+            store_quad(o + half + j, hi);
+        } else if (slot >= 0) {
+            const int q = it - n_rot, h = q / (a.hd / 4), dd = (q % (a.hd / 4)) * 4;
+            const f32x4 v = summed((a.H + a.KV + h) * a.hd + dd);
+            elem_t* o = a.vpool + (((size_t)page * a.KV + h) * a.hd + dd) * a.ps + off;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[(size_t)e * a.ps] = from_f32<elem_t>(v[e]);
+        }
+    }
+}
+
 }  // namespace ms
 
 using namespace ms;
@@ -250,6 +320,17 @@ extern "C" int ms_rope_kv_write(const float* qkv, int n_partials, const float* b
     MS_REQUIRE(stride * sizeof(float) <= 60000, "rope: a row of %d values exceeds the row buffer", stride);
     RopeArgs a{qkv, bias, n_partials, (size_t)T * stride, positions, inv_freq, slot_map, (elem_t*)q_out, (elem_t*)kpool,
                (elem_t*)vpool, stride, H, KV, hd, ps};
+    const bool aligned = ((reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(bias) | reinterpret_cast<uintptr_t>(q_out) |
+                           reinterpret_cast<uintptr_t>(kpool)) & 15) == 0;
+    if (hd % 8 == 0 && stride % 4 == 0 && a.partial_stride % 4 == 0 && aligned && n_partials <= 4) {
+        switch (n_partials) {
+            case 1: hipLaunchKernelGGL(rope_kv_write_quads_kernel<1>, dim3(T), dim3(256), 0, stream, a); break;
+            case 2: hipLaunchKernelGGL(rope_kv_write_quads_kernel<2>, dim3(T), dim3(256), 0, stream, a); break;
+            case 3: hipLaunchKernelGGL(rope_kv_write_quads_kernel<3>, dim3(T), dim3(256), 0, stream, a); break;
+            default: hipLaunchKernelGGL(rope_kv_write_quads_kernel<4>, dim3(T), dim3(256), 0, stream, a); break;
+        }
+        return check_launch("rope_kv_write");
+    }
     hipLaunchKernelGGL(rope_kv_write_kernel, dim3(T), dim3(256), (size_t)stride * sizeof(float), stream, a);
     return check_launch("rope_kv_write");
 }
