@@ -49,11 +49,13 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, con
 // four consecutive columns (group t, t + 256, ...) and asks for all of the row it needs - stream,
 // weights and the NP pending sums - before it uses the first value, so the kernel pays one memory
 // round trip instead of one per column and pending sum.  The sums are added in the same order.
-template <typename OutT, int G, int NP>
+// With more than eight pending sums (MORE, NP = 8) the rest, up to eight again, follows in a second
+// round of loads.
+template <typename OutT, int G, int NP, bool MORE = false>
 __global__ __launch_bounds__(256) void rmsnorm_wide_kernel(float* __restrict__ x, const float* __restrict__ partials,
                                                            size_t partial_stride, const int* __restrict__ rows,
                                                            const float* __restrict__ w, OutT* __restrict__ out, int d,
-                                                           float eps) {
+                                                           float eps, int n_more) {
     __shared__ float scratch[4];
     const int i = blockIdx.x, ng = d / 4;
     const size_t r = rows ? rows[i] : i;
@@ -72,13 +74,35 @@ __global__ __launch_bounds__(256) void rmsnorm_wide_kernel(float* __restrict__ x
     for (int p = 0; p < NP; ++p)
 #pragma unroll
         for (int g = 0; g < G; ++g) pend[p][g] = reinterpret_cast<const f32x4*>(partials + p * partial_stride + r * d)[at[g]];
+    if constexpr (MORE) {
+        static_assert(NP == 8, "a second round follows a full first one");
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int p = 0; p < NP; ++p) v[g] += pend[p][g];
+        // sums beyond the last one read the last one again and count for nothing
+#pragma unroll
+        for (int p = 0; p < NP; ++p)
+#pragma unroll
+            for (int g = 0; g < G; ++g)
+                pend[p][g] = reinterpret_cast<const f32x4*>(partials + (size_t)(NP + min(p, n_more - 1)) * partial_stride + r * d)[at[g]];
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int p = 0; p < NP; ++p) {
+                const float keep = p < n_more ? 1.f : 0.f;
+                v[g] += pend[p][g] * keep;
+            }
+    }
     float ss = 0.f;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
+        if constexpr (!MORE) {
 #pragma unroll
-        for (int p = 0; p < NP; ++p) v[g] += pend[p][g];
+            for (int p = 0; p < NP; ++p) v[g] += pend[p][g];
+        }
         if (threadIdx.x + g * 256 < ng) {
-            if (NP > 0 && !rows) src[at[g]] = v[g];
+            if ((NP > 0 || MORE) && !rows) src[at[g]] = v[g];
             ss += v[g].x * v[g].x + v[g].y * v[g].y + v[g].z * v[g].z + v[g].w * v[g].w;
         }
     }
@@ -260,10 +284,13 @@ extern "C" int ms_rmsnorm(float* x, const float* partials, int n_partials, int T
     const bool f32_out = out_f32 || !kBf16;
     const int groups = d % 4 == 0 ? (d <= 1024 ? 1 : (d <= 2048 ? 2 : (d <= 4096 ? 4 : 0))) : 0;
     const bool aligned = (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(partials)) % 16 == 0;
-    if (groups && aligned && n_partials <= 8) {
+    if (groups && aligned && n_partials <= 16) {
 #define MS_NORM(OUT_, G_, NP_)                                                                                   \
     hipLaunchKernelGGL((rmsnorm_wide_kernel<OUT_, G_, NP_>), dim3(n), dim3(256), 0, stream, x, partials, ps, rows, w, \
-                       (OUT_*)out, d, eps)
+                       (OUT_*)out, d, eps, 0)
+#define MS_NORM_MORE(OUT_, G_)                                                                                          \
+    hipLaunchKernelGGL((rmsnorm_wide_kernel<OUT_, G_, 8, true>), dim3(n), dim3(256), 0, stream, x, partials, ps, rows, w, \
+                       (OUT_*)out, d, eps, n_partials - 8)
 #define MS_NORM_NP(OUT_, G_)                                    \
     switch (n_partials) {                                       \
         case 0: MS_NORM(OUT_, G_, 0); break;                    \
@@ -274,7 +301,8 @@ extern "C" int ms_rmsnorm(float* x, const float* partials, int n_partials, int T
         case 5: MS_NORM(OUT_, G_, 5); break;                    \
         case 6: MS_NORM(OUT_, G_, 6); break;                    \
         case 7: MS_NORM(OUT_, G_, 7); break;                    \
-        default: MS_NORM(OUT_, G_, 8); break;                   \
+        case 8: MS_NORM(OUT_, G_, 8); break;                    \
+        default: MS_NORM_MORE(OUT_, G_); break;                 \
     }
 #define MS_NORM_G(OUT_)                                         \
     if (groups == 1) { MS_NORM_NP(OUT_, 1) }                    \
@@ -283,6 +311,7 @@ extern "C" int ms_rmsnorm(float* x, const float* partials, int n_partials, int T
         if (f32_out) { MS_NORM_G(float) } else { MS_NORM_G(elem_t) }
 #undef MS_NORM_G
 #undef MS_NORM_NP
+#undef MS_NORM_MORE
 #undef MS_NORM
         return check_launch("rmsnorm");
     }

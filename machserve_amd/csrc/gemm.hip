@@ -256,8 +256,11 @@ static int plan_tiled_splits(int M, int N, int K) {
     const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
     if (b128 >= 300 && g_force_splits == 0) return 1;
     // about 1.75 blocks a CU; more than six slices cost more in the consumer's sums than they gain here
-    // (with very few tiles - a portion of a few hundred rows - slices of 256 still pay)
-    int want = max(1, min(min((int)ceil_div(448, b128), K / (b128 <= 32 ? 256 : 512)), 6));
+    // (with very few tiles - a portion of a few hundred rows - slices of 256 still pay).  With few rows
+    // the partial sums are small and the weight is all the traffic: a long K is then cut up to 16 times
+    // (7B down projection at 64 rows: 49 us with 6 slices, 33 with 12 to 16).
+    const int most = M <= 128 ? (K >= 8192 ? 16 : 8) : 6;
+    int want = max(1, min(min((int)ceil_div(448, b128), K / (b128 <= 32 ? 256 : 512)), most));
     if (g_force_splits > 0) want = g_force_splits;
     // what the launcher's rounding of a slice to a multiple of 64 really yields
     const int k_per_split = ceil_div(ceil_div(K, want), 64) * 64;
@@ -306,7 +309,8 @@ extern "C" int ms_tiled_partials(int M, int N, int K) { return plan_tiled_splits
 extern "C" int ms_prefers_tiled(int M, int N, int K) {
     if (M > 64) return 1;
 #ifdef MS_ELEM_BF16
-    if (N < 2048) return 0;
+    // a narrow output with a long K (a down projection): the tiled kernel cuts K over many blocks
+    if (N < 2048) return (M >= 48 && K >= 4096) || (M >= 32 && K >= 8192);
     const double nk = (double)N * (double)K;
     if (M >= 8 && nk >= 100e6) return 1;  // a vocabulary-sized product
     return M >= 16 && nk * M >= 280e6;

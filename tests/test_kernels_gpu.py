@@ -57,6 +57,14 @@ def test_rmsnorm(dtype, T, d, eps):
     assert torch.equal(xd.cpu(), x), "gathered rows leave the stream alone"
     ops.add_partials(xd, parts.to(DEV))
     assert_close(xd, total, torch.float32, "add_partials")
+    # eight, nine, twelve and sixteen pending sums (more than eight come in a second round of loads), each
+    # plane with a value of its own scale so that a plane left out or taken twice shows
+    for n in (8, 9, 12, 16, 17):
+        parts = torch.stack([rnd((T, d), torch.float32, 20 + k, 0.5 + 0.25 * k) for k in range(n)])
+        total = x + parts.sum(0)
+        xd = x.to(DEV).clone()
+        assert_close(ops.rmsnorm(xd, w.to(DEV), eps, partials=parts.to(DEV)), P.rms_norm(total, w, eps), dtype, f"norm of {n} sums")
+        assert_close(xd, total, torch.float32, f"{n} sums written back")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
