@@ -324,10 +324,14 @@ class HipOps:
     DECODE_MAX_GROUP = 16  # query heads per key/value head the decode kernel takes
 
     @staticmethod
-    def _decode_splits(S: int, KV: int, table_width: int, page_size: int, window: Optional[int], key_tile: int) -> int:
+    def _decode_splits(S: int, KV: int, table_width: int, page_size: int, window: Optional[int], key_tile: int,
+                       hd: int = 64) -> int:
+        """Blocks sharing a request's keys: enough for two blocks a CU with small heads, one with heads
+        above 64 (measured at head sizes 64 and 128, 1 to 64 requests), at least four key tiles each."""
         span = table_width * page_size if not window else min(table_width * page_size, window + key_tile)
         tiles = max(1, -(-span // key_tile))
-        return max(1, min(-(-512 // (S * KV)), -(-tiles // 4), 64))
+        blocks = 512 if hd <= 64 else 256
+        return max(1, min(-(-blocks // (S * KV)), -(-tiles // 4), 64))
 
     def decode_attention_fused(self, qkv: torch.Tensor, bias: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor],
                                slot_map: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
@@ -355,7 +359,7 @@ class HipOps:
         self._want(seq_pos0, torch.int32, "seq_pos0", S)
         if H // KV > self.DECODE_MAX_GROUP:
             raise KernelError(f"decode attention: {H // KV} heads per key/value head, at most {self.DECODE_MAX_GROUP}")
-        nsplit = self._decode_splits(S, KV, block_table.shape[1], page_size, window, key_tile)
+        nsplit = self._decode_splits(S, KV, block_table.shape[1], page_size, window, key_tile, hd)
         out = torch.empty((S, H * hd), dtype=self.dtype, device=qkv.device)
         part_o = part_ml = None
         if nsplit > 1:
@@ -385,7 +389,7 @@ class HipOps:
         self._want(seq_pos0, torch.int32, "seq_pos0", S)
         if H // KV > self.DECODE_MAX_GROUP:
             raise KernelError(f"decode attention: {H // KV} heads per key/value head, at most {self.DECODE_MAX_GROUP}")
-        nsplit = self._decode_splits(S, KV, block_table.shape[1], page_size, window, key_tile)
+        nsplit = self._decode_splits(S, KV, block_table.shape[1], page_size, window, key_tile, hd)
         out = torch.empty((S, H * hd), dtype=self.dtype, device=q.device)
         part_o = part_ml = None
         if nsplit > 1:
