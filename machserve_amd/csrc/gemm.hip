@@ -247,20 +247,35 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
 #undef MS_GEMM
 }
 
-// K slices for a product of many rows whose consumer adds partial sums: enough 128x128 blocks to
-// fill the chip, at least 512 of K each.  The 32-bit build never slices: its sums keep one order.
+// K slices for a product whose consumer adds partial sums: enough 128x128 blocks to fill the chip,
+// at least 512 of K each.  The 32-bit build never slices: its sums keep one order.
 static int g_force_splits = 0;  // measurements only
 
 static int plan_tiled_splits(int M, int N, int K) {
 #ifdef MS_ELEM_BF16
     const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
     if (b128 >= 300 && g_force_splits == 0) return 1;
-    // about 1.75 blocks a CU; more than six slices cost more in the consumer's sums than they gain here
-    // (with very few tiles - a portion of a few hundred rows - slices of 256 still pay).  With few rows
-    // the partial sums are small and the weight is all the traffic: a long K is then cut up to 16 times
-    // (7B down projection at 64 rows: 49 us with 6 slices, 33 with 12 to 16).
+    // More than six slices cost more in the consumer's sums than they gain here (with very few tiles - a
+    // portion of a few hundred rows - slices of 256 still pay).  With few rows the partial sums are small
+    // and the weight is all the traffic: a long K is then cut up to 16 times (7B down projection at 64
+    // rows: 49 us with 6 slices, 33 with 12 to 16).
     const int most = M <= 128 ? (K >= 8192 ? 16 : 8) : 6;
-    int want = max(1, min(min((int)ceil_div(448, b128), K / (b128 <= 32 ? 256 : 512)), most));
+    const int limit = max(1, min(K / (b128 <= 32 ? 256 : 512), most));
+    // The chip holds 512 of the 128x128 blocks at a time (two a CU), and a last round that is nearly
+    // empty takes as long as a full one: the fewest slices that fill their rounds to 70 %, else the
+    // count that fills them best (1.5B down projection at 2,048 rows, 192 tiles: 3 slices make a
+    // full round and an eighth, 118 us; 2 slices one round three quarters full, 97 us).
+    int want = 1;
+    double best = 0.0;
+    for (int sl = 1; sl <= limit; ++sl) {
+        const long blocks = b128 * sl, rounds = (blocks + 511) / 512;
+        const double filled = (double)blocks / (double)(rounds * 512);
+        if (filled > best + 1e-9) {
+            best = filled;
+            want = sl;
+        }
+        if (filled >= 0.7) break;
+    }
     if (g_force_splits > 0) want = g_force_splits;
     // what the launcher's rounding of a slice to a multiple of 64 really yields
     const int k_per_split = ceil_div(ceil_div(K, want), 64) * 64;
