@@ -1,8 +1,10 @@
 """The engine: scheduler above, step function and sampler below.
 
 ``add`` queues a request, ``step`` runs one scheduled batch and returns the tokens it
-produced, ``generate`` runs a list of prompts to the end.  Role of ``ContinuousModel`` in
-the reference (``crates/mach-model/src/continuous.rs:715, 943, 1294``)."""
+produced, ``step_pipelined`` does the same but launches a decode step before the tokens of
+the step before it have reached the host (``run`` and ``generate`` use it), ``cancel`` ends a
+request, ``generate`` runs a list of prompts to the end.  Role of ``ContinuousModel`` in the
+reference (``crates/mach-model/src/continuous.rs:715, 943, 1294``)."""
 from __future__ import annotations
 
 import gc
