@@ -18,7 +18,7 @@ from .step import StepEntry
 
 class Engine:
     def __init__(self, loaded: LoadedModel, max_batch_tokens: int = 512, chunk_size: Optional[int] = None,
-                 max_running: Optional[int] = None):
+                 max_running: Optional[int] = None, freeze_gc: bool = True):
         self.loaded = loaded
         self.scheduler = Scheduler(loaded.cache, max_batch_tokens, chunk_size, max_running,
                                    loaded.model.spec.max_positions)
@@ -28,9 +28,11 @@ class Engine:
         self._inflight = None  # (plan, launched step) of step_pipelined
         # Every step makes a few hundred short-lived objects; with the interpreter's whole heap in the
         # collector's oldest generation its full passes cost more than the scheduling itself.  What
-        # exists now (modules, the model) is taken out of the collector's reach.
-        gc.collect()
-        gc.freeze()
+        # exists now (modules, the model) is taken out of the collector's reach (``freeze_gc=False``
+        # leaves the collector as it is).
+        if freeze_gc:
+            gc.collect()
+            gc.freeze()
 
     @classmethod
     def from_dir(cls, model_dir: str, *, dtype="bfloat16", device="cuda:0", page_size: int = 64,
