@@ -96,7 +96,7 @@ def main() -> int:
         return [torch.randint(0, cfg.vocab_size, (length,), generator=gen).tolist() for _ in range(n)]
 
     def make_engine(batch, budget):
-        per_req = -(-(ctx + args.warmup + args.steps + 2 * batch + 72) // page)
+        per_req = -(-(ctx + args.warmup + args.steps + 2 * batch + 96) // page)
         lm = load_model(config=cfg, tensors=tensors, dtype=dt, page_size=page, num_pages=batch * per_req + 4,
                         max_requests=batch)
         return Engine(lm, max_batch_tokens=budget, max_running=batch)
@@ -104,12 +104,16 @@ def main() -> int:
     def decode_run(batch):
         eng = make_engine(batch, 4096)
         for p in prompts(batch, ctx):
-            eng.add(p, args.warmup + args.steps + 2 * batch + 64, SamplingParams())  # early ones decode while later ones prefill
+            eng.add(p, args.warmup + args.steps + 2 * batch + 88, SamplingParams())  # early ones decode while later ones prefill
         while any(not r.decoding for r in eng.scheduler.running) or eng.scheduler.waiting:
             eng.step()
         # the engine's own loop (Engine.run): a step is launched while the tokens of the step before
         # are on their way to the host, so the tokens a call returns are those of the launch before it
         step = eng.step if args.sync_steps else eng.step_pipelined
+        # the engine captures a decode step into a graph once its shape has come a number of times:
+        # that happens before the warm-up, not in the timed steps
+        for _ in range(eng.loaded.step.DECODE_CAPTURE_AFTER + 2):
+            step()
         for _ in range(args.warmup):
             step()
         torch.cuda.synchronize()

@@ -79,22 +79,23 @@ class Engine:
         if self._inflight is None:
             plan = sched.schedule()
             launched = self._launch(plan, None)
-            if launched is None:
-                return self._run_plan(plan)
+            if not launched:
+                # False: the step function has declined (no graph for this shape yet); not asked again
+                return self._run_plan(plan, try_fast=launched is None)
             self._inflight = (plan, launched)
             return [], []
         prev_plan, prev = self._inflight
         plan = sched.schedule()
         launched = self._launch(plan, prev) if self._continues(prev_plan, plan) else None
         emitted, done = sched.complete(prev_plan, *self.loaded.step.collect(prev))
-        if launched is not None:
+        if launched:
             self._inflight = (plan, launched)
             return emitted, done
         self._inflight = None
         # the plan was made before these tokens were known: what has ended meanwhile drops out of it
         plan.items = [it for it in plan.items if it.request.closing is None or it.request.pending > 0]
         plan.native = [n for n in plan.native if n.id in sched.requests]
-        em2, done2 = self._run_plan(plan)
+        em2, done2 = self._run_plan(plan, try_fast=launched is None)
         return emitted + em2, done + done2
 
     def _continues(self, before: StepPlan, plan: StepPlan) -> bool:
@@ -103,7 +104,8 @@ class Engine:
                 and all(a.request is b.request and a.sample and a.count == 1 for a, b in zip(plan.items, before.items)))
 
     def _launch(self, plan: StepPlan, after):
-        """Launch ``plan`` without waiting if it is plain decoding; None (nothing done) if it is not."""
+        """Launch ``plan`` without waiting if it is plain decoding; None (nothing done) if it is not,
+        False if the step function declined."""
         if not plan.items or not all(it.sample and it.count == 1 and it.request.params.plain() for it in plan.items):
             return None
         if after is None and any(it.request.pending for it in plan.items):
@@ -115,7 +117,7 @@ class Engine:
             entries, [r.params.temperature for r in reqs], [r.params.top_k for r in reqs], [r.params.top_p for r in reqs],
             [r.rng_state for r in reqs], after)
         if launched is None:
-            return None
+            return False
         from ..sampling import advance
         for r in reqs:
             r.rng_state = advance(r.rng_state)  # one draw a sampled row, whatever the token
@@ -130,7 +132,7 @@ class Engine:
         self._inflight = None
         return self.scheduler.complete(plan, *self.loaded.step.collect(launched))
 
-    def _run_plan(self, plan: StepPlan):
+    def _run_plan(self, plan: StepPlan, try_fast: bool = True):
         if not plan.items:
             return [], []
         entries, sampled_items = [], []
@@ -142,7 +144,7 @@ class Engine:
         self.steps += 1
         self.tokens_run += plan.n_tokens
         reqs = [it.request for it in sampled_items]
-        if len(sampled_items) == len(plan.items) and all(r.params.plain() for r in reqs):
+        if try_fast and len(sampled_items) == len(plan.items) and all(r.params.plain() for r in reqs):
             # every request decodes one token: forward pass and sampling are one captured graph
             fast = self.loaded.step.decode_and_sample(
                 entries, [r.params.temperature for r in reqs], [r.params.top_k for r in reqs],

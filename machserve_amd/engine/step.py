@@ -60,20 +60,24 @@ class LaunchedDecode:
 
 class StepFunction:
     TABLE_BUCKET = 8        # captured block tables are this many pages wide, or a multiple
-    MAX_GRAPHS = 48         # captured steps kept; the one unused longest goes first
+    MAX_GRAPHS = 256        # captured steps kept; the one unused longest goes first
     CAPTURE_MAX_ROWS = 320  # a larger step keeps the device busy longer than the host needs to launch it (and replays slower)
-    CAPTURE_AFTER = 3       # a shape other than plain decoding is captured when it has come this often before
+    # A capture costs as much as the launches of twenty to seventy steps save (7 ms against 0.1 to 0.3 ms
+    # a step), and while requests end one by one most shapes last a few steps: a shape is captured when it
+    # has come this often before, which at worst doubles what the better choice would have cost.
+    CAPTURE_AFTER = 16         # a step other than plain decoding
+    DECODE_CAPTURE_AFTER = 16  # a decode step
 
     def __init__(self, model, cache: CacheManager, rt, attention_rows_per_block: int = 64, use_graphs: bool = True):
         self.model, self.cache, self.rt = model, cache, rt
         self.rows_per_block = attention_rows_per_block
         self.heads_per_kv = model.attention_rows_per_token()
         # A step of few tokens is bound by its launches: it is captured into a HIP graph and replayed.
-        # A decode step (one token a request) at its first occurrence; any other step of few rows
-        # when its shape (tokens per request, wanted rows, table widths) keeps coming, as it does
-        # while a long prompt is fed in small portions beside the same decoding requests (a
-        # capture costs as much as a few dozen launched steps, so a shape must earn it).  Only for
-        # models whose parts read nothing but device memory from the context.
+        # A decode step (one token a request), and any other step of few rows, when its shape
+        # (tokens per request, wanted rows, table widths) keeps coming, as it does while the same
+        # requests decode, or while a long prompt is fed in small portions beside them (a capture
+        # costs as much as a few dozen launched steps, so a shape must earn it).  Only for models
+        # whose parts read nothing but device memory from the context.
         self.use_graphs = (use_graphs and rt.device.type == "cuda"
                            and all(getattr(b.mixer, "graph_safe", False) for b in getattr(model, "blocks", [])))
         self._graphs: "OrderedDict[tuple, _DecodeGraph]" = OrderedDict()
@@ -138,17 +142,27 @@ class StepFunction:
         return self._context_from(dev, offsets, widths, lists)
 
     # ------------------------------------------------------------------ captured decode steps
-    def _run_decode_graph(self, entries: Sequence[StepEntry], sampling=None, after: Optional["LaunchedDecode"] = None):
-        """Replay (or first capture) the graph of a decode step; every row's logits are computed.
-        ``sampling`` = (temperatures, top_ks, top_ps, states) makes sampling part of the graph;
-        the result is then the int32 ``[2, B]`` tensor of :meth:`HipOps.sample_packed`, else the
-        logits.  With ``after`` (the launched step before this one, of the same requests) the
-        step's tokens are that step's samples, on the device, and the entries' own tokens are
-        placeholders.  Returns the result and the graph."""
+    def _decode_shape(self, entries: Sequence[StepEntry], sampled: bool):
+        """The buffer of a decode step (every row's logits are computed) and its graph's key."""
         slots, counts, tokens, _ = self._check_entries(entries)
-        built = self.cache.build_step(slots, counts, tokens, list(range(len(slots))), self.heads_per_kv,
-                                      self.rows_per_block, self.TABLE_BUCKET)
-        return self._run_graph(self._graph_key(counts, len(slots), built[2], sampling is not None), built, sampling, after)
+        try:
+            built = self.cache.build_step(slots, counts, tokens, list(range(len(slots))), self.heads_per_kv,
+                                          self.rows_per_block, self.TABLE_BUCKET)
+        except CacheError as e:
+            raise StepError(str(e)) from e
+        return built, self._graph_key(counts, len(slots), built[2], sampled)
+
+    def _ready(self, key: tuple, after: int) -> bool:
+        """Whether the step of this shape runs from a graph: it has one, or has come ``after`` times."""
+        if key in self._graphs:
+            return True
+        n = self._seen.get(key, 0)
+        if n >= after:
+            return True
+        if len(self._seen) > 4096:
+            self._seen.clear()
+        self._seen[key] = n + 1
+        return False
 
     @staticmethod
     def _graph_key(counts, n_want: int, widths, sampled: bool) -> tuple:
@@ -230,7 +244,8 @@ class StepFunction:
         """The same step, launched and not waited for.  With ``after`` - the launched step before
         this one, of the same requests in the same order - the tokens are that step's samples,
         taken on the device: the host need not have seen them.  None if the step cannot take this
-        path; ``OutOfPages`` before anything ran if the pages are not there."""
+        path or its shape has not come often enough to be captured; ``OutOfPages`` before anything
+        ran if the pages are not there."""
         if not (self.use_graphs and all(len(e.tokens) == 1 for e in entries)
                 and len({e.slot for e in entries}) == len(entries)):
             return None
@@ -247,7 +262,10 @@ class StepFunction:
                 raise OutOfPages(f"group {k}: the step needs {v} new pages, {cache.free_pages(k)} are free")
         for e in entries:
             cache.extend(e.slot, 1)
-        sampled, graph = self._run_decode_graph(entries, (temperatures, top_ks, top_ps, states), after)
+        built, key = self._decode_shape(entries, True)
+        if not self._ready(key, self.DECODE_CAPTURE_AFTER):
+            return None  # the pages stay with the requests; the caller runs the step as it is
+        sampled, graph = self._run_graph(key, built, (temperatures, top_ks, top_ps, states), after)
         for e in entries:
             cache.commit(e.slot, 1)
         # the samples go to a pinned buffer of their own (the graph's is overwritten by its next replay)
@@ -285,7 +303,13 @@ class StepFunction:
         for e in entries:
             cache.extend(e.slot, len(e.tokens))
         if self.use_graphs and all(len(e.tokens) == 1 for e in entries) and len({e.slot for e in entries}) == len(entries):
-            logits, _ = self._run_decode_graph(entries)
+            built, key = self._decode_shape(entries, False)
+            if self._ready(key, self.DECODE_CAPTURE_AFTER):
+                logits, _ = self._run_graph(key, built)
+            else:
+                host, offsets, widths = built
+                logits = self.model.forward(self._context_from(torch.from_numpy(host).to(self.rt.device), offsets, widths))
+                borrow_logits = True  # a fresh tensor: nothing overwrites it
             wanted = [i for i, e in enumerate(entries) if len(e.want)]
             if not wanted:
                 logits = None
@@ -306,14 +330,11 @@ class StepFunction:
             except CacheError as e:
                 raise StepError(str(e)) from e
             key = self._graph_key(counts, len(want), built[2], False)
-            if len(tokens) <= self.CAPTURE_MAX_ROWS and (key in self._graphs or self._seen.get(key, 0) >= self.CAPTURE_AFTER):
+            if len(tokens) <= self.CAPTURE_MAX_ROWS and self._ready(key, self.CAPTURE_AFTER):
                 logits, _ = self._run_graph(key, built)
                 if logits is not None and not borrow_logits:
                     logits = logits.clone()
-            else:  # a shape seen for the first time runs as it is: most shapes never come again
-                if len(self._seen) > 4096:
-                    self._seen.clear()
-                self._seen[key] = self._seen.get(key, 0) + 1
+            else:  # most shapes never come again: they run as they are
                 host, offsets, widths = built
                 logits = self.model.forward(self._context_from(torch.from_numpy(host).to(self.rt.device), offsets, widths))
         else:

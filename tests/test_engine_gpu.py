@@ -74,6 +74,7 @@ def test_steps_launched_ahead_give_what_steps_one_at_a_time_give(dirs, dtype):
 
     def run(pipelined, eos=None):
         eng = Engine.from_dir(dirs["B"], dtype=dtype, page_size=32, num_pages=16, capacity=4, max_batch_tokens=48)
+        eng.loaded.step.DECODE_CAPTURE_AFTER = 0  # every decode step from a captured graph: nothing is launched ahead without one
         fed_from_device = [0]
         launch = eng.loaded.step.launch_decode
 
