@@ -62,11 +62,12 @@ class StepFunction:
     TABLE_BUCKET = 8        # captured block tables are this many pages wide, or a multiple
     MAX_GRAPHS = 256        # captured steps kept; the one unused longest goes first
     CAPTURE_MAX_ROWS = 320  # a larger step keeps the device busy longer than the host needs to launch it (and replays slower)
-    # A capture costs as much as the launches of twenty to seventy steps save (7 ms against 0.1 to 0.3 ms
-    # a step), and while requests end one by one most shapes last a few steps: a shape is captured when it
-    # has come this often before, which at worst doubles what the better choice would have cost.
-    CAPTURE_AFTER = 16         # a step other than plain decoding
-    DECODE_CAPTURE_AFTER = 16  # a decode step
+    # A capture costs 7 ms; a replayed step is 0.9 ms shorter than a launched one with a few requests, 0.3 to
+    # 0.4 ms with 64 requests or a few hundred rows.  While requests end one by one most shapes last a few
+    # steps, so a shape is captured only when it has come this often before: at worst that doubles what the
+    # better choice would have cost.
+    CAPTURE_AFTER = 16        # a step other than plain decoding
+    DECODE_CAPTURE_AFTER = 8  # a decode step
 
     def __init__(self, model, cache: CacheManager, rt, attention_rows_per_block: int = 64, use_graphs: bool = True):
         self.model, self.cache, self.rt = model, cache, rt
