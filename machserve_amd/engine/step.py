@@ -143,15 +143,31 @@ class StepFunction:
         return self._context_from(dev, offsets, widths, lists)
 
     # ------------------------------------------------------------------ captured decode steps
+    @staticmethod
+    def _decode_bucket(n: int) -> int:
+        """Rows of the captured decode step that takes ``n`` requests: 1, 2, 4, 8, then multiples of 8."""
+        if n <= 8:
+            b = 1
+            while b < n:
+                b *= 2
+            return b
+        return -(-n // 8) * 8
+
     def _decode_shape(self, entries: Sequence[StepEntry], sampled: bool):
-        """The buffer of a decode step (every row's logits are computed) and its graph's key."""
+        """The buffer of a decode step (every row's logits are computed), its graph's key, and the
+        number of rows added.  The step is filled up to a bucket's size with copies of its first row,
+        so that a few graphs serve every batch size while requests end one by one: a copy writes the
+        same key and value to the same place and its logits are dropped; a decode step's time hardly
+        depends on a few rows more."""
         slots, counts, tokens, _ = self._check_entries(entries)
+        pad = self._decode_bucket(len(slots)) - len(slots)
+        slots, counts, tokens = slots + [slots[0]] * pad, counts + [1] * pad, tokens + [tokens[0]] * pad
         try:
             built = self.cache.build_step(slots, counts, tokens, list(range(len(slots))), self.heads_per_kv,
                                           self.rows_per_block, self.TABLE_BUCKET)
         except CacheError as e:
             raise StepError(str(e)) from e
-        return built, self._graph_key(counts, len(slots), built[2], sampled)
+        return built, self._graph_key(counts, len(slots), built[2], sampled), pad
 
     def _ready(self, key: tuple, after: int) -> bool:
         """Whether the step of this shape runs from a graph: it has one, or has come ``after`` times."""
@@ -263,16 +279,19 @@ class StepFunction:
                 raise OutOfPages(f"group {k}: the step needs {v} new pages, {cache.free_pages(k)} are free")
         for e in entries:
             cache.extend(e.slot, 1)
-        built, key = self._decode_shape(entries, True)
+        built, key, pad = self._decode_shape(entries, True)
         if not self._ready(key, self.DECODE_CAPTURE_AFTER):
             return None  # the pages stay with the requests; the caller runs the step as it is
-        sampled, graph = self._run_graph(key, built, (temperatures, top_ks, top_ps, states), after)
+        # the added rows sample as the first row does (same logits, same state): the same token
+        filled = [list(v) + [v[0]] * pad for v in (temperatures, top_ks, top_ps, states)]
+        sampled, graph = self._run_graph(key, built, tuple(filled), after)
         for e in entries:
             cache.commit(e.slot, 1)
         # the samples go to a pinned buffer of their own (the graph's is overwritten by its next replay)
-        ring = self._results.get(len(slots))
+        rows = len(slots) + pad
+        ring = self._results.get(rows)
         if ring is None:
-            ring = self._results[len(slots)] = [torch.empty((2, len(slots)), dtype=torch.int32, pin_memory=True) for _ in range(3)]
+            ring = self._results[rows] = [torch.empty((2, rows), dtype=torch.int32, pin_memory=True) for _ in range(3)]
         result = ring[self._launches % 3]  # at most two steps are in flight: a buffer is read before its next turn
         self._launches += 1
         result.copy_(sampled, non_blocking=True)
@@ -283,7 +302,8 @@ class StepFunction:
     def collect(self, launched: "LaunchedDecode"):
         """``(tokens, logprobs)`` of a launched step as host lists; waits for them."""
         launched.done.synchronize()
-        return launched.result[0].tolist(), launched.result[1].view(torch.float32).tolist()
+        n = len(launched.slots)  # rows beyond are copies of the first
+        return launched.result[0, :n].tolist(), launched.result[1, :n].view(torch.float32).tolist()
 
     # ------------------------------------------------------------------ the step
     def __call__(self, entries: Sequence[StepEntry], borrow_logits: bool = False) -> Optional[torch.Tensor]:
@@ -304,13 +324,15 @@ class StepFunction:
         for e in entries:
             cache.extend(e.slot, len(e.tokens))
         if self.use_graphs and all(len(e.tokens) == 1 for e in entries) and len({e.slot for e in entries}) == len(entries):
-            built, key = self._decode_shape(entries, False)
+            built, key, pad = self._decode_shape(entries, False)
             if self._ready(key, self.DECODE_CAPTURE_AFTER):
                 logits, _ = self._run_graph(key, built)
             else:
                 host, offsets, widths = built
                 logits = self.model.forward(self._context_from(torch.from_numpy(host).to(self.rt.device), offsets, widths))
                 borrow_logits = True  # a fresh tensor: nothing overwrites it
+            if pad:
+                logits = logits[:len(entries)]
             wanted = [i for i, e in enumerate(entries) if len(e.want)]
             if not wanted:
                 logits = None
