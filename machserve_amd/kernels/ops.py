@@ -47,9 +47,12 @@ class HipOps:
             raise KernelError("no GPU is visible: the HIP kernels have no CPU fallback")
         self.dtype = dtype
         self.device = torch.device(device)
+        self._index = self.device.index if self.device.index is not None else torch.cuda.current_device()
         self.elem = "bf16" if dtype == torch.bfloat16 else "f32"
         self._core = self._load(build.ensure_library("core", self.elem))
         self._attn = {}
+        # what the library plans for a product depends on its sizes alone: asked once per size
+        self._plans: dict = {}
 
     def _load(self, path: str):
         try:
@@ -58,6 +61,12 @@ class HipOps:
             raise KernelError(f"cannot load {path}: {e}") from None
         lib.ms_last_error.restype = ctypes.c_char_p
         return lib
+
+    def _stream(self):
+        """torch's current stream on this object's device as a raw handle."""
+        if _raw_stream is not None:
+            return _c_void(_raw_stream(self._index))
+        return _c_void(torch.cuda.current_stream(self.device).cuda_stream)
 
     def _check(self, lib, rc: int):
         if rc != 0:
@@ -76,7 +85,7 @@ class HipOps:
         self._want(tokens, torch.int32, "embed tokens", T)
         self._want(table, self.dtype, "embed table")
         x = torch.empty((T, d), dtype=torch.float32, device=table.device)
-        self._check(self._core, self._core.ms_embed(_ptr(tokens), _ptr(table), _ptr(x), _c_int(T), _c_int(d), _stream()))
+        self._check(self._core, self._core.ms_embed(_ptr(tokens), _ptr(table), _ptr(x), _c_int(T), _c_int(d), self._stream()))
         return x
 
     def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, rows: Optional[torch.Tensor] = None,
@@ -96,7 +105,7 @@ class HipOps:
         out = torch.empty((n, d), dtype=torch.float32 if out_f32 else self.dtype, device=x.device)
         self._check(self._core, self._core.ms_rmsnorm(_ptr(x), _ptr(partials), _c_int(P), _c_int(T), _ptr(rows),
                                                       _ptr(weight), _ptr(out), _c_int(int(out_f32)), _c_int(n), _c_int(d),
-                                                      _c_float(eps), _stream()))
+                                                      _c_float(eps), self._stream()))
         return out
 
     def add_partials(self, x: torch.Tensor, partials: torch.Tensor) -> None:
@@ -105,7 +114,7 @@ class HipOps:
         self._want(x, torch.float32, "stream")
         self._want(partials, torch.float32, "partial sums", partials.shape[0], T, d)
         self._check(self._core, self._core.ms_add_partials(_ptr(x), _ptr(partials), _c_int(partials.shape[0]), _c_int(T),
-                                                           _c_int(d), _stream()))
+                                                           _c_int(d), self._stream()))
 
     def rope_kv_write(self, qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
                       inv_freq: Optional[torch.Tensor], slot_map: Optional[torch.Tensor], kpool: Optional[torch.Tensor],
@@ -130,7 +139,7 @@ class HipOps:
         q = torch.empty((T, H * hd), dtype=self.dtype, device=qkv.device)
         self._check(self._core, self._core.ms_rope_kv_write(
             _ptr(qkv), _c_int(P), _ptr(bias), _c_int(stride), _ptr(positions), _ptr(inv_freq), _ptr(slot_map), _ptr(q),
-            _ptr(kpool), _ptr(vpool), _c_int(T), _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), _stream()))
+            _ptr(kpool), _ptr(vpool), _c_int(T), _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), self._stream()))
         return q
 
     # ------------------------------------------------------------------ matrix products
@@ -144,10 +153,17 @@ class HipOps:
 
     SKINNY_ROWS = 64  # at most this many rows: the weight-streaming kernels
 
+    def _plan(self, what: str, *sizes: int) -> int:
+        key = (what, sizes)
+        v = self._plans.get(key)
+        if v is None:
+            v = self._plans[key] = int(getattr(self._core, what)(*[_c_int(x) for x in sizes]))
+        return v
+
     def _tiled(self, M: int, N: int, K: int) -> bool:
         """Whether the tiled kernel takes this product (always above SKINNY_ROWS rows; below, when the
         weight is large enough that the few-rows kernel's repeated reads of the rows cost more)."""
-        return M > self.SKINNY_ROWS or bool(self._core.ms_prefers_tiled(_c_int(M), _c_int(N), _c_int(K)))
+        return M > self.SKINNY_ROWS or bool(self._plan("ms_prefers_tiled", M, N, K))
 
     def linear_split(self, a: torch.Tensor, w: torch.Tensor, allow_partials: bool = True) -> torch.Tensor:
         """Float32 ``[P, M, N]`` whose sum over P is ``a @ w.T``.  Within one kernel family the cut
@@ -156,17 +172,17 @@ class HipOps:
         :meth:`_tiled`), and the two differ in rounding."""
         M, N, K = self._mm_operands(a, w, "linear_split")
         if self._tiled(M, N, K):
-            P = self._core.ms_tiled_partials(_c_int(M), _c_int(N), _c_int(K)) if allow_partials else 1
+            P = self._plan("ms_tiled_partials", M, N, K) if allow_partials else 1
             if P == 1:
                 return self.linear(a, w, None, out_f32=True).unsqueeze(0)
             out = torch.empty((P, M, N), dtype=torch.float32, device=a.device)
             self._check(self._core, self._core.ms_linear_split_tiled(_ptr(a), _ptr(w), _ptr(out), _c_int(M), _c_int(N),
-                                                                     _c_int(K), _stream()))
+                                                                     _c_int(K), self._stream()))
             return out
-        P = self._core.ms_skinny_partials(_c_int(M), _c_int(N), _c_int(K), _c_int(int(allow_partials)))
+        P = self._plan("ms_skinny_partials", M, N, K, int(allow_partials))
         out = torch.empty((P, M, N), dtype=torch.float32, device=a.device)
         self._check(self._core, self._core.ms_linear_skinny(_ptr(a), _ptr(w), _ptr(out), _c_int(M), _c_int(N), _c_int(K),
-                                                            _c_int(int(allow_partials)), _stream()))
+                                                            _c_int(int(allow_partials)), self._stream()))
         return out
 
     def linear(self, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
@@ -179,7 +195,7 @@ class HipOps:
             self._want(bias, torch.float32, "linear bias", N)
         out = torch.empty((M, N), dtype=torch.float32 if out_f32 else self.dtype, device=a.device)
         self._check(self._core, self._core.ms_linear(_ptr(a), _ptr(w), _ptr(bias), _ptr(out), _c_int(int(out_f32)),
-                                                     _c_int(M), _c_int(N), _c_int(K), _stream()))
+                                                     _c_int(M), _c_int(N), _c_int(K), self._stream()))
         return out
 
     def linear_residual(self, a: torch.Tensor, w: torch.Tensor, x: torch.Tensor) -> Optional[torch.Tensor]:
@@ -190,17 +206,17 @@ class HipOps:
         M, N, K = self._mm_operands(a, w, "linear_residual")
         self._want(x, torch.float32, "residual stream", M, N)
         if not self._tiled(M, N, K):
-            if M > 32 or self._core.ms_skinny_partials(_c_int(M), _c_int(N), _c_int(K), _c_int(1)) > 1:
+            if M > 32 or self._plan("ms_skinny_partials", M, N, K, 1) > 1:
                 return self.linear_split(a, w)
             # all of K inside one block: one writer an element, added in the epilogue (up to 32 rows the
             # kernel has registers to ask for the stream's values ahead; beyond, the next norm adds the sum)
             self._check(self._core, self._core.ms_linear_residual_skinny(_ptr(a), _ptr(w), _ptr(x), _c_int(M), _c_int(N),
-                                                                         _c_int(K), _stream()))
+                                                                         _c_int(K), self._stream()))
             return None
-        if self._core.ms_tiled_partials(_c_int(M), _c_int(N), _c_int(K)) > 1:
+        if self._plan("ms_tiled_partials", M, N, K) > 1:
             return self.linear_split(a, w)
         self._check(self._core, self._core.ms_linear_residual(_ptr(a), _ptr(w), _ptr(x), _c_int(M), _c_int(N), _c_int(K),
-                                                              _stream()))
+                                                              self._stream()))
         return None
 
     def linear_swiglu(self, a: torch.Tensor, w_gate_up: torch.Tensor, intermediate: int) -> torch.Tensor:
@@ -212,7 +228,7 @@ class HipOps:
         out = torch.empty((M, intermediate), dtype=self.dtype, device=a.device)
         fn = self._core.ms_linear_swiglu if self._tiled(M, N, K) else self._core.ms_linear_swiglu_skinny
         self._check(self._core, fn(_ptr(a), _ptr(w_gate_up), _ptr(out), _c_int(M), _c_int(intermediate), _c_int(K),
-                                   _stream()))
+                                   self._stream()))
         return out
 
     # ------------------------------------------------------------------ products with the norm folded in
@@ -220,7 +236,7 @@ class HipOps:
         """Whether a few-rows product over the stream can apply the stream's RMS norm itself (at most
         16 rows, and a shape the few-rows kernel would take anyway)."""
         return (not self._tiled(M, N, K)
-                and bool(self._core.ms_skinny_norm_takes(_c_int(M), _c_int(N), _c_int(K), _c_int(n_partials))))
+                and bool(self._plan("ms_skinny_norm_takes", M, N, K, n_partials)))
 
     def _normed_operands(self, x, partials, norm_w, w, what):
         M, K = x.shape
@@ -244,7 +260,7 @@ class HipOps:
         out = torch.empty((1, M, N), dtype=torch.float32, device=x.device)
         self._check(self._core, self._core.ms_linear_norm_skinny(
             _ptr(x), _ptr(partials), _c_int(P), _c_int(M), _ptr(norm_w), _c_float(eps), _ptr(x_new), _ptr(w), _ptr(out),
-            _c_int(M), _c_int(N), _c_int(K), _stream()))
+            _c_int(M), _c_int(N), _c_int(K), self._stream()))
         return out, x_new
 
     def linear_swiglu_normed(self, x: torch.Tensor, partials: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float,
@@ -257,7 +273,7 @@ class HipOps:
         out = torch.empty((M, intermediate), dtype=self.dtype, device=x.device)
         self._check(self._core, self._core.ms_linear_swiglu_norm_skinny(
             _ptr(x), _ptr(partials), _c_int(P), _c_int(M), _ptr(norm_w), _c_float(eps), _ptr(x_new), _ptr(w_gate_up), _ptr(out),
-            _c_int(M), _c_int(intermediate), _c_int(K), _stream()))
+            _c_int(M), _c_int(intermediate), _c_int(K), self._stream()))
         return out, x_new
 
     # ------------------------------------------------------------------ attention
@@ -306,7 +322,7 @@ class HipOps:
                             _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_pos0), _ptr(work), _c_int(work.shape[0]),
                             _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), _c_int(pages), _c_int(window or 0),
                             _c_float(scale), _c_int(max_key_groups), _c_int(T), _c_int(nsplit), _ptr(part_o), _ptr(part_ml),
-                            _stream()))
+                            self._stream()))
         return out
 
     @staticmethod
@@ -368,7 +384,7 @@ class HipOps:
         self._check(lib, fn(_ptr(qkv), _c_int(P), _c_int(stride), _ptr(bias), _ptr(inv_freq), _ptr(slot_map), _ptr(kpool),
                             _ptr(vpool), _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(block_table),
                             _c_int(block_table.shape[1]), _ptr(seq_pos0), _c_int(S), _c_int(H), _c_int(KV), _c_int(hd),
-                            _c_int(page_size), _c_int(window or 0), _c_int(nsplit), _c_float(scale), _stream()))
+                            _c_int(page_size), _c_int(window or 0), _c_int(nsplit), _c_float(scale), self._stream()))
         return out
 
     def decode_attention(self, q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
@@ -397,7 +413,7 @@ class HipOps:
             part_ml = torch.empty((S, H, nsplit, 2), dtype=torch.float32, device=q.device)
         self._check(lib, fn(_ptr(q), _ptr(kpool), _ptr(vpool), _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(block_table),
                             _c_int(block_table.shape[1]), _ptr(seq_pos0), _c_int(S), _c_int(H), _c_int(KV), _c_int(hd),
-                            _c_int(page_size), _c_int(window or 0), _c_int(nsplit), _c_float(scale), _stream()))
+                            _c_int(page_size), _c_int(window or 0), _c_int(nsplit), _c_float(scale), self._stream()))
         return out
 
     # ------------------------------------------------------------------ sampling
@@ -431,7 +447,7 @@ class HipOps:
             pi = torch.empty((W, chunks), dtype=torch.int32, device=logits.device)
         self._check(self._core, self._core.ms_sample(_ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p),
                                                      _ptr(state), _ptr(tok), _ptr(lp), _ptr(pv), _ptr(pi),
-                                                     _ptr(also_tokens), _c_int(W), _c_int(V), _stream()))
+                                                     _ptr(also_tokens), _c_int(W), _c_int(V), self._stream()))
         return both
 
     def top_logprobs(self, logits: torch.Tensor, inv_t: torch.Tensor, k: int):
@@ -444,7 +460,7 @@ class HipOps:
         tok = torch.empty((W, width), dtype=torch.int32, device=logits.device)
         lp = torch.empty((W, width), dtype=torch.float32, device=logits.device)
         self._check(self._core, self._core.ms_top_logprobs(_ptr(logits), _ptr(inv_t), _ptr(tok), _ptr(lp), _c_int(W),
-                                                           _c_int(V), _c_int(k), _stream()))
+                                                           _c_int(V), _c_int(k), self._stream()))
         return tok[:, :k], lp[:, :k]
 
     def logit_edit(self, logits: torch.Tensor, row_of: torch.Tensor, token: torch.Tensor, delta: torch.Tensor) -> None:
@@ -455,7 +471,7 @@ class HipOps:
         self._want(token, torch.int32, "logit_edit tokens", n)
         self._want(delta, torch.float32, "logit_edit deltas", n)
         self._check(self._core, self._core.ms_logit_edit(_ptr(logits), _c_int(logits.shape[1]), _ptr(row_of), _ptr(token),
-                                                         _ptr(delta), _c_int(n), _stream()))
+                                                         _ptr(delta), _c_int(n), self._stream()))
 
 
 def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
