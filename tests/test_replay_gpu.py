@@ -237,3 +237,39 @@ def test_a_step_shape_that_recurs_is_replayed_from_its_graph(models, which, dtyp
     for i in captured:
         check(captured[i], plain_logits(models, which, dtype, i), dtype, f"{which} request {i} with captured steps")
         check(plain_run[i], plain_logits(models, which, dtype, i), dtype, f"{which} request {i} without captured steps")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("captured", [True, False])
+def test_decode_steps_filled_up_to_a_bucket(models, dtype, captured):
+    """Three, five, six and seven requests decode side by side: the step is filled up to four or eight
+    rows with copies of its first row, whose logits are dropped.  Captured at once, or launched as it
+    is; every request's logits against the plain model, and the cache consistent afterwards."""
+    from machserve_amd.engine import StepEntry
+    which = "A"
+    d, w, sizes, prompts, _ = models[which]
+    seqs = [prompts[i % len(prompts)][:20 + 3 * i] if len(prompts[i % len(prompts)]) >= 20 + 3 * i else prompts[i % len(prompts)]
+            for i in range(7)]
+    lm = engine(models, which, dtype, 40)
+    lm.step.DECODE_CAPTURE_AFTER = 0 if captured else 10 ** 6
+    slots = [lm.cache.admit() for _ in seqs]
+    got = [[] for _ in seqs]
+    fed = []
+    for i, sq in enumerate(seqs):  # all but the last four tokens at once
+        n = max(1, len(sq) - 4)
+        got[i].append(lm.step([StepEntry(slots[i], sq[:n], list(range(n)))]))
+        fed.append(n)
+    for live in ([0, 1, 2], [0, 1, 2, 3, 4], [1, 2, 3, 4, 5, 6], [0, 1, 2, 3, 4, 5, 6], [6, 5, 4, 3, 2]):
+        live = [i for i in live if fed[i] < len(seqs[i])]
+        if not live:
+            continue
+        out = lm.step([StepEntry(slots[i], seqs[i][fed[i]:fed[i] + 1], [0]) for i in live])
+        assert out.shape[0] == len(live)
+        for k, i in enumerate(live):
+            got[i].append(out[k:k + 1])
+            fed[i] += 1
+    lm.cache.check()
+    for i, sq in enumerate(seqs):
+        ww = w if dtype == torch.float32 else {k: v.to(torch.bfloat16).float() if v.dim() == 2 else v for k, v in w.items()}
+        ref = P.forward(ww, sizes, sq)[:fed[i]]
+        check(torch.cat(got[i]), ref, dtype, f"request {i} in filled decode steps")
