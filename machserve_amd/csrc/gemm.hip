@@ -260,7 +260,10 @@ static int plan_tiled_splits(int M, int N, int K) {
     // and the weight is all the traffic: a long K is then cut up to 16 times (7B down projection at 64
     // rows: 49 us with 6 slices, 33 with 12 to 16).
     const int most = M <= 128 ? (K >= 8192 ? 16 : 8) : 6;
-    const int limit = max(1, min(K / (b128 <= 32 ? 256 : 512), most));
+    // (a handful of tiles under few rows - a small projection in a decode step of 33 to 64 requests:
+    // slices of 128, or the step's few blocks leave the chip idle)
+    const int shortest = b128 <= 16 && M <= 128 ? 128 : (b128 <= 32 ? 256 : 512);
+    const int limit = max(1, min(K / shortest, most));
     // The chip holds 512 of the 128x128 blocks at a time (two a CU), and a last round that is nearly
     // empty takes as long as a full one: the fewest slices that fill their rounds to 70 %, else the
     // count that fills them best (1.5B down projection at 2,048 rows, 192 tiles: 3 slices make a
@@ -324,6 +327,9 @@ extern "C" int ms_tiled_partials(int M, int N, int K) { return plan_tiled_splits
 extern "C" int ms_prefers_tiled(int M, int N, int K) {
     if (M > 64) return 1;
 #ifdef MS_ELEM_BF16
+    // Above 32 rows the tiled kernel, with K cut over enough blocks, beats the few-rows kernel for every
+    // weight (0.5B q/k/v projection at 64 rows: 9.7 us few-rows, 4.9 us tiled in seven slices).
+    if (M > 32) return 1;
     // a narrow output with a long K (a down projection): the tiled kernel cuts K over many blocks
     if (N < 2048) return (M >= 48 && K >= 4096) || (M >= 32 && K >= 8192);
     const double nk = (double)N * (double)K;
