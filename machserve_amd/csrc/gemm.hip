@@ -157,13 +157,17 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
     const int row_base = m0 + wm * (BM / WM) + grp * 4;
     const int col_base = n0 + wn * (BN / WN) + r16;
     const bool whole = m0 + BM <= M && n0 + BN <= N && (EPI != EPI_SWIGLU || (n0 + BN) / 2 <= ep.n_out);
-    auto emit = [&](auto checked) {
-        constexpr bool CHECKED = decltype(checked)::value;
+    // A tile at the lower edge of an output whose rows come in whole groups of sixteen (a decode step
+    // of 48 requests in a 64-row tile) skips the groups beyond the last row and stores the others
+    // without checks as well.
+    auto emit = [&](auto checked, auto row_groups) {
+        constexpr bool CHECKED = decltype(checked)::value, ROW_GROUPS = decltype(row_groups)::value;
         if constexpr (EPI == EPI_SWIGLU) {
             static_assert(TN % 2 == 0, "gate and up tiles come in pairs");
             elem_t* out = reinterpret_cast<elem_t*>(ep.out);
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < TM; ++i) {
+                if (ROW_GROUPS && m0 + wm * (BM / WM) + i * 16 >= M) continue;
 #pragma unroll
                 for (int j = 0; j < TN; j += 2) {
                     const int col = (col_base + j * 16 - r16) / 2 + r16;  // tiles 2t, 2t+1 -> output tile t
@@ -174,9 +178,11 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
                         out[(size_t)row * ep.ldo + col] = from_f32<elem_t>(silu_f(acc[i][j][e]) * acc[i][j + 1][e]);
                     }
                 }
+            }
         } else {
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < TM; ++i) {
+                if (ROW_GROUPS && m0 + wm * (BM / WM) + i * 16 >= M) continue;
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
                     const int col = col_base + j * 16;
@@ -192,10 +198,13 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
                         else reinterpret_cast<float*>(ep.out)[o] += v;  // residual stream, 32-bit
                     }
                 }
+            }
         }
     };
-    if (whole) emit(std::false_type{});
-    else emit(std::true_type{});
+    const bool cols_whole = n0 + BN <= N && (EPI != EPI_SWIGLU || (n0 + BN) / 2 <= ep.n_out);
+    if (whole) emit(std::false_type{}, std::false_type{});
+    else if (cols_whole && M % 16 == 0) emit(std::false_type{}, std::true_type{});
+    else emit(std::true_type{}, std::false_type{});
 }
 
 static int g_gemm_config = 0;  // 0: chosen by shape; else a fixed tile (measurements only)
