@@ -5,10 +5,15 @@
 // kernels (crates/mach-model/src/kernels.rs:5772-5798, 6416-6455, 131-160).
 //
 // Both operands are contiguous along K, so a 16x32 MFMA fragment of either is "row
-// l % 16, elements (l / 16) * 8 .. + 8": tiles go global -> registers -> LDS -> fragments.  LDS has
-// 64 banks of 4 bytes; the 16-byte fragment reads of a wave are free of bank conflicts when the
-// row pitch is 32 modulo 64 bytes (measured: pitches of 80 or 144 bytes take twice as long).
-// Two LDS buffers, one barrier per K step.
+// l % 16, elements (l / 16) * 8 .. + 8".  Two LDS buffers, one barrier per K step.  LDS has 64 banks
+// of 4 bytes; the 16-byte fragment reads of a wave are free of bank conflicts when the row pitch is
+// 32 modulo 64 bytes (measured: pitches of 80 or 144 bytes take twice as long), or, with unpadded
+// rows of 128 bytes, when chunk c of row r lies at position c ^ (r & 7).
+// bfloat16 with K steps of 64: tiles go global -> LDS directly (global_load_lds_dwordx4, a wave's
+// 64 lanes fill 1 KB = 8 unpadded rows in lane order, so the swizzle is applied to the global
+// address), and the next step's tile is in flight while this one is multiplied; only a partial last
+// step goes through registers, where what lies beyond K is masked.  The 32-bit build and K steps of
+// 32 go global -> registers -> LDS (padded rows).
 // Every output element is the sum over K in steps of 32 in ascending order whatever the
 // tile shape or the number of rows, so a row's result does not depend on its batch.
 #include <type_traits>
@@ -49,8 +54,15 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
                                                    int M, int N, int K, EpiArgs ep) {
     static_assert(WM * WN == 4, "four waves");
     static_assert(BK % 32 == 0, "K step in MFMA steps of 32");
-    constexpr int LDS_LD = BK + KPAD;
+#ifdef MS_ELEM_BF16
+    constexpr bool DIRECT = BK == 64;
+#else
+    constexpr bool DIRECT = false;
+#endif
+    constexpr int LDS_LD = DIRECT ? BK : BK + KPAD;
     constexpr int CPR = BK / EPC;  // chunks per tile row
+    // where chunk `chunk` of tile row `row` lies in a buffer
+    auto at = [](int row, int chunk) { return row * LDS_LD + (DIRECT ? (chunk ^ (row & 7)) : chunk) * EPC; };
     constexpr int TM = BM / WM / 16, TN = BN / WN / 16;
     constexpr int A_CHUNKS = BM * CPR / 256, W_CHUNKS = BN * CPR / 256;
     static_assert(BM * CPR % 256 == 0 && BN * CPR % 256 == 0, "tile loads divide over the block");
@@ -71,15 +83,18 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
     u32x4 ra[A_CHUNKS], rw[W_CHUNKS];
     const elem_t* pa[A_CHUNKS];
     const elem_t* pw[W_CHUNKS];
+    // Thread t owns position (t + i * 256) % CPR of tile row (t + i * 256) / CPR; with swizzled rows that
+    // position holds another chunk of K, the same one for every i (256 / CPR rows on is a multiple of 8).
+    const int my_chunk = DIRECT ? (tid % CPR) ^ ((tid / CPR) & 7) : tid % CPR;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
         const int c = tid + i * 256;
-        pa[i] = A + (size_t)min(m0 + c / CPR, M - 1) * K + (c % CPR) * EPC;
+        pa[i] = A + (size_t)min(m0 + c / CPR, M - 1) * K + my_chunk * EPC;
     }
 #pragma unroll
     for (int i = 0; i < W_CHUNKS; ++i) {
         const int c = tid + i * 256;
-        pw[i] = W + (size_t)min(n0 + c / CPR, N - 1) * K + (c % CPR) * EPC;
+        pw[i] = W + (size_t)min(n0 + c / CPR, N - 1) * K + my_chunk * EPC;
     }
     auto load_global = [&](int k0) {
 #pragma unroll
@@ -88,7 +103,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
         for (int i = 0; i < W_CHUNKS; ++i) rw[i] = *reinterpret_cast<const u32x4*>(pw[i] + k0);
     };
     auto load_global_tail = [&](int k0) {
-        const int kk = k0 + (tid % CPR) * EPC;  // 256 % CPR == 0: the same K chunk for all of a thread's loads
+        const int kk = k0 + my_chunk * EPC;  // the same K chunk for all of a thread's loads
         const bool in = kk < k_end;
         const uint32_t keep = opaque(in ? 0xffffffffu : 0u);
 #pragma unroll
@@ -105,13 +120,40 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
     auto store_lds = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < A_CHUNKS; ++i) {
-            const int c = tid + i * 256, row = c / CPR, cc = c % CPR;
-            *reinterpret_cast<u32x4*>(&As[buf][row * LDS_LD + cc * EPC]) = ra[i];
+            const int c = tid + i * 256, row = c / CPR;
+            *reinterpret_cast<u32x4*>(&As[buf][at(row, my_chunk)]) = ra[i];
         }
 #pragma unroll
         for (int i = 0; i < W_CHUNKS; ++i) {
-            const int c = tid + i * 256, row = c / CPR, cc = c % CPR;
-            *reinterpret_cast<u32x4*>(&Ws[buf][row * LDS_LD + cc * EPC]) = rw[i];
+            const int c = tid + i * 256, row = c / CPR;
+            *reinterpret_cast<u32x4*>(&Ws[buf][at(row, my_chunk)]) = rw[i];
+        }
+    };
+#ifdef MS_ELEM_BF16
+    // One K step of both tiles straight into LDS buffer `buf`: lane l of a wave's load lands at the wave's
+    // base + 16 l.  Written in assembly: of a load that it knows to write LDS the compiler makes every later
+    // LDS read wait (vmcnt(0)), and nothing would be in flight during the multiplications; the waits are
+    // explicit instead (`step_barrier`).
+    auto load_direct = [&](int k0, int buf) {
+        auto issue = [](const elem_t* g, const elem_t* l) {
+            const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)l);
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(base) : "memory", "m0");
+        };
+#pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) issue(pa[i] + k0, &As[buf][(i * 256 + wave * 64) * EPC]);
+#pragma unroll
+        for (int i = 0; i < W_CHUNKS; ++i) issue(pw[i] + k0, &Ws[buf][(i * 256 + wave * 64) * EPC]);
+    };
+#endif
+    // End of a K step: this wave's loads and LDS accesses have completed, then everybody's.
+    auto step_barrier = [&]() {
+        if constexpr (DIRECT) {
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+        } else {
+            __syncthreads();
         }
     };
 
@@ -125,28 +167,62 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
     const int k_begin = split * ep.k_per_split;
     const int nk = ceil_div(k_end - k_begin, BK);
     const bool partial = (k_end - k_begin) % BK != 0;  // the last step is a partial one
-    if (nk == 1 && partial) load_global_tail(k_begin);
-    else load_global(k_begin);
-    store_lds(0);
-    __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 2 < nk || (kt + 2 == nk && !partial)) load_global(k_begin + (kt + 1) * BK);
-        else if (kt + 1 < nk) load_global_tail(k_begin + (kt + 1) * BK);
+    auto multiply = [&](int buf) {
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 32) {
             Frag fa[TM], fb[TN];
+            if constexpr (DIRECT) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i) fa[i] = frag_load(&As[buf][(wm * (BM / WM) + i * 16 + r16) * LDS_LD + kk + grp * 8]);
+                for (int i = 0; i < TM; ++i) fa[i] = frag_load(&As[buf][at(wm * (BM / WM) + i * 16 + r16, kk / EPC + grp)]);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) fb[j] = frag_load(&Ws[buf][(wn * (BN / WN) + j * 16 + r16) * LDS_LD + kk + grp * 8]);
+                for (int j = 0; j < TN; ++j) fb[j] = frag_load(&Ws[buf][at(wn * (BN / WN) + j * 16 + r16, kk / EPC + grp)]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < TM; ++i) fa[i] = frag_load(&As[buf][(wm * (BM / WM) + i * 16 + r16) * LDS_LD + kk + grp * 8]);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) fb[j] = frag_load(&Ws[buf][(wn * (BN / WN) + j * 16 + r16) * LDS_LD + kk + grp * 8]);
+            }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j) mma_16x16x32(acc[i][j], fa[i], fb[j]);
         }
-        if (kt + 1 < nk) store_lds(buf ^ 1);
+    };
+    if constexpr (DIRECT) {
+#ifdef MS_ELEM_BF16
+        if (nk == 1 && partial) {
+            load_global_tail(k_begin);
+            store_lds(0);
+        } else {
+            load_direct(k_begin, 0);
+        }
+        step_barrier();
+        for (int kt = 0; kt < nk; ++kt) {
+            const int buf = kt & 1;
+            // the next step: a whole one straight into the other buffer, a partial one into registers
+            const bool tail_next = kt + 2 == nk && partial;
+            if (kt + 1 < nk) {
+                if (tail_next) load_global_tail(k_begin + (kt + 1) * BK);
+                else load_direct(k_begin + (kt + 1) * BK, buf ^ 1);
+            }
+            multiply(buf);
+            if (tail_next) store_lds(buf ^ 1);
+            step_barrier();
+        }
+#endif
+    } else {
+        if (nk == 1 && partial) load_global_tail(k_begin);
+        else load_global(k_begin);
+        store_lds(0);
         __syncthreads();
+        for (int kt = 0; kt < nk; ++kt) {
+            const int buf = kt & 1;
+            if (kt + 2 < nk || (kt + 2 == nk && !partial)) load_global(k_begin + (kt + 1) * BK);
+            else if (kt + 1 < nk) load_global_tail(k_begin + (kt + 1) * BK);
+            multiply(buf);
+            if (kt + 1 < nk) store_lds(buf ^ 1);
+            __syncthreads();
+        }
     }
 
     // Epilogue.  Lane holds rows grp * 4 + e of column r16 in each 16x16 tile: sixteen lanes write
