@@ -69,7 +69,9 @@ def test_rmsnorm(dtype, T, d, eps):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 16, 8), (7, 1000, 200), (64, 130, 896), (65, 257, 72), (300, 896, 4864),
-                                   (129, 9728 + 16, 64)])
+                                   (129, 9728 + 16, 64),
+                                   # the tiled kernel's K steps: one partial step, one whole, two whole, whole + partial
+                                   (70, 100, 40), (130, 64, 64), (100, 96, 128), (513, 1200, 136), (2048, 1152, 904)])
 def test_linear(dtype, M, N, K):
     ops = ops_for(dtype)
     a, w = rnd((M, K), dtype, 5), rnd((N, K), dtype, 6, K ** -0.5)
