@@ -49,7 +49,7 @@ __device__ __forceinline__ float silu_f(float g) {
 #endif
 }
 
-template <int BM, int BN, int WM, int WN, int BK, int EPI>
+template <int BM, int BN, int WM, int WN, int BK, int EPI, int STAGES = 2>
 __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A, const elem_t* __restrict__ W,
                                                    int M, int N, int K, EpiArgs ep) {
     static_assert(WM * WN == 4, "four waves");
@@ -66,8 +66,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
     constexpr int TM = BM / WM / 16, TN = BN / WN / 16;
     constexpr int A_CHUNKS = BM * CPR / 256, W_CHUNKS = BN * CPR / 256;
     static_assert(BM * CPR % 256 == 0 && BN * CPR % 256 == 0, "tile loads divide over the block");
-    __shared__ __attribute__((aligned(16))) elem_t As[2][BM * LDS_LD];
-    __shared__ __attribute__((aligned(16))) elem_t Ws[2][BN * LDS_LD];
+    static_assert(STAGES == 2 || DIRECT, "more than two LDS buffers only with direct loads");
+    __shared__ __attribute__((aligned(16))) elem_t As[STAGES][BM * LDS_LD];
+    __shared__ __attribute__((aligned(16))) elem_t Ws[STAGES][BN * LDS_LD];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
@@ -188,7 +189,37 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
                 for (int j = 0; j < TN; ++j) mma_16x16x32(acc[i][j], fa[i], fb[j]);
         }
     };
-    if constexpr (DIRECT) {
+    if constexpr (DIRECT && STAGES > 2) {
+#ifdef MS_ELEM_BF16
+        // A block that is alone on its CU (few tiles: one tile of rows under a weight of a few hundred column
+        // tiles) has nobody to hide its loads behind, and with one step in flight every step costs a trip to
+        // memory.  Here STAGES - 1 steps are in flight: the loads of step kt + STAGES - 1 go out before step
+        // kt is multiplied, and the step's end waits only for the loads of step kt + 1 (a wave's loads
+        // complete in order, so "all but the last (STAGES - 2) steps' loads" is a count).  The launcher
+        // gives this variant whole K steps only.
+        constexpr int PER_STEP = A_CHUNKS + W_CHUNKS;
+        static_assert(PER_STEP * (STAGES - 2) <= 63, "the wait count is a 6-bit field");
+        for (int s = 0; s < STAGES - 1; ++s)
+            if (s < nk) load_direct(k_begin + s * BK, s);
+        // the first step's loads: the earliest of up to STAGES - 1 steps' loads
+        __builtin_amdgcn_sched_barrier(0);
+        if (nk >= STAGES - 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_STEP * (STAGES - 2)) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        for (int kt = 0; kt < nk; ++kt) {
+            const bool more = kt + STAGES - 1 < nk;
+            if (more) load_direct(k_begin + (kt + STAGES - 1) * BK, (kt + STAGES - 1) % STAGES);
+            multiply(kt % STAGES);
+            __builtin_amdgcn_sched_barrier(0);
+            // towards the end fewer steps are in flight behind step kt + 1: wait for everything
+            if (more) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(PER_STEP * (STAGES - 2)) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#endif
+    } else if constexpr (DIRECT) {
 #ifdef MS_ELEM_BF16
         if (nk == 1 && partial) {
             load_global_tail(k_begin);
@@ -298,6 +329,13 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
     ep.split_stride = (size_t)M * N;
     const unsigned ns = (unsigned)ceil_div(K, ep.k_per_split);
     MS_REQUIRE(nsplit == 1 || (int)ns == nsplit, "gemm: %d K slices asked for, %u fit", nsplit, ns);
+#define MS_GEMM_DEEP(BM_, BN_, WM_, WN_, BK_, ST_)                                                                         \
+    do {                                                                                                                  \
+        const long nb = (long)ceil_div(M, BM_) * ceil_div(N, BN_);                                                        \
+        hipLaunchKernelGGL((gemm_kernel<BM_, BN_, WM_, WN_, BK_, EPI, ST_>), dim3((unsigned)nb, ns), dim3(256), 0, stream, \
+                           A, W, M, N, K, ep);                                                                            \
+        return check_launch("gemm " #BM_ "x" #BN_ "x" #BK_ " deep");                                                      \
+    } while (0)
 #define MS_GEMM(BM_, BN_, WM_, WN_, BK_)                                                                              \
     do {                                                                                                              \
         const long nb = (long)ceil_div(M, BM_) * ceil_div(N, BN_);                                                    \
@@ -311,6 +349,9 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
     if (forced == 2) MS_GEMM(128, 128, 2, 2, 64);
     if (forced == 5) MS_GEMM(128, 64, 2, 2, 64);
     if (forced == 6) MS_GEMM(64, 64, 2, 2, 64);
+    const bool whole_steps = ep.k_per_split % 64 == 0 && K % 64 == 0;
+    if (forced == 7 && whole_steps) MS_GEMM_DEEP(64, 64, 2, 2, 64, 3);
+    if (forced == 8 && whole_steps) MS_GEMM_DEEP(64, 64, 2, 2, 64, 4);
     // The largest tile that still gives every CU of the chip a block or two, with K steps of 64 (half
     // the barriers of steps of 32).  Measured on M = 512..8192 of the 0.5B shapes; larger wave tiles
     // (256x128) lose: their accumulators no longer fit the registers of two blocks a CU.
@@ -325,11 +366,16 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
             MS_GEMM(128, 64, 2, 2, 32);
         }
     }
+    // At most two blocks a CU, each a chain of K steps: four LDS buffers keep three steps in flight (0.5B
+    // gate/up product at 64 rows, 152 blocks of 14 steps: 10.5 -> 7.8 us; 1.5B: 23.7 -> 21.1; with more
+    // blocks than that the blocks hide each other's loads and the two-buffer kernel is as fast).
+    if ((long)ceil_div(M, 64) * ceil_div(N, 64) * ns <= 512 && whole_steps && ep.k_per_split >= 256) MS_GEMM_DEEP(64, 64, 2, 2, 64, 4);
     MS_GEMM(64, 64, 2, 2, 64);
 #else
     MS_GEMM(64, 64, 2, 2, 32);
 #endif
 #undef MS_GEMM
+#undef MS_GEMM_DEEP
 }
 
 // K slices for a product whose consumer adds partial sums: enough 128x128 blocks to fill the chip,

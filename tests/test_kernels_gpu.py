@@ -71,7 +71,9 @@ def test_rmsnorm(dtype, T, d, eps):
 @pytest.mark.parametrize("M,N,K", [(1, 16, 8), (7, 1000, 200), (64, 130, 896), (65, 257, 72), (300, 896, 4864),
                                    (129, 9728 + 16, 64),
                                    # the tiled kernel's K steps: one partial step, one whole, two whole, whole + partial
-                                   (70, 100, 40), (130, 64, 64), (100, 96, 128), (513, 1200, 136), (2048, 1152, 904)])
+                                   (70, 100, 40), (130, 64, 64), (100, 96, 128), (513, 1200, 136), (2048, 1152, 904),
+                                   # few tiles, whole K steps: four LDS buffers in turn, with four, five, seven and nineteen steps
+                                   (64, 200, 256), (48, 264, 320), (40, 130, 448), (100, 72, 1216)])
 def test_linear(dtype, M, N, K):
     ops = ops_for(dtype)
     a, w = rnd((M, K), dtype, 5), rnd((N, K), dtype, 6, K ** -0.5)
@@ -168,7 +170,8 @@ def test_products_with_the_norm_folded_in(dtype, M, N, K, NP):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,I,K", [(1, 16, 8), (9, 160, 64), (70, 328, 192), (200, 4864, 896), (64, 4864, 896), (33, 264, 136)])
+@pytest.mark.parametrize("M,I,K", [(1, 16, 8), (9, 160, 64), (70, 328, 192), (200, 4864, 896), (64, 4864, 896), (33, 264, 136),
+                                   (64, 328, 256), (50, 1000, 576)])
 def test_linear_swiglu(dtype, M, I, K):
     from machserve_amd.kernels import interleave_gate_up
     ops = ops_for(dtype)
