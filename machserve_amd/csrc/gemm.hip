@@ -461,11 +461,23 @@ extern "C" int ms_prefers_tiled(int M, int N, int K) {
     // Above 32 rows the tiled kernel, with K cut over enough blocks, beats the few-rows kernel for every
     // weight (0.5B q/k/v projection at 64 rows: 9.7 us few-rows, 4.9 us tiled in seven slices).
     if (M > 32) return 1;
-    // a narrow output with a long K (a down projection): the tiled kernel cuts K over many blocks
-    if (N < 2048) return (M >= 48 && K >= 4096) || (M >= 32 && K >= 8192);
     const double nk = (double)N * (double)K;
-    if (M >= 8 && nk >= 100e6) return 1;  // a vocabulary-sized product
-    return M >= 16 && nk * M >= 280e6;
+    if (N >= 2048) {
+        // A large weight under a wide output: the tiled kernel's blocks each stream their columns' rows of the
+        // weight step after step, several steps in flight, while every wave of the few-rows kernel asks for its
+        // whole share at once and then waits.  From one row on (decode steps of the 1.5B and 7B layer sizes at
+        // batch 1, 2, 4, 8: 7 to 12 % shorter; the vocabulary-sized head of every shape); a smaller weight
+        // (0.5B gate/up) from 17 rows on, where the few-rows kernel can no longer apply the norm itself and
+        // re-reads its rows for every 32 columns (batch 32: 1.53 -> 1.40 ms a step).
+        return nk >= 10e6 || M >= 17;
+    }
+    if (N >= 1024) {
+        // a projection of the width (q/k/v, output): from 16 rows, or 8 if it is not small (batch 32: 1.40 ->
+        // 1.36 ms a step; 0.5B q/k/v at 8 rows is faster in the few-rows kernel)
+        return M >= 16 || (M >= 8 && nk >= 2e6);
+    }
+    // a narrow output with a long K (a down projection): the tiled kernel cuts K over many blocks
+    return M >= 32 && K >= 4096;
 #else
     return 0;
 #endif
