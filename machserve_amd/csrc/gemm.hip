@@ -350,7 +350,6 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
     if (forced == 5) MS_GEMM(128, 64, 2, 2, 64);
     if (forced == 6) MS_GEMM(64, 64, 2, 2, 64);
     const bool whole_steps = ep.k_per_split % 64 == 0 && K % 64 == 0;
-    if (forced == 7 && whole_steps) MS_GEMM_DEEP(64, 64, 2, 2, 64, 3);
     if (forced == 8 && whole_steps) MS_GEMM_DEEP(64, 64, 2, 2, 64, 4);
     // The largest tile that still gives every CU of the chip a block or two, with K steps of 64 (half
     // the barriers of steps of 32).  Measured on M = 512..8192 of the 0.5B shapes; larger wave tiles
