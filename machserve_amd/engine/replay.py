@@ -70,5 +70,6 @@ def main(argv=None) -> int:
         sys.stdout.write(msg + "\n")
         sys.stdout.flush()
 
-    replay(lm, sys.stdin, args.out, say)
+    # line by line as they arrive: the sender waits for each step's "done" before it writes the next
+    replay(lm, iter(sys.stdin.readline, ""), args.out, say)
     return 0

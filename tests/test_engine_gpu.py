@@ -218,6 +218,40 @@ def test_trace_run_program(dirs, tmp_path):
             assert (got - ref).abs().max() <= tolr * (1 + ref.abs().max())
 
 
+def test_trace_run_takes_a_step_only_after_the_one_before_is_done(dirs, tmp_path):
+    """The sender writes a step, waits for its 'done' line, and only then writes the next; a request is left
+    out of a step and goes on later; the input's end ends the program with 0."""
+    w, sizes = read_for_plain(dirs["B"])
+    a, b = random_prompt(70, 1000, 3), random_prompt(9, 1000, 4)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:40], "want": [39]}], "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": b, "want": [8]}], "end": ["b"]},
+        {"step": 2, "entries": [{"id": "a", "tokens": a[40:68], "want": [0]}], "end": []},
+        {"step": 3, "entries": [{"id": "a", "tokens": a[68:], "want": [0, 1]}], "end": ["a"]},
+    ]
+    out = tmp_path / "out"
+    proc = subprocess.Popen([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", dirs["B"], "--dtype", "float32",
+                             "--out", str(out), "--max-tokens", "128"], stdin=subprocess.PIPE, stdout=subprocess.PIPE,
+                            stderr=subprocess.DEVNULL, text=True)
+    try:
+        for s in steps:
+            proc.stdin.write(json.dumps(s) + "\n")
+            proc.stdin.flush()
+            assert proc.stdout.readline().split() == ["done", str(s["step"])]
+            assert (out / f"{s['step']}.f32").exists(), "a step's logits are there when its 'done' line is"
+        proc.stdin.close()
+        assert proc.wait(timeout=60) == 0
+    finally:
+        if proc.poll() is None:
+            proc.kill()
+    ra, rb = P.forward(w, sizes, a), P.forward(w, sizes, b)
+    want = {0: ra[[39]], 1: rb[[8]], 2: ra[[40]], 3: ra[[68, 69]]}
+    for s, ref in want.items():
+        got = torch.from_numpy(np.fromfile(out / f"{s}.f32", dtype="<f4").reshape(-1, 1000))
+        assert got.shape == ref.shape
+        assert (got - ref).abs().max() <= 2e-5 * (1 + ref.abs().max())
+
+
 def test_command_line(dirs, tmp_path):
     w, sizes = read_for_plain(dirs["A"])
     p = random_prompt(7, 512, 9)
