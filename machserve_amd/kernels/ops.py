@@ -79,6 +79,18 @@ class HipOps:
         if shape and tuple(t.shape) != tuple(shape):
             raise KernelError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
 
+    def require_sizes(self, what: str, reductions=(), head_dim: Optional[int] = None) -> None:
+        """Refuses, when a model is put together, sizes that the kernels do not take: a product sums over a
+        multiple of 8 elements, a head has a multiple of 16 up to the largest attention tile."""
+        for name, k in reductions:
+            if k <= 0 or k % 8:
+                raise KernelError(f"{what}: {name} = {k} must be a positive multiple of 8 (the products sum over it in 16-byte chunks)")
+        if head_dim is not None:
+            try:
+                build.attention_tile_for(head_dim)
+            except build.BuildError as e:
+                raise KernelError(f"{what}: {e}") from None
+
     # ------------------------------------------------------------------ elementwise
     def embed(self, tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
         T, (V, d) = tokens.numel(), table.shape

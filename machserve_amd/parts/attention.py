@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import Mixer, PagedKVRequest, PendingNorm, SharedKVRequest, TensorDecl
+from .base import Mixer, PagedKVRequest, PendingNorm, SharedKVRequest, TensorDecl, require_kernel_sizes
 from .registry import POSITION_ENCODINGS, register_mixer
 
 
@@ -25,6 +25,7 @@ class Attention(Mixer):
         if s.heads % s.kv_heads:
             raise ValueError(f"attention: {s.heads} heads are not a multiple of {s.kv_heads} key/value heads")
         self.nq, self.nkv = s.heads * s.head_dim, s.kv_heads * s.head_dim
+        require_kernel_sizes(rt, "attention", [("hidden size", s.hidden), ("heads x head size", self.nq)], s.head_dim)
         self.scale = float(s.head_dim) ** -0.5
         self.position = POSITION_ENCODINGS.build(s.position, rt) if s.position is not None else None
         self.writes_cache = s.kv_source is None

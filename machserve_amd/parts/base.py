@@ -182,6 +182,14 @@ class PendingNorm:
         return self.stream.normed_linear_swiglu(self.weight, self.eps, w_gate_up, intermediate)
 
 
+def require_kernel_sizes(rt: "Runtime", what: str, reductions=(), head_dim: Optional[int] = None) -> None:
+    """Lets the kernels refuse sizes they do not take while the model is built, with the size's name
+    (``reductions``: pairs of name and size that products sum over), rather than at the first step."""
+    check = getattr(rt.ops, "require_sizes", None)
+    if check is not None:
+        check(what, reductions, head_dim)
+
+
 class Part:
     takes_pending_norm = False  # True: forward's normalised input may be a PendingNorm
 

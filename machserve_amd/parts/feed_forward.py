@@ -5,7 +5,7 @@ the 32-bit stream."""
 from __future__ import annotations
 
 from ..kernels.ops import interleave_gate_up
-from .base import FeedForward, PendingNorm, TensorDecl
+from .base import FeedForward, PendingNorm, TensorDecl, require_kernel_sizes
 from .registry import register_feed_forward
 
 
@@ -17,6 +17,7 @@ class GatedMlp(FeedForward):
         super().__init__(spec, rt)
         if spec.activation != "silu":
             raise ValueError(f"gated_mlp: activation {spec.activation!r} is not built (silu only)")
+        require_kernel_sizes(rt, "gated_mlp", [("hidden size", spec.hidden), ("intermediate size", spec.intermediate)])
 
     def tensor_decls(self):
         s = self.spec

@@ -10,7 +10,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..config.specs import ModelSpec
-from .base import Block, Part, ResidualStream, Runtime, StepContext, TensorDecl
+from .base import Block, Part, ResidualStream, Runtime, StepContext, TensorDecl, require_kernel_sizes
 from .registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
 
 
@@ -56,6 +56,7 @@ class DecoderModel:
     def __init__(self, spec: ModelSpec, rt: Runtime):
         spec.validate()
         self.spec, self.rt = spec, rt
+        require_kernel_sizes(rt, "output head", [("width", spec.embedding.width)])
         self.embedding = Embedding(spec.embedding, rt)
         self.blocks: List[Block] = []
         for layer in spec.layers:

@@ -35,6 +35,46 @@ def test_greedy_generation_through_the_entry_point(dirs, which):
         assert g == P.greedy_generate(w, sizes, p, 12)
 
 
+ODD = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_size": 88, "num_hidden_layers": 2,
+    "num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 80, "intermediate_size": 104, "vocab_size": 333,
+    "max_position_embeddings": 128, "rms_norm_eps": 2e-6, "rope_theta": 3000.0, "tie_word_embeddings": True,
+    "hidden_act": "silu", "use_sliding_window": False,
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_at_the_edge_of_what_the_kernels_take(tmp_path, dtype):
+    """Width, intermediate size and vocabulary that are multiples of 8 only, three heads in one group, a head
+    size that fills five sixths of its tile: logits of a prompt in portions against the plain model."""
+    from machserve_amd.engine import StepEntry, load_model
+    from machserve_amd.weights import write_random_model
+    d = write_random_model(dict(ODD), 5, str(tmp_path / "odd"), torch.float32)
+    w, sizes = read_for_plain(d)
+    if dtype == "bfloat16":
+        w = {k: v.to(torch.bfloat16).float() if v.dim() == 2 else v for k, v in w.items()}
+    p = random_prompt(50, 333, 8)
+    ref = P.forward(w, sizes, p)
+    lm = load_model(d, dtype=dtype, device=DEV, page_size=16, num_pages=4)
+    slot = lm.cache.admit()
+    got = [lm.step([StepEntry(slot, p[:33], list(range(33)))]), lm.step([StepEntry(slot, p[33:35], [0, 1])])]
+    got += [lm.step([StepEntry(slot, p[i:i + 1], [0])]) for i in range(35, 50)]
+    got = torch.cat(got).float().cpu()
+    scale = ref.abs().max().item()
+    allowed = 2e-5 + 2e-5 * scale if dtype == "float32" else 3e-2 * scale
+    assert (got - ref).abs().max().item() <= allowed
+
+
+@pytest.mark.parametrize("key,value,said", [("intermediate_size", 100, "intermediate size = 100"), ("hidden_size", 92, "width = 92"),
+                                            ("head_dim", 72, "head size 72")])
+def test_sizes_the_kernels_do_not_take_are_refused_when_the_model_is_built(tmp_path, key, value, said):
+    from machserve_amd.engine import load_model
+    from machserve_amd.weights import write_random_model
+    d = write_random_model(dict(ODD, **{key: value}), 5, str(tmp_path / "refused"), torch.float32)
+    with pytest.raises(Exception, match=said):
+        load_model(d, dtype="bfloat16", device=DEV, page_size=16, num_pages=4)
+
+
 def test_eos_stops_generation(dirs):
     import machserve_amd
     w, sizes = read_for_plain(dirs["A"])
