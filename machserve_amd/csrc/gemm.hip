@@ -389,10 +389,14 @@ static int plan_tiled_splits(int M, int N, int K) {
     // portion of a few hundred rows - slices of 256 still pay).  With few rows the partial sums are small
     // and the weight is all the traffic: a long K is then cut up to 16 times (7B down projection at 64
     // rows: 49 us with 6 slices, 33 with 12 to 16).
-    const int most = M <= 128 ? (K >= 8192 ? 16 : 8) : 6;
+    // (measured again at 33 and 64 rows of the three layer sizes: 1.5B down projection, K = 8,960, 9.0 us in 10
+    // slices, 10.0 in 16, and its consumer sums fewer planes)
+    const int most = M <= 128 ? (K >= 16384 ? 16 : (K >= 8192 ? 10 : 8)) : 6;
     // (a handful of tiles under few rows - a small projection in a decode step of 33 to 64 requests:
     // slices of 128, or the step's few blocks leave the chip idle)
-    const int shortest = b128 <= 16 && M <= 128 ? 128 : (b128 <= 32 ? 256 : 512);
+    // (from K = 1,536 on slices of 256, which run with four LDS buffers in turn: 1.5B output projection at 64
+    // rows 5.1 us in 6 slices, 5.5 in 8)
+    const int shortest = b128 <= 16 && M <= 128 ? (K >= 1536 ? 256 : 128) : (b128 <= 32 ? 256 : 512);
     const int limit = max(1, min(K / shortest, most));
     // The chip holds 512 of the 128x128 blocks at a time (two a CU), and a last round that is nearly
     // empty takes as long as a full one: the fewest slices that fill their rounds to 70 %, else the
