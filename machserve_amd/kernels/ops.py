@@ -173,8 +173,9 @@ class HipOps:
         return v
 
     def _tiled(self, M: int, N: int, K: int) -> bool:
-        """Whether the tiled kernel takes this product (always above SKINNY_ROWS rows; below, when the
-        weight is large enough that the few-rows kernel's repeated reads of the rows cost more)."""
+        """Whether the tiled kernel takes this product: always above SKINNY_ROWS rows; below, where it was
+        measured faster (in bfloat16 every large weight from one row on, because its blocks stream the
+        weight with several K steps in flight, and smaller ones from 8 to 32 rows on; never in 32-bit)."""
         return M > self.SKINNY_ROWS or bool(self._plan("ms_prefers_tiled", M, N, K))
 
     def linear_split(self, a: torch.Tensor, w: torch.Tensor, allow_partials: bool = True) -> torch.Tensor:
