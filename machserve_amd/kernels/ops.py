@@ -14,7 +14,14 @@ import torch
 
 from . import build
 
-_c_int, _c_float, _c_void = ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+_c_float, _c_void = ctypes.c_float, ctypes.c_void_p
+
+
+def _c_int(v) -> int:
+    """An argument of C type int: ctypes passes a Python int as one by itself (and refuses one that does not
+    fit), which spares an object per argument; pointers and floats need their wrappers."""
+    return int(v)
+
 
 
 class KernelError(RuntimeError):
@@ -73,10 +80,12 @@ class HipOps:
             raise KernelError(lib.ms_last_error().decode())
 
     def _want(self, t: torch.Tensor, dtype, name: str, *shape):
-        if t.device.type != "cuda" or t.dtype != dtype or not t.is_contiguous():
+        """The operand is what the kernel assumes: on the GPU, of this type, contiguous, of this shape if one
+        is given.  Runs for every operand of every launch, so the good case is a few attribute reads."""
+        if not t.is_cuda or t.dtype is not dtype or not t.is_contiguous():
             raise KernelError(f"{name}: expected a contiguous {dtype} GPU tensor, got {t.dtype} on {t.device}"
                               f"{'' if t.is_contiguous() else ' (not contiguous)'}")
-        if shape and tuple(t.shape) != tuple(shape):
+        if shape and t.shape != shape:
             raise KernelError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
 
     def require_sizes(self, what: str, reductions=(), head_dim: Optional[int] = None) -> None:
