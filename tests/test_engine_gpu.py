@@ -101,6 +101,35 @@ def test_generation_under_page_pressure_equals_roomy_generation(dirs):
     assert n0 == 0 and n1 > 0 and roomy == tight
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_arrivals_under_page_pressure_equal_the_plain_model(dirs, seed):
+    """Requests of random lengths arrive at random steps in an engine with few slots, few pages and a small
+    token budget: portions, decoded tokens, ends, slot and page reuse and preemptions in whatever order the
+    seed brings; every request's greedy tokens against the plain model, and no page lost at the end."""
+    import random
+    from machserve_amd.engine import Engine
+    w, sizes = read_for_plain(dirs["B"])
+    rnd_ = random.Random(seed)
+    reqs = [(random_prompt(rnd_.randrange(1, 90), 1000, 100 * seed + i), rnd_.randrange(1, 18)) for i in range(12)]
+    eng = Engine.from_dir(dirs["B"], dtype="float32", page_size=16, num_pages=10, capacity=4,
+                          max_batch_tokens=rnd_.choice([24, 40, 64]))
+    arrivals = sorted(rnd_.randrange(0, 60) for _ in reqs)
+    ids, step, nxt = [], 0, 0
+    while nxt < len(reqs) or eng.has_work():
+        while nxt < len(reqs) and (arrivals[nxt] <= step or not eng.has_work()):
+            ids.append(eng.add(reqs[nxt][0], reqs[nxt][1]))
+            nxt += 1
+        (eng.step_pipelined if step % 3 else eng.step)()
+        step += 1
+        assert step < 5000
+    done = eng.scheduler.finished
+    eng.loaded.cache.check()
+    assert not eng.loaded.cache.live_requests()
+    for rid, (prompt, max_new) in zip(ids, reqs):
+        assert done[rid].generated == P.greedy_generate(w, sizes, prompt, max_new), f"request {rid} ({len(prompt)} tokens, {max_new} new)"
+    print(f"seed {seed}: {step} steps, {sum(done[r].preemptions for r in ids)} preemptions")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_steps_launched_ahead_give_what_steps_one_at_a_time_give(dirs, dtype):
     """Engine.run launches a decode step before the samples of the step before have reached the
