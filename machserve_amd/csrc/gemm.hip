@@ -39,6 +39,11 @@ struct EpiArgs {
     int n_out;          // SWIGLU: number of output columns (intermediate size)
     int k_per_split;    // K range of one blockIdx.y slice (multiple of 32); K itself without split
     size_t split_stride;  // STORE_F32 with gridDim.y > 1: elements between the slices' outputs
+    // a factor a row for the finished sums (the RMS norm of rows that came in multiplied by the norm's weight only):
+    // 1 / sqrt(sum over parts of row_ss[part, row] / K + ss_eps)
+    const float* row_ss;  // [ss_parts, M] or null
+    int ss_parts;
+    float ss_eps;
 };
 
 __device__ __forceinline__ float silu_f(float g) {
@@ -49,7 +54,7 @@ __device__ __forceinline__ float silu_f(float g) {
 #endif
 }
 
-template <int BM, int BN, int WM, int WN, int BK, int EPI, int STAGES = 2>
+template <int BM, int BN, int WM, int WN, int BK, int EPI, int STAGES = 2, bool SCALED = false>
 __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A, const elem_t* __restrict__ W,
                                                    int M, int N, int K, EpiArgs ep) {
     static_assert(WM * WN == 4, "four waves");
@@ -67,6 +72,11 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
     constexpr int A_CHUNKS = BM * CPR / 256, W_CHUNKS = BN * CPR / 256;
     static_assert(BM * CPR % 256 == 0 && BN * CPR % 256 == 0, "tile loads divide over the block");
     static_assert(STAGES == 2 || DIRECT, "more than two LDS buffers only with direct loads");
+    static_assert(!SCALED || (STAGES > 2 && EPI == EPI_SWIGLU), "row factors: built for the gated product with several steps in flight");
+    static_assert(256 % BM == 0 || !SCALED, "threads are dealt to the rows");
+    __shared__ float ss_q[SCALED ? 256 / BM : 1][SCALED ? BM : 1];  // the rows' sums of squares, in 256 / BM interleaved shares
+    float ss_v[SCALED ? 8 : 1];
+    int ss_r = 0;
     __shared__ __attribute__((aligned(16))) elem_t As[STAGES][BM * LDS_LD];
     __shared__ __attribute__((aligned(16))) elem_t Ws[STAGES][BN * LDS_LD];
 
@@ -201,6 +211,14 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
         static_assert(PER_STEP * (STAGES - 2) <= 63, "the wait count is a 6-bit field");
         for (int s = 0; s < STAGES - 1; ++s)
             if (s < nk) load_direct(k_begin + s * BK, s);
+        if constexpr (SCALED) {
+            // The rows' sums of squares, asked for behind the first K steps and not used before the last one is
+            // multiplied: what they are made of was written by the kernel before this one, a slow read that the
+            // walk over K covers.  Thread (row, q) takes parts q, q + 256 / BM, ...
+            ss_r = min(m0 + tid % BM, M - 1);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) ss_v[u] = ep.row_ss[(size_t)min(tid / BM + u * (256 / BM), ep.ss_parts - 1) * M + ss_r];
+        }
         // the first step's loads: the earliest of up to STAGES - 1 steps' loads
         __builtin_amdgcn_sched_barrier(0);
         if (nk >= STAGES - 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_STEP * (STAGES - 2)) : "memory");
@@ -217,6 +235,16 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
             else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();
             __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (SCALED) {
+            constexpr int Q = 256 / BM;
+            const int q = tid / BM;
+            float ssum = 0.f;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) ssum += q + u * Q < ep.ss_parts ? ss_v[u] : 0.f;
+            for (int p = q + 8 * Q; p < ep.ss_parts; p += Q) ssum += ep.row_ss[(size_t)p * M + ss_r];  // more than 8 * Q parts: a very wide stream
+            ss_q[q][tid % BM] = ssum;
+            __syncthreads();
         }
 #endif
     } else if constexpr (DIRECT) {
@@ -275,6 +303,17 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
                 if (ROW_GROUPS && m0 + wm * (BM / WM) + i * 16 >= M) continue;
+                float f[4] = {1.f, 1.f, 1.f, 1.f};  // SCALED: of the rows this lane holds
+                if constexpr (SCALED) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int lr = wm * (BM / WM) + i * 16 + grp * 4 + e;
+                        float ssum = 0.f;
+#pragma unroll
+                        for (int qq = 0; qq < 256 / BM; ++qq) ssum += ss_q[qq][lr];
+                        f[e] = 1.0f / sqrtf(ssum / (float)K + ep.ss_eps);
+                    }
+                }
 #pragma unroll
                 for (int j = 0; j < TN; j += 2) {
                     const int col = (col_base + j * 16 - r16) / 2 + r16;  // tiles 2t, 2t+1 -> output tile t
@@ -282,7 +321,12 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
                     for (int e = 0; e < 4; ++e) {
                         const int row = row_base + i * 16 + e;
                         if (CHECKED && !(row < M && col < ep.n_out)) continue;
-                        out[(size_t)row * ep.ldo + col] = from_f32<elem_t>(silu_f(acc[i][j][e]) * acc[i][j + 1][e]);
+                        float gv = acc[i][j][e], uv = acc[i][j + 1][e];
+                        if constexpr (SCALED) {
+                            gv *= f[e];
+                            uv *= f[e];
+                        }
+                        out[(size_t)row * ep.ldo + col] = from_f32<elem_t>(silu_f(gv) * uv);
                     }
                 }
             }
@@ -448,6 +492,36 @@ extern "C" int ms_linear_swiglu(const void* a, const void* w, void* out, int M, 
     const int n = 2 * ceil_div(I, 16) * 16;
     EpiArgs ep{out, nullptr, I, I, 0, 0};
     return launch_gemm<EPI_SWIGLU>((const elem_t*)a, (const elem_t*)w, M, n, K, ep, stream);
+}
+
+// Whether ms_linear_swiglu_scaled takes this shape: bfloat16, one tile of rows, whole K steps of 64.
+extern "C" int ms_swiglu_scaled_takes(int M, int I, int K) {
+#ifdef MS_ELEM_BF16
+    (void)I;
+    return M >= 1 && M <= 64 && K % 64 == 0 && K >= 256;
+#else
+    (void)M; (void)I; (void)K;
+    return 0;
+#endif
+}
+
+// ms_linear_swiglu for rows that came in multiplied by a norm's weight only: both products of a row are
+// divided by the row's root mean square, 1 / sqrt(sum_p row_ss[p, row] / K + eps), before the activation.
+extern "C" int ms_linear_swiglu_scaled(const void* a, const float* row_ss, int ss_parts, float eps, const void* w, void* out, int M, int I,
+                                       int K, hipStream_t stream) {
+#ifdef MS_ELEM_BF16
+    MS_REQUIRE(ms_swiglu_scaled_takes(M, I, K), "gated product with row factors: M=%d K=%d is not taken", M, K);
+    MS_REQUIRE(row_ss && ss_parts >= 1, "gated product with row factors: the rows' sums of squares are missing");
+    MS_REQUIRE((reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0, "gemm: operands must be 16-byte aligned");
+    const int n = 2 * ceil_div(I, 16) * 16;
+    EpiArgs ep{out, nullptr, I, I, K, 0, row_ss, ss_parts, eps};
+    hipLaunchKernelGGL((gemm_kernel<64, 64, 2, 2, 64, EPI_SWIGLU, 4, true>), dim3((unsigned)ceil_div(n, 64), 1), dim3(256), 0, stream,
+                       (const elem_t*)a, (const elem_t*)w, M, n, K, ep);
+    return check_launch("gemm 64x64x64 deep, row factors");
+#else
+    (void)a; (void)row_ss; (void)ss_parts; (void)eps; (void)w; (void)out; (void)M; (void)I; (void)K; (void)stream;
+    MS_REQUIRE(false, "gated product with row factors: built for bfloat16 only");
+#endif
 }
 
 // Number of partial sums ms_linear_split_tiled writes for this problem (1 = the complete product).

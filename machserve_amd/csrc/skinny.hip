@@ -19,7 +19,7 @@ namespace ms {
 constexpr int KSTEP = 128;  // K elements per wave iteration: four fragments per lane; fragment c of the wave is the
                             // contiguous chunk c of 32 elements (the four key groups side by side: 64 bytes a row in bf16)
 
-enum SkinnyEpi { SK_STORE_F32 = 0, SK_SWIGLU = 1, SK_RESIDUAL = 2 };
+enum SkinnyEpi { SK_STORE_F32 = 0, SK_SWIGLU = 1, SK_RESIDUAL = 2, SK_RESIDUAL_PRENORM = 3 };
 
 struct SkinnyArgs {
     const elem_t* A;  // [M, K]
@@ -28,6 +28,10 @@ struct SkinnyArgs {
     int M, N, K;
     int k_per_wave;   // multiple of 32
     int n_out;        // SK_SWIGLU: intermediate size
+    // SK_RESIDUAL_PRENORM: beside the sum, what the norm that follows needs from it
+    const float* norm_w;  // [N]
+    elem_t* hn;           // [M, N]: (stream + product) * norm_w, not yet divided by the root mean square
+    float* ss_part;       // [column waves, M]: each column wave's share of the rows' sums of squares
 };
 
 __device__ __forceinline__ float silu_sk(float g) {
@@ -55,7 +59,9 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
         for (int j = 0; j < NT; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     // SK_RESIDUAL: the stream's values are asked for now, with everything else, not after the sums
-    constexpr bool PRIOR_EARLY = EPI == SK_RESIDUAL && MT <= 2;  // with more row tiles the registers are needed elsewhere
+    constexpr bool ADDS = EPI == SK_RESIDUAL || EPI == SK_RESIDUAL_PRENORM;
+    static_assert(EPI != SK_RESIDUAL_PRENORM || MT <= 2, "the form that prepares the norm is for at most 32 rows");
+    constexpr bool PRIOR_EARLY = ADDS && MT <= 2;  // with more row tiles the registers are needed elsewhere
     float prior[PRIOR_EARLY ? MT : 1][NT][4];
     if constexpr (PRIOR_EARLY) {
         const float* xs = reinterpret_cast<const float*>(a.out);
@@ -68,6 +74,12 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
                     const int row = min(i * 16 + grp * 4 + e, a.M - 1), col = min(n0 + j * 16 + r16, a.N - 1);
                     prior[i][j][e] = xs[(size_t)row * a.N + col];
                 }
+    }
+    // SK_RESIDUAL_PRENORM: the norm's weights of this wave's columns, asked for with everything else
+    float nw_early[EPI == SK_RESIDUAL_PRENORM ? NT : 1];
+    if constexpr (EPI == SK_RESIDUAL_PRENORM) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) nw_early[j] = a.norm_w[min(n0 + j * 16 + r16, a.N - 1)];
     }
     if (n0 < a.N) {
         // Every load is unconditional, so that all of a slice's fragments are in flight at once and
@@ -183,6 +195,41 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
                         out[(size_t)row * a.n_out + col] = from_f32<elem_t>(silu_sk(acc[i][j][e]) * acc[i][j + 1][e]);
                 }
             }
+    } else if constexpr (EPI == SK_RESIDUAL_PRENORM) {
+        // The stream takes the sum as in SK_RESIDUAL.  The RMS norm that reads it next is prepared here: the new
+        // values times the norm's weight in the element type, and this wave's columns' share of every row's sum
+        // of squares (a lane's column of each tile, then the sixteen lanes by shuffles); the reader adds the
+        // shares in column order and applies the factor to its finished sums.
+        if (!owner) return;  // the same for a whole wave
+        float* out = reinterpret_cast<float*>(a.out);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            float ss[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                const int col = n0 + j * 16 + r16;
+                const float nw = nw_early[j];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int row = i * 16 + grp * 4 + e;
+                    const bool on = col < a.N && row < a.M;
+                    const float v = prior[i][j][e] + acc[i][j][e];
+                    if (on) {
+                        out[(size_t)row * a.N + col] = v;
+                        a.hn[(size_t)row * a.N + col] = from_f32<elem_t>(v * nw);
+                    }
+                    ss[e] += on ? v * v : 0.f;  // this lane's column of each tile, the tiles in order
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float sq = ss[e];
+#pragma unroll
+                for (int o = 1; o < 16; o <<= 1) sq += __shfl_xor(sq, o, WAVE);
+                const int row = i * 16 + grp * 4 + e;
+                if (r16 == 0 && row < a.M) a.ss_part[(size_t)(blockIdx.x * WN + wn) * a.M + row] = sq;
+            }
+        }
     } else {
         if (owner) {
             // SK_RESIDUAL: all of K lies in this block (gridDim.y == 1), so every element has one writer
@@ -517,4 +564,24 @@ extern "C" int ms_linear_residual_skinny(const void* a, const void* w, float* x,
     MS_REQUIRE(p.ksb == 1, "few-rows product into the stream: K=%d is cut over %d blocks", K, p.ksb);
     SkinnyArgs args{(const elem_t*)a, (const elem_t*)w, x, M, N, K, 0, 0};
     return launch_skinny<SK_RESIDUAL>(args, p, stream);
+}
+
+// Column waves of ms_linear_residual_prenorm_skinny for this shape (the first size of its ss_part), or 0 if the
+// shape is not taken: more than 32 rows, or a K that is cut over several blocks.
+extern "C" int ms_skinny_prenorm_parts(int M, int N, int K) {
+    if (M < 1 || M > 32 || K % 8) return 0;
+    const SkinnyPlan p = plan_skinny(M, N, K, true);
+    return p.ksb == 1 ? ceil_div(N, 32) : 0;
+}
+
+// x[M, N] += a w^T as ms_linear_residual_skinny does, and beside it hn[M, N] = x * norm_w in the element type and
+// ss_part[parts, M], whose sum over parts is the rows' sums of squares of x (parts = ms_skinny_prenorm_parts).
+extern "C" int ms_linear_residual_prenorm_skinny(const void* a, const void* w, float* x, const float* norm_w, void* hn, float* ss_part,
+                                                 int M, int N, int K, hipStream_t stream) {
+    MS_REQUIRE(ms_skinny_prenorm_parts(M, N, K) > 0, "few-rows product that prepares the norm: M=%d N=%d K=%d is not taken", M, N, K);
+    MS_REQUIRE(norm_w && hn && ss_part, "few-rows product that prepares the norm: its outputs are missing");
+    const SkinnyPlan p = plan_skinny(M, N, K, true);
+    SkinnyArgs args{(const elem_t*)a, (const elem_t*)w, x, M, N, K, 0, 0, norm_w, (elem_t*)hn, ss_part};
+    if (M <= 16) return launch_skinny_mt<1, 2, SK_RESIDUAL_PRENORM>(args, p, stream);
+    return launch_skinny_mt<2, 2, SK_RESIDUAL_PRENORM>(args, p, stream);
 }

@@ -241,6 +241,43 @@ class HipOps:
                                                               self._stream()))
         return None
 
+    def prenorm_swiglu_takes(self, M: int, N: int, K: int, n_gate_up: int) -> bool:
+        """Whether ``x += a @ w.T`` (``w [N, K]``) followed by the gated product of ``rmsnorm(x)`` with an
+        interleaved weight of ``n_gate_up`` rows can run as two kernels without a norm between them: the
+        first leaves ``x * norm_w`` and the rows' sums of squares beside the sum, the second divides its
+        finished sums by the root mean square (:meth:`linear_residual_prenorm`, :meth:`linear_swiglu_scaled`)."""
+        return (not self._tiled(M, N, K) and self._plan("ms_skinny_prenorm_parts", M, N, K) > 0
+                and bool(self._plan("ms_swiglu_scaled_takes", M, n_gate_up // 2, N)))
+
+    def linear_residual_prenorm(self, a: torch.Tensor, w: torch.Tensor, x: torch.Tensor, norm_w: torch.Tensor):
+        """``x += a @ w.T`` in place; returns ``(x * norm_w`` in the element type, float32 ``[parts, M]`` whose sum
+        over parts is the rows' sums of squares of ``x``)``."""
+        M, N, K = self._mm_operands(a, w, "linear_residual_prenorm")
+        self._want(x, torch.float32, "residual stream", M, N)
+        self._want(norm_w, torch.float32, "norm weight", N)
+        parts = self._plan("ms_skinny_prenorm_parts", M, N, K)
+        if parts < 1:
+            raise KernelError(f"linear_residual_prenorm: M={M} N={N} K={K} is not taken")
+        hn = torch.empty((M, N), dtype=self.dtype, device=a.device)
+        ss = torch.empty((parts, M), dtype=torch.float32, device=a.device)
+        self._check(self._core, self._core.ms_linear_residual_prenorm_skinny(
+            _ptr(a), _ptr(w), _ptr(x), _ptr(norm_w), _ptr(hn), _ptr(ss), _c_int(M), _c_int(N), _c_int(K), self._stream()))
+        return hn, ss
+
+    def linear_swiglu_scaled(self, hn: torch.Tensor, row_ss: torch.Tensor, eps: float, w_gate_up: torch.Tensor,
+                             intermediate: int) -> torch.Tensor:
+        """:meth:`linear_swiglu` of rows ``hn`` that lack their norm's division: both products of a row are
+        divided by ``sqrt(sum(row_ss[:, row]) / K + eps)`` before the activation."""
+        M, N, K = self._mm_operands(hn, w_gate_up, "linear_swiglu_scaled")
+        if N != 2 * ((intermediate + 15) // 16) * 16:
+            raise KernelError(f"linear_swiglu_scaled: interleaved weight has {N} rows for intermediate size {intermediate}")
+        self._want(row_ss, torch.float32, "linear_swiglu_scaled sums of squares", row_ss.shape[0], M)
+        out = torch.empty((M, intermediate), dtype=self.dtype, device=hn.device)
+        self._check(self._core, self._core.ms_linear_swiglu_scaled(
+            _ptr(hn), _ptr(row_ss), _c_int(row_ss.shape[0]), _c_float(eps), _ptr(w_gate_up), _ptr(out), _c_int(M),
+            _c_int(intermediate), _c_int(K), self._stream()))
+        return out
+
     def linear_swiglu(self, a: torch.Tensor, w_gate_up: torch.Tensor, intermediate: int) -> torch.Tensor:
         """``silu(a @ gate.T) * (a @ up.T)`` with gate and up rows interleaved in blocks of 16
         (see :func:`interleave_gate_up`)."""

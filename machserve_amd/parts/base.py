@@ -144,6 +144,15 @@ class ResidualStream:
 
     def normed_linear_swiglu(self, weight: torch.Tensor, eps: float, w_gate_up: torch.Tensor, intermediate: int) -> torch.Tensor:
         """``silu(h @ gate.T) * (h @ up.T)`` for ``h = rmsnorm(x)``, the norm folded in where possible."""
+        if self.deferred is not None and self.pending is None:
+            # a product that is still to be added: where the kernels can, it leaves what the norm needs beside its
+            # sum, and the gated product applies the norm's factor to its own finished sums
+            a, w = self.deferred
+            takes = getattr(self.ops, "prenorm_swiglu_takes", None)
+            if takes is not None and takes(a.shape[0], w.shape[0], w.shape[1], w_gate_up.shape[0]):
+                self.deferred = None
+                hn, row_ss = self.ops.linear_residual_prenorm(a, w, self.x, weight)
+                return self.ops.linear_swiglu_scaled(hn, row_ss, eps, w_gate_up, intermediate)
         self._launch_deferred()
         T, K = self.x.shape
         P = 0 if self.pending is None else self.pending.shape[0]

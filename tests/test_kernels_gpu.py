@@ -171,6 +171,36 @@ def test_products_with_the_norm_folded_in(dtype, M, N, K, NP):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K,I", [(8, 896, 896, 4864), (1, 896, 896, 4864), (20, 320, 264, 203), (32, 256, 128, 100),
+                                     (5, 1000, 200, 50), (16, 1536, 904, 120)])
+def test_residual_product_prepares_the_norm_for_the_gated_product(dtype, M, N, K, I):
+    """x += a w^T leaves x * norm_w and the rows' sums of squares beside the sum; the gated product of those rows
+    divides its finished sums by the root mean square: together rmsnorm(x + a w^T) through gate and up."""
+    from machserve_amd.kernels import interleave_gate_up
+    ops = ops_for(dtype)
+    if ops._plan("ms_skinny_prenorm_parts", M, N, K) < 1:
+        pytest.skip("K is cut over several blocks for this shape")
+    eps = 1e-5
+    a, w = rnd((M, K), dtype, 51), rnd((N, K), dtype, 52, K ** -0.5)
+    x, nw = rnd((M, N), torch.float32, 53, 2.0), 1 + rnd((N,), torch.float32, 54, 0.1)
+    x_new = x.double() + P.linear(a.double(), w.double())
+    xd = x.to(DEV).clone()
+    hn, ss = ops.linear_residual_prenorm(a.to(DEV), w.to(DEV), xd, nw.to(DEV))
+    plain = torch.float32 if dtype == torch.float32 else dtype
+    assert_close(xd, x_new, plain, "stream")
+    assert_close(hn, xd.cpu().double() * nw.double(), dtype, "stream times the norm's weight")
+    assert_close(ss.sum(0), (xd.cpu().double() ** 2).sum(1), torch.float32, "sums of squares")
+    g, u = rnd((I, N), dtype, 55, N ** -0.5 * 3), rnd((I, N), dtype, 56, N ** -0.5)
+    takes = ops.prenorm_swiglu_takes(M, N, K, 2 * ((I + 15) // 16) * 16)
+    assert takes == (dtype == torch.bfloat16 and N % 64 == 0 and N >= 256 and not ops._tiled(M, N, K))
+    if takes:
+        h = P.rms_norm(x_new.float(), nw, eps)
+        ref = P.silu(P.linear(h.double(), g.double())) * P.linear(h.double(), u.double())
+        got = ops.linear_swiglu_scaled(hn, ss, eps, interleave_gate_up(g, u).to(DEV), I)
+        assert_close(got, ref, dtype, "gated product of the normed stream")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,I,K", [(1, 16, 8), (9, 160, 64), (70, 328, 192), (200, 4864, 896), (64, 4864, 896), (33, 264, 136),
                                    (64, 328, 256), (50, 1000, 576)])
 def test_linear_swiglu(dtype, M, I, K):
