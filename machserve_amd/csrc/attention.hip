@@ -652,12 +652,23 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
                 col[u] = c < g * hd ? qcol + c : (c < (g + 1) * hd ? kcol + c - g * hd : vcol + c - (g + 1) * hd);
                 v[u] = bias[col[u]] * bias_on;
             }
-            for (int p = 0; p < a.n_partials; ++p) {
-                float t[4];
+            // eight partial sums at a time, all of their loads asked for before the first is added: the sums
+            // were written by the kernel before this one, and one load after the other would be as many
+            // trips to them (beyond the last partial sum: the last one again, not added)
+            for (int p0 = 0; p0 < a.n_partials; p0 += 8) {
+                float t[8][4];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) t[u] = row0[p * pstride + col[u]];
+                for (int q = 0; q < 8; ++q) {
+                    const size_t po = (size_t)min(p0 + q, a.n_partials - 1) * pstride;
 #pragma unroll
-                for (int u = 0; u < 4; ++u) v[u] += t[u];
+                    for (int u = 0; u < 4; ++u) t[q][u] = row0[po + col[u]];
+                }
+#pragma unroll
+                for (int q = 0; q < 8; ++q)
+                    if (p0 + q < a.n_partials) {
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) v[u] += t[q][u];
+                    }
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u)
