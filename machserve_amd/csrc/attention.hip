@@ -19,6 +19,8 @@
 //
 // Compiled once per MS_ATTN_ND (tile head size / 16); a smaller head size runs in the next
 // larger tile with the unused columns zero.
+#include <type_traits>
+
 #include "common.cuh"
 
 #ifndef MS_ATTN_ND
@@ -652,24 +654,30 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
                 col[u] = c < g * hd ? qcol + c : (c < (g + 1) * hd ? kcol + c - g * hd : vcol + c - (g + 1) * hd);
                 v[u] = bias[col[u]] * bias_on;
             }
-            // eight partial sums at a time, all of their loads asked for before the first is added: the sums
-            // were written by the kernel before this one, and one load after the other would be as many
-            // trips to them (beyond the last partial sum: the last one again, not added)
-            for (int p0 = 0; p0 < a.n_partials; p0 += 8) {
-                float t[8][4];
+            // Several partial sums at a time, all of their loads asked for before the first is added: the sums
+            // were written by the kernel before this one, and one load after the other would be as many trips
+            // to them (beyond the last partial sum: the last one again, not added).  Two at a time when there
+            // are no more (a few-rows projection), eight otherwise (a projection cut along K).
+            auto add_partials = [&](auto batch) {
+                constexpr int NB = decltype(batch)::value;
+                for (int p0 = 0; p0 < a.n_partials; p0 += NB) {
+                    float t[NB][4];
 #pragma unroll
-                for (int q = 0; q < 8; ++q) {
-                    const size_t po = (size_t)min(p0 + q, a.n_partials - 1) * pstride;
+                    for (int q = 0; q < NB; ++q) {
+                        const size_t po = (size_t)min(p0 + q, a.n_partials - 1) * pstride;
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) t[q][u] = row0[po + col[u]];
-                }
-#pragma unroll
-                for (int q = 0; q < 8; ++q)
-                    if (p0 + q < a.n_partials) {
-#pragma unroll
-                        for (int u = 0; u < 4; ++u) v[u] += t[q][u];
+                        for (int u = 0; u < 4; ++u) t[q][u] = row0[po + col[u]];
                     }
-            }
+#pragma unroll
+                    for (int q = 0; q < NB; ++q)
+                        if (p0 + q < a.n_partials) {
+#pragma unroll
+                            for (int u = 0; u < 4; ++u) v[u] += t[q][u];
+                        }
+                }
+            };
+            if (a.n_partials <= 2) add_partials(std::integral_constant<int, 2>{});
+            else add_partials(std::integral_constant<int, 8>{});
 #pragma unroll
             for (int u = 0; u < 4; ++u)
                 if (c0 + u * 256 < width) rowv[c0 + u * 256] = v[u];
