@@ -4,7 +4,8 @@ Keys and their meaning follow ``crates/mach-server/src/startup.rs:55-98`` of the
 reference (hidden_size, num_hidden_layers, num_attention_heads, num_key_value_heads,
 vocab_size, intermediate_size, max_position_embeddings, rms_norm_eps, rope_theta,
 head_dim, nested ``text_config``).  The reference falls back to Qwen2.5-0.5B's sizes
-when a key is missing; here a missing size is an error, so no size stands in code.
+and constants when a key is missing; here a missing size, ``max_position_embeddings``,
+``rms_norm_eps`` or ``rope_theta`` is an error that names the key, so none of them stands in code.
 Keys the reference ignores but that change the result are read and checked:
 ``tie_word_embeddings``, ``hidden_act``, ``rope_scaling``, and the sliding-window trio
 ``use_sliding_window`` / ``sliding_window`` / ``max_window_layers``.
@@ -31,12 +32,12 @@ def _need_int(d: dict, key: str, minimum: int = 1) -> int:
     return v
 
 
-def _opt_number(d: dict, key: str, default: float) -> float:
+def _need_number(d: dict, key: str) -> float:
     v = d.get(key)
     if v is None:
-        return default
-    if isinstance(v, bool) or not isinstance(v, (int, float)):
-        raise ConfigError(f"config.json: '{key}' must be a number, got {v!r}")
+        raise ConfigError(f"config.json: missing key '{key}'")
+    if isinstance(v, bool) or not isinstance(v, (int, float)) or v <= 0:
+        raise ConfigError(f"config.json: '{key}' must be a positive number, got {v!r}")
     return float(v)
 
 
@@ -86,7 +87,11 @@ class Qwen2Config:
         theta = d.get("rope_theta")
         if theta is None and isinstance(d.get("rope_parameters"), dict):
             theta = d["rope_parameters"].get("rope_theta")
-        theta = 10000.0 if theta is None else float(theta)
+        if theta is None:
+            raise ConfigError("config.json: missing key 'rope_theta' (or 'rope_parameters.rope_theta')")
+        if isinstance(theta, bool) or not isinstance(theta, (int, float)) or theta <= 0:
+            raise ConfigError(f"config.json: 'rope_theta' must be a positive number, got {theta!r}")
+        theta = float(theta)
         use_win = bool(d.get("use_sliding_window", False))
         window = d.get("sliding_window")
         max_win_layers = d.get("max_window_layers")
@@ -100,9 +105,8 @@ class Qwen2Config:
             hidden_size=hidden, num_hidden_layers=layers, num_attention_heads=heads, num_key_value_heads=kv,
             head_dim=head_dim, intermediate_size=_need_int(d, "intermediate_size"),
             vocab_size=_need_int(d, "vocab_size"),
-            max_position_embeddings=_need_int(d, "max_position_embeddings") if d.get("max_position_embeddings")
-            is not None else 2048,
-            rms_norm_eps=_opt_number(d, "rms_norm_eps", 1e-6), rope_theta=theta,
+            max_position_embeddings=_need_int(d, "max_position_embeddings"),
+            rms_norm_eps=_need_number(d, "rms_norm_eps"), rope_theta=theta,
             tie_word_embeddings=None if tie is None else bool(tie),
             use_sliding_window=use_win, sliding_window=window if use_win else None,
             max_window_layers=int(max_win_layers) if max_win_layers is not None else layers,

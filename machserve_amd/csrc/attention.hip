@@ -1022,7 +1022,7 @@ extern "C" int MS_CAT(ms_decode_attention_nd, MS_ATTN_ND)(
     MS_REQUIRE(hd % 16 == 0 && hd > 0 && hd <= HDT, "decode attention: head size %d does not fit this tile of %d", hd, HDT);
     MS_REQUIRE(KV > 0 && H % KV == 0 && H / KV <= 16, "decode attention: %d heads over %d key/value heads (at most 16 each)", H, KV);
     MS_REQUIRE(ps % 16 == 0 && ps > 0, "decode attention: page size %d must be a multiple of 16", ps);
-    MS_REQUIRE(nsplit >= 1 && nsplit <= 65535 && (nsplit == 1 || (part_o && part_ml)), "decode attention: %d splits", nsplit);
+    MS_REQUIRE(nsplit >= 1 && nsplit <= MAX_SPLITS && (nsplit == 1 || (part_o && part_ml)), "decode attention: %d splits (at most %d)", nsplit, MAX_SPLITS);
     DecodeArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, (elem_t*)out, part_o, part_ml, block_table,
                  seq_pos0, table_stride, H, KV, hd, ps, window, nsplit, scale, nullptr, nullptr, nullptr, nullptr, 0, 0};
     hipLaunchKernelGGL(decode_attention_kernel<false>, dim3((unsigned)S, (unsigned)KV, (unsigned)nsplit), dim3(256), 0, stream, a);

@@ -358,7 +358,11 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
     else emit(std::true_type{}, std::false_type{});
 }
 
-static int g_gemm_config = 0;  // 0: chosen by shape; else a fixed tile (measurements only)
+#ifdef MS_MEASURE  // switches for measurements, in no library that serves
+static int g_gemm_config = 0;  // 0: chosen by shape; else a fixed tile
+#else
+static constexpr int g_gemm_config = 0;
+#endif
 
 template <int EPI>
 static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, EpiArgs ep, hipStream_t stream,
@@ -423,7 +427,11 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
 
 // K slices for a product whose consumer adds partial sums: enough 128x128 blocks to fill the chip,
 // at least 512 of K each.  The 32-bit build never slices: its sums keep one order.
-static int g_force_splits = 0;  // measurements only
+#ifdef MS_MEASURE
+static int g_force_splits = 0;
+#else
+static constexpr int g_force_splits = 0;
+#endif
 
 static int plan_tiled_splits(int M, int N, int K) {
 #ifdef MS_ELEM_BF16
@@ -567,5 +575,7 @@ extern "C" int ms_linear_split_tiled(const void* a, const void* w, float* out, i
 }
 
 // Measurements only: force one tile configuration (0 = choose by shape).
+#ifdef MS_MEASURE
 extern "C" void ms_gemm_force_config(int c) { g_gemm_config = c; }
 extern "C" void ms_gemm_force_splits(int n) { g_force_splits = n; }
+#endif

@@ -51,11 +51,17 @@ public:
             throw SchedulerError(cat("prompt of ", prompt_len, " tokens leaves no room within ", max_positions_, " positions"));
         int total = prompt_len + max_new - 1;  // the last generated token is never fed
         if (max_positions_ > 0) total = std::min(total, max_positions_);
-        const int ps = cache_.page_size(), pages = (total + ps - 1) / ps;
-        for (int g = 0; g < cache_.num_groups(); ++g)
+        const int ps = cache_.page_size();
+        for (int g = 0; g < cache_.num_groups(); ++g) {
+            // a window group holds the pages that the keys [L - window + 1, L + n) of a step touch, n being a
+            // portion at most; a group of all keys holds every page of the request
+            int pages = (total + ps - 1) / ps;
+            const int window = cache_.group_window(g);
+            if (window > 0) pages = std::min(pages, (window + std::min(chunk_, budget_) - 1 + ps - 1) / ps + 1);
             if (pages > cache_.group_pages(g))
-                throw SchedulerError(cat("request of up to ", total, " cached tokens needs ", pages, " pages; group ",
+                throw SchedulerError(cat("request of up to ", total, " cached tokens needs ", pages, " pages at a time; group ",
                                          cache_.group_name(g), " has ", cache_.group_pages(g)));
+        }
         if (reqs_.count(id)) throw SchedulerError(cat("request ", id, " exists already"));
         reqs_[id] = Req{id, prompt_len, prompt_len, 0, -1};
         waiting_.push_back(id);
@@ -75,14 +81,20 @@ public:
         while (true) {
             plan.items.clear();
             int budget = budget_;
-            // 1. decoded tokens, oldest request first; they must all fit, or the youngest goes
+            // 1. decoded tokens, oldest request first; they must all fit, or the youngest goes.  There are never
+            //    more decoding requests than the budget holds: a request starts (and a prompt ends) only in a step
+            //    that had budget left for it beside every decoding request, so the sum never grows beyond it.
             std::vector<int> need(G, 0);
+            int decoders = 0;
             for (long id : running_) {
                 const Req& r = reqs_.at(id);
                 if (!r.decoding()) continue;
+                ++decoders;
                 auto n = cache_.pages_needed(r.slot, 1);
                 for (int g = 0; g < G; ++g) need[g] += n[g];
             }
+            if (decoders > budget)
+                throw SchedulerError(cat(decoders, " requests decode under a budget of ", budget, " tokens a step"));
             bool short_of = false;
             for (int g = 0; g < G; ++g) short_of |= cache_.group_available(g) < need[g];
             if (short_of) {
@@ -92,7 +104,6 @@ public:
             for (long id : running_) {
                 const Req& r = reqs_.at(id);
                 if (!r.decoding()) continue;
-                if (budget == 0) break;
                 plan.items.push_back({id, r.fed, 1, true});
                 --budget;
             }

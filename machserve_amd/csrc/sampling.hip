@@ -232,13 +232,17 @@ __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs a) {
     if (tid == 0) {
         int found = s_found;
         if (found < 0) {
-            // rounding at the top of the mass: the last allowed token, as a walk that never
-            // exceeds the target ends there
-            for (int i = V - 1; i >= 0 && found < 0; --i) {
+            // rounding at the top of the mass: no segment's walk went past the target.  As the reference
+            // (crates/mach-model/src/sampling.rs:385-400): the first allowed token, else the row's maximum
+            for (int i = 0; i < V && found < 0; ++i) {
                 const float pr = expf((row[i] - maxv) * inv_t);
                 if (allowed(row[i], pr)) found = i;
             }
-            if (found < 0) found = 0;
+            if (found < 0) {
+                found = 0;
+                for (int i = 1; i < V; ++i)
+                    if (row[i] > row[found]) found = i;
+            }
         }
         a.out_token[r] = found;
         if (a.also_token) a.also_token[r] = found;

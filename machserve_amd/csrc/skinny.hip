@@ -10,8 +10,10 @@
 // A block is WN x KSI waves: WN groups of output columns, KSI slices of K.  The KSI slices
 // of a block are summed through LDS in slice order; gridDim.y further slices write partial
 // sums out[ks][M][N] that the consumer adds in order (the norm that follows a residual, the
-// rotation that follows the q/k/v projection).  How K is cut depends on N and K only, never
-// on M, so a row's result does not depend on what else is in the batch.
+// rotation that follows the q/k/v projection).  How K is cut depends on N, K and on whether the
+// step has more than 32 rows (then a wave takes 64 columns instead of 32 under a wide output, which
+// changes how many waves share K); within either range a row's sums do not depend on what else is
+// in the batch, and between them they differ in the order of summation only.
 #include "common.cuh"
 
 namespace ms {
@@ -412,8 +414,12 @@ struct SkinnyPlan { int wn, ksi, ksb, k_per_wave; };
 // weigh no more than the weights it streams.
 static int skinny_nt(int M, int N) { return (kBf16 && M > 32 && N >= 4096) ? 4 : 2; }  // 32-bit fragments are twice as large
 
-static int g_force_ksi = 0;  // measurements only: waves along K inside a block (1 = four column waves)
-static int g_max_ksb = 0;    // measurements only: most blocks along K
+#ifdef MS_MEASURE  // switches for measurements, in no library that serves
+static int g_force_ksi = 0;  // waves along K inside a block (1 = four column waves)
+static int g_max_ksb = 0;    // most blocks along K
+#else
+static constexpr int g_force_ksi = 0, g_max_ksb = 0;
+#endif
 
 static SkinnyPlan plan_skinny(int M, int N, int K, bool allow_partials) {
     const int NT = skinny_nt(M, N);
@@ -512,8 +518,10 @@ static int launch_skinny_norm(SkinnyNormArgs a, int n_partials, hipStream_t stre
 
 using namespace ms;
 
+#ifdef MS_MEASURE
 extern "C" void ms_skinny_force_ksi(int ksi) { g_force_ksi = ksi; }
 extern "C" void ms_skinny_max_ksb(int ksb) { g_max_ksb = ksb; }
+#endif
 
 // Number of partial sums ms_linear_skinny writes for M rows of this N and K (1 = the complete product).
 extern "C" int ms_skinny_partials(int M, int N, int K, int allow_partials) { return plan_skinny(M, N, K, allow_partials != 0).ksb; }

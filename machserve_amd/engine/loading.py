@@ -59,6 +59,6 @@ def load_model(model_dir: Optional[str] = None, *, dtype="bfloat16", device: str
     cache = CacheManager(model.cache_requests(), page_size, num_pages, max_requests)
     device_cache = DeviceCache(cache, dt, rt.device)
     model.bind_cache(device_cache)
-    rows_per_block = getattr(ops, "attention_rows_per_block_default", 64)
-    step = StepFunction(model, cache, rt, rows_per_block, use_graphs)
+    # the work lists of a step are cut in the unit that the attention kernels themselves report
+    step = StepFunction(model, cache, rt, model.attention_rows_per_block() or 64, use_graphs)
     return LoadedModel(config, model, cache, device_cache, step, rt)

@@ -69,6 +69,9 @@ class Attention(Mixer):
     def attention_rows_per_token(self):
         return self.spec.heads // self.spec.kv_heads
 
+    def attention_rows_per_block(self):
+        return self.rt.ops.attention_rows_per_block(self.spec.head_dim)
+
     def forward(self, h, stream, ctx):
         s, ops = self.spec, self.rt.ops
         view = ctx.groups[self.group]

@@ -250,6 +250,11 @@ class Mixer(Part):
         """Query heads per KV head if the mixer needs attention work lists, else None."""
         return None
 
+    def attention_rows_per_block(self) -> Optional[int]:
+        """Flat rows (token x head of a group) that one block of the mixer's attention kernel takes: the
+        unit in which the step's work lists are cut.  None if the mixer needs no work lists."""
+        return None
+
     def forward(self, h: torch.Tensor, stream: ResidualStream, ctx: StepContext) -> None:
         """Add the mixer's output for the normalised input ``h`` into the stream
         (``stream.add_linear`` for a final projection, ``stream.add`` for a finished tensor)."""

@@ -105,6 +105,16 @@ class DecoderModel:
     def attention_rows_per_token(self) -> List[int]:
         return sorted({g for g in (b.mixer.attention_rows_per_token() for b in self.blocks) if g})
 
+    def attention_rows_per_block(self) -> Optional[int]:
+        """The unit of the attention work lists, which every mixer's kernel must share (the lists are made
+        once per step); None if no mixer wants them."""
+        units = {(u, type(b.mixer).__name__, getattr(b.mixer.spec, "head_dim", None))
+                 for b in self.blocks for u in [b.mixer.attention_rows_per_block()] if u}
+        if len({u for u, _, _ in units}) > 1:
+            raise ValueError("the mixers' attention kernels take blocks of different numbers of rows: "
+                             + ", ".join(f"{name} (head size {hd}): {u}" for u, name, hd in sorted(units)))
+        return next(iter(units))[0] if units else None
+
     @property
     def vocab(self) -> int:
         return self.spec.head.vocab

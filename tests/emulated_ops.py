@@ -15,7 +15,6 @@ MASK64 = (1 << 64) - 1
 
 
 class EmulatedOps:
-    attention_rows_per_block_default = 64
 
     def __init__(self, dtype=torch.float32, device="cpu"):
         self.dtype = dtype

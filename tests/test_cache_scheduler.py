@@ -197,6 +197,49 @@ def test_pages_run_out_the_youngest_is_preempted_and_recomputed():
     assert s.finished[b].preemptions >= 1 and s.cache.free_pages() == 4
 
 
+def test_decoders_never_outnumber_the_budget_and_nobody_starves():
+    """A budget of two tokens a step and four requests: a request starts only in a step that has budget left
+    beside every decoding request, so at most two decode at a time, the others wait their turn in the queue,
+    every step is full, nobody is preempted while pages suffice, and all finish."""
+    s = _scheduler(pages=9, page_size=16, max_batch_tokens=2, chunk_size=2, slots=4)
+    ids = [s.add([1, 2], 12) for _ in range(4)]
+    steps = 0
+    while s.has_work():
+        p = s.schedule()
+        assert not p.preempted and 1 <= p.n_tokens <= 2
+        assert sum(r.decoding for r in s.running) <= 2
+        _run_plan(s, p)
+        s.cache.check()
+        steps += 1
+    assert all(len(s.finished[i].generated) == 12 for i in ids)
+    assert steps <= 4 * 13 // 2 + 4   # 52 tokens through a budget of two, a few half-empty steps at the seams
+
+
+def test_a_window_group_is_sized_by_its_window_not_by_the_request():
+    """A long request on a model whose layers all see a window needs pages for window + portion keys
+    only: it is admitted with a pool far smaller than its length, and runs to the end."""
+    from machserve_amd.cache import CacheManager
+    from machserve_amd.engine import Scheduler, SchedulerError
+    from machserve_amd.parts import PagedKVRequest
+    m = CacheManager([PagedKVRequest(2, 16, 40)], 16, 6, 2)      # window 40, 6 pages of 16
+    s = Scheduler(m, max_batch_tokens=32, chunk_size=32)
+    rid = s.add(list(range(600)), 8)        # 607 cached tokens = 38 pages if all keys were kept
+    while s.has_work():
+        p = s.schedule()
+        assert p.items and not p.preempted
+        _run_plan(s, p)
+        m.check()
+    assert len(s.finished[rid].generated) == 8 and m.free_pages() == 6
+    # with a group of all keys beside it the request is refused, by that group's name
+    m2 = CacheManager([PagedKVRequest(2, 16, 40), PagedKVRequest(2, 16)], 16, 6, 2)
+    with pytest.raises(SchedulerError, match="group full"):
+        Scheduler(m2, max_batch_tokens=32, chunk_size=32).add(list(range(600)), 8)
+    # and a window group too small for window + portion refuses as well
+    m3 = CacheManager([PagedKVRequest(2, 16, 40)], 16, 4, 2)
+    with pytest.raises(SchedulerError, match="window40"):
+        Scheduler(m3, max_batch_tokens=32, chunk_size=32).add(list(range(600)), 8)
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_random_load_always_finishes(seed):
     rng = random.Random(seed)

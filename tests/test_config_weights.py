@@ -24,9 +24,10 @@ def test_qwen2_config_reads_its_keys():
     # nested text_config, num_key_value_heads defaulting to the heads, rope_parameters
     raw = {"architectures": ["Qwen2ForCausalLM"], "text_config": {
         "hidden_size": 32, "num_hidden_layers": 1, "num_attention_heads": 2, "intermediate_size": 64, "vocab_size": 10,
-        "rope_parameters": {"rope_theta": 123.0}}}
+        "max_position_embeddings": 77, "rms_norm_eps": 2e-6, "rope_parameters": {"rope_theta": 123.0}}}
     c = config_from_dict(raw)
     assert c.num_key_value_heads == 2 and c.head_dim == 16 and c.rope_theta == 123.0 and c.tie_word_embeddings is None
+    assert c.max_position_embeddings == 77 and c.rms_norm_eps == 2e-6
 
 
 @pytest.mark.parametrize("change,match", [
@@ -38,6 +39,11 @@ def test_qwen2_config_reads_its_keys():
     ({"use_sliding_window": True}, "sliding_window"),
     ({"architectures": ["LlamaForCausalLM"]}, "not supported"),
     ({"hidden_size": 66}, "head_dim"),
+    # constants that change every logit (or cap every request) are not guessed either
+    ({"max_position_embeddings": None}, "missing key 'max_position_embeddings'"),
+    ({"rms_norm_eps": None}, "missing key 'rms_norm_eps'"),
+    ({"rope_theta": None}, "missing key 'rope_theta'"),
+    ({"rope_theta": -1.0}, "rope_theta"),
 ])
 def test_config_errors_name_the_key(change, match):
     from machserve_amd.config import ConfigError, config_from_dict
@@ -218,6 +224,63 @@ def test_shards_equal_single_file_and_renaming(tmp_path):
     save_file({names[0]: whole[names[0]]}, str(sh / "model-00003.safetensors"))
     with pytest.raises(SafetensorsError, match="appears in"):
         Checkpoint(str(sh))
+
+
+def test_the_folders_index_is_checked_against_its_files(tmp_path):
+    """crates/mach-model/src/loader.rs:327-502: a right index passes; every disagreement between
+    ``model.safetensors.index.json`` and the shards is reported, all in one message."""
+    from safetensors.torch import load_file, save_file
+    from machserve_amd.engine import load_model
+    from machserve_amd.weights import Checkpoint, SafetensorsError
+    d = make_model_dir(tmp_path, "A")
+    whole = load_file(os.path.join(d, "model.safetensors"))
+    names = sorted(whole)
+    sh = tmp_path / "indexed"
+    sh.mkdir()
+    files = ["model-00001-of-00002.safetensors", "model-00002-of-00002.safetensors"]
+    save_file({n: whole[n] for n in names[::2]}, str(sh / files[0]))
+    save_file({n: whole[n] for n in names[1::2]}, str(sh / files[1]))
+    total = sum(t.numel() * t.element_size() for t in whole.values())
+    weight_map = {n: files[i % 2] for i, n in enumerate(names)}
+
+    def write(wm, total_size=total):
+        (sh / "model.safetensors.index.json").write_text(json.dumps({"metadata": {"total_size": total_size}, "weight_map": wm}))
+
+    write(weight_map)
+    ck = Checkpoint(str(sh))
+    assert sorted(ck.names()) == names
+    (sh / "config.json").write_text(open(os.path.join(d, "config.json")).read())
+    load_model(str(sh), dtype="float32", device="cpu", page_size=16, num_pages=2, ops=EmulatedOps())   # and the model loads from it
+    # several disagreements at once: a tensor the index does not list, one listed in the other shard, one that
+    # no shard holds, and a wrong total
+    wm = dict(weight_map)
+    del wm[names[0]]
+    wm[names[1]] = files[0]
+    wm["model.layers.9.ghost.weight"] = files[1]
+    write(wm, total + 4)
+    with pytest.raises(SafetensorsError) as e:
+        Checkpoint(str(sh))
+    msg = str(e.value)
+    assert f"{names[0]!r} of {files[0]} is absent from the index" in msg
+    assert f"{names[1]!r} lies in {files[1]}, the index lists it in {files[0]}" in msg
+    assert "'model.layers.9.ghost.weight' is listed in" in msg and "no shard holds it" in msg
+    assert f"total_size = {total + 4}" in msg and f"describe {total} bytes" in msg
+    # a shard that is missing, a file that is not indexed
+    write({**weight_map, "x": "model-00003-of-00002.safetensors"})
+    with pytest.raises(SafetensorsError, match="named by the index but missing"):
+        Checkpoint(str(sh))
+    write({n: files[0] for n in names[::2]})
+    with pytest.raises(SafetensorsError, match="'model-00002-of-00002.safetensors' is not named by the index"):
+        Checkpoint(str(sh))
+    # a shard named by a path, and a broken index
+    write({**weight_map, "y": "../elsewhere.safetensors"})
+    with pytest.raises(SafetensorsError, match="beside the index"):
+        Checkpoint(str(sh))
+    (sh / "model.safetensors.index.json").write_text("{\"weight_map\": 3}")
+    with pytest.raises(SafetensorsError, match="weight_map"):
+        Checkpoint(str(sh))
+    # a single file is read on its own, whatever index lies beside it
+    assert sorted(Checkpoint(str(sh / files[0])).names()) == names[::2]
 
 
 def test_random_weights_command(tmp_path):

@@ -250,9 +250,19 @@ def test_rope_kv_write(dtype, H, KV, hd, ps, theta):
     assert_close(vd, vp2, dtype, "value pages from partial sums")
 
 
-def _attention_case(dtype, H, KV, hd, ps, window, seqs, seed, peak=False, groups=0, splits=0):
+def _dead_pages_removed(table, seqs, ps, window):
+    """The block table as the cache manager hands it over once pages behind the window have been given
+    back: a logical page that ends at or before ``cached - window + 1`` (no row of the step sees it) is -1."""
+    table = table.clone()
+    for i, (c, n) in enumerate(seqs):
+        table[i, :max(0, c - window + 1) // ps] = -1
+    return table
+
+
+def _attention_case(dtype, H, KV, hd, ps, window, seqs, seed, peak=False, groups=0, splits=0, dead_pages=False):
     """seqs: list of (cached length, rows in this step).  Builds scattered pages holding random
-    keys and values for positions < cached + rows and queries for the step's rows."""
+    keys and values for positions < cached + rows and queries for the step's rows.  With
+    ``dead_pages`` the kernel's block table has -1 where the pages lie wholly behind the window."""
     ops, emu = ops_for(dtype), EmulatedOps(dtype)
     g = H // KV
     gen = torch.Generator().manual_seed(seed)
@@ -286,6 +296,9 @@ def _attention_case(dtype, H, KV, hd, ps, window, seqs, seed, peak=False, groups
     if groups or splits:
         emu = EmulatedOps(torch.float32)  # the reference unrounded: the tolerance allows the output's one rounding
     ref = emu.paged_attention(q, kp, vp, table, *args, H, KV, hd, ps, window, hd ** -0.5)
+    if dead_pages:
+        table = _dead_pages_removed(table, seqs, ps, window)
+        assert (table < 0).sum() > (table.shape[1] - torch.tensor([-(-(c + n) // ps) for c, n in seqs])).sum(), "no page is dead"
     got = ops.paged_attention(q.to(DEV), kp.to(DEV), vp.to(DEV), table.to(DEV), *[a.to(DEV) for a in args], H, KV, hd,
                               ps, window, hd ** -0.5, groups, splits)
     return got, ref
@@ -330,6 +343,17 @@ def test_attention_window(dtype, window):
     seqs = [(0, 150), (200, 1), (63, 3), (0, 1)]
     got, ref = _attention_case(dtype, 6, 2, 32, 16, window, seqs, 200 + window)
     assert_close(got, ref, dtype, f"attention with window {window}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window,splits", [(17, 0), (100, 0), (100, 3), (333, 0)])
+def test_attention_window_with_pages_given_back(dtype, window, splits):
+    """The pages behind the window are gone (-1 in the block table), as the cache manager leaves them:
+    the kernel never looks a dead page up, whichever key tile, group of waves or split would hold it; the far
+    key at the window's edge still counts."""
+    seqs = [(0, 150), (200, 1), (63, 3), (0, 1), (700, 30), (1023, 1)]
+    got, ref = _attention_case(dtype, 6, 2, 32, 16, window, seqs, 500 + window, peak=True, splits=splits, dead_pages=True)
+    assert_close(got, ref, dtype, f"attention with window {window} and dead pages")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -379,6 +403,12 @@ def test_decode_attention(dtype, H, KV, hd, ps, window):
     one = ops.decode_attention(q[S - 1:].to(DEV).contiguous(), kp.to(DEV), vp.to(DEV), table[S - 1:].to(DEV).contiguous(),
                                pos0[S - 1:].to(DEV), H, KV, hd, ps, window, hd ** -0.5)
     assert_close(one, ref[S - 1:], dtype, "decode attention of one request")
+    if window:
+        # the pages behind the window given back, as the cache manager leaves the table
+        dead = _dead_pages_removed(table, [(c, 1) for c in lens], ps, window)
+        assert (dead[S - 1] < 0).sum() > 0
+        got = ops.decode_attention(q.to(DEV), kp.to(DEV), vp.to(DEV), dead.to(DEV), pos0.to(DEV), H, KV, hd, ps, window, hd ** -0.5)
+        assert_close(got, ref, dtype, "decode attention with dead pages")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -460,12 +490,33 @@ def test_attention_long_contexts(dtype, H, KV, hd, ps, window):
     assert_close(got2[n - 1:].float().cpu(), got[1:2].float().cpu(), dtype, "its last row against the decode kernel")
 
 
-def test_attention_equals_library_attention_without_rotation_or_paging():
-    """One request, whole prompt, pages in order: the kernel is plain causal attention."""
-    dtype = torch.float32
-    H, KV, hd, ps, T = 4, 4, 32, 16, 50
-    got, ref = _attention_case(dtype, H, KV, hd, ps, None, [(0, T)], 400)
-    assert_close(got, ref, dtype)
+@pytest.mark.parametrize("H,KV,hd,ps,T", [(4, 4, 32, 16, 50), (6, 2, 64, 32, 131), (3, 1, 48, 16, 70)])
+def test_attention_equals_library_attention_without_rotation_or_paging(H, KV, hd, ps, T):
+    """One request, its whole prompt in one step, pages in order: the kernel is plain causal attention,
+    ``torch.nn.functional.scaled_dot_product_attention`` with the key/value heads repeated for their
+    groups (head h reads key/value head h // g).  Then the last row again through the decode kernel."""
+    import torch.nn.functional as F
+    dtype, g = torch.float32, H // KV
+    ops = ops_for(dtype)
+    q, k, v = rnd((T, H, hd), dtype, 1), rnd((T, KV, hd), dtype, 2), rnd((T, KV, hd), dtype, 3)
+    want = F.scaled_dot_product_attention(q.transpose(0, 1)[None].double(),
+                                          k.transpose(0, 1).repeat_interleave(g, 0)[None].double(),
+                                          v.transpose(0, 1).repeat_interleave(g, 0)[None].double(), is_causal=True)
+    want = want[0].transpose(0, 1).reshape(T, H * hd).float()
+    n_pages = -(-T // ps)
+    kp, vp = torch.zeros(n_pages, KV, ps, hd), torch.zeros(n_pages, KV, hd, ps)
+    for t in range(T):
+        kp[t // ps, :, t % ps, :] = k[t]
+        vp[t // ps, :, :, t % ps] = v[t]
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    table = i32(list(range(n_pages))).view(1, -1)
+    work = i32([(0, r0) for r0 in range(0, T * g, ops.attention_rows_per_block(hd))]).view(-1, 2)
+    got = ops.paged_attention(q.reshape(T, H * hd).to(DEV), kp.to(DEV), vp.to(DEV), table, i32([0]), i32([T]), i32([0]), work,
+                              H, KV, hd, ps, None, hd ** -0.5)
+    assert_close(got, want, dtype, "kernel against library attention")
+    last = ops.decode_attention(q[T - 1:].reshape(1, H * hd).to(DEV), kp.to(DEV), vp.to(DEV), table, i32([T - 1]), H, KV, hd, ps,
+                                None, hd ** -0.5)
+    assert_close(last, want[T - 1:], dtype, "decode kernel against library attention")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -504,6 +555,33 @@ def test_sampler_matches_cpu_mirror():
             assert int(got[i]) == want, f"row {i} rep {rep}"
     want_state = [(int(s) + 3 * P.RNG_GOLDEN) & P.MASK64 for s in seeds]
     assert [int(v) & P.MASK64 for v in state.cpu().tolist()] == want_state
+
+
+def test_sampler_draw_at_the_top_of_the_mass_falls_back_to_the_first_allowed_token():
+    """A draw of u = 1 - 2^-24 (state 4375518: the finalizer's top 24 bits are all ones) on a row whose
+    last segment is 64 tokens of probability 2^-26 behind a mass of one: each of them is lost when added
+    to the running sum, so no walk passes the target, and the rule for that case decides: the first
+    allowed token, then the maximum (crates/mach-model/src/sampling.rs:385-400).  In the second row the
+    first allowed token is not the maximum: the kernel's rule gives token 0 where the reference's CPU
+    mirror, which falls back to the maximum (sampling.rs:1270-1273), would give token 5."""
+    ops = ops_for(torch.float32)
+    assert P.next_uniform(4375518)[0] == 1.0 - 2.0 ** -24
+    V = 1024 * 64
+    tiny = -26.0 * 0.6931471805599453
+    logits = torch.full((2, V), -200.0)
+    logits[:, -64:] = tiny
+    logits[0, 0] = 0.0                    # the maximum is also the first allowed token
+    logits[1, 0], logits[1, 5] = tiny, 0.0
+    state = torch.tensor([4375518, 4375518], dtype=torch.int64, device=DEV)
+    got, _ = ops.sample(logits.to(DEV), torch.ones(2, device=DEV), torch.zeros(2, dtype=torch.int32, device=DEV),
+                        torch.ones(2, device=DEV), state, any_greedy=False)
+    assert got.cpu().tolist() == [0, 0]
+    assert P.sample(logits[0].numpy(), 1.0, 0, 1.0, 4375518)[0] == 0     # the mirror agrees where the two rules do
+    # a draw far from the top of the same rows walks as usual
+    state = torch.tensor([5, 5], dtype=torch.int64, device=DEV)
+    got, _ = ops.sample(logits.to(DEV), torch.ones(2, device=DEV), torch.zeros(2, dtype=torch.int32, device=DEV),
+                        torch.ones(2, device=DEV), state, any_greedy=False)
+    assert got.cpu().tolist() == [0, 5]
 
 
 def test_sampler_greedy_ties_and_spread():

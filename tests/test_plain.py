@@ -138,6 +138,56 @@ def test_whole_sequence_equals_token_by_token(tmp_path, which):
         assert torch.allclose(logits, whole[pos], atol=1e-10), pos
 
 
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_one_token_reduces_the_whole_model_to_library_routines(tmp_path, which):
+    """A sequence of one token at position 0 has no attention to speak of: the softmax over one key is 1,
+    the rotation at position 0 is the identity, so a layer's mixer is ``o_proj(v)`` with each value head
+    repeated for its group.  What is left is the *composition*, written here with library routines only
+    (``F.rms_norm``, ``F.linear``, ``F.silu``): the stream is normalised for each branch's input and never in
+    place, the feed-forward reads the stream after the mixer's output was added, ``input_layernorm`` feeds
+    the mixer and ``post_attention_layernorm`` the feed-forward, and the final norm comes before the head.
+    A post-norm or parallel arrangement, swapped norm weights or a missing final norm fail it."""
+    w, sizes = read_for_plain(make_model_dir(tmp_path, which))
+    w = {k: v.double() for k, v in w.items()}
+    d, g, hd, eps = sizes["hidden"], sizes["heads"] // sizes["kv_heads"], sizes["head_dim"], sizes["eps"]
+    head = w["model.embed_tokens.weight"] if sizes["tied"] else w["lm_head.weight"]
+    for tok in (0, 7, sizes["vocab"] - 1):
+        x = w["model.embed_tokens.weight"][tok]
+        for i in range(sizes["layers"]):
+            p = f"model.layers.{i}."
+            h = F.rms_norm(x, (d,), w[p + "input_layernorm.weight"], eps)
+            v = F.linear(h, w[p + "self_attn.v_proj.weight"], w.get(p + "self_attn.v_proj.bias"))
+            x = x + F.linear(v.view(-1, hd).repeat_interleave(g, dim=0).reshape(-1), w[p + "self_attn.o_proj.weight"])
+            h = F.rms_norm(x, (d,), w[p + "post_attention_layernorm.weight"], eps)
+            x = x + F.linear(F.silu(F.linear(h, w[p + "mlp.gate_proj.weight"])) * F.linear(h, w[p + "mlp.up_proj.weight"]),
+                             w[p + "mlp.down_proj.weight"])
+        want = F.linear(F.rms_norm(x, (d,), w["model.norm.weight"], eps), head)
+        got = P.forward(w, sizes, [tok], torch.float64)[0]
+        assert torch.allclose(got, want, atol=1e-10)
+        wrong = F.linear(x, head)   # the check has teeth: without the final norm the logits are others
+        assert not torch.allclose(got, wrong, atol=1e-3)
+
+
+def test_branches_add_to_a_stream_that_is_never_normalised_in_place(tmp_path):
+    """With every output projection (o_proj, down_proj) zero the branches add nothing, and the logits at every
+    position are ``head(norm(embedding))``: an arrangement that normalises the stream itself (post-norm)
+    does not reduce to this.  And with the embedding scaled up by 10^4 the branches, which read a normalised
+    stream and therefore stay as they were, vanish beside it: the logits tend to the same value."""
+    w, sizes = read_for_plain(make_model_dir(tmp_path, "B"))
+    w = {k: v.double() for k, v in w.items()}
+    toks = random_prompt(11, sizes["vocab"], 8)
+    d, eps = sizes["hidden"], sizes["eps"]
+    bare = F.linear(F.rms_norm(w["model.embed_tokens.weight"][toks], (d,), w["model.norm.weight"], eps), w["lm_head.weight"])
+    off = {k: (torch.zeros_like(v) if k.endswith(("o_proj.weight", "down_proj.weight")) else v) for k, v in w.items()}
+    assert torch.allclose(P.forward(off, sizes, toks, torch.float64), bare, atol=1e-10)
+    full = P.forward(w, sizes, toks, torch.float64)
+    assert not torch.allclose(full, bare, atol=1e-3)
+    big = dict(w)
+    big["model.embed_tokens.weight"] = w["model.embed_tokens.weight"] * 1e4
+    bare_big = F.linear(F.rms_norm(big["model.embed_tokens.weight"][toks], (d,), w["model.norm.weight"], eps), w["lm_head.weight"])
+    assert (P.forward(big, sizes, toks, torch.float64) - bare_big).abs().max() < 1e-3 * bare_big.abs().max()
+
+
 def test_shift_of_all_positions_changes_nothing():
     """Only distances count: the same tokens at positions 100.. give the same logits."""
     import tempfile
