@@ -19,9 +19,11 @@
 //
 // Compiled once per MS_ATTN_ND (tile head size / 16); a smaller head size runs in the next
 // larger tile with the unused columns zero.
+#include <mutex>
 #include <type_traits>
 
 #include "common.cuh"
+#include "no_alloc.h"
 
 #ifndef MS_ATTN_ND
 #error "MS_ATTN_ND: head-size tile in units of 16"
@@ -1031,6 +1033,66 @@ extern "C" int MS_CAT(ms_decode_attention_nd, MS_ATTN_ND)(
     hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)(S * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit);
     return check_launch("decode_merge");
 }
+
+// Scratch memory of ms_decode_attention_noalloc_nd*: the splits' partial outputs, then their (max, sum)
+// pairs.  Each GPU on which the library runs holds its own copy of this array, at its own address, until
+// the process ends.  In host code the name is only a handle for hipGetSymbolAddress; the address that
+// kernels and copies take is looked up once per device and kept in g_scratch_ptr.
+constexpr size_t NOALLOC_SCRATCH_FLOATS = (size_t)1 << 20;  // 4 MiB
+static __device__ __align__(256) float scratch[NOALLOC_SCRATCH_FLOATS];
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static float* g_scratch_ptr[NOALLOC_MAX_DEVICES] = {};
+static std::mutex g_scratch_mutex;
+
+// The device address of `scratch` on the current device (null and an error message if it cannot be had).
+static float* scratch_of_current_device() {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= NOALLOC_MAX_DEVICES) {
+        ms::set_error("decode attention (no allocation): device %d (%s); at most %d devices", dev, hipGetErrorString(e),
+                      NOALLOC_MAX_DEVICES);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> hold(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        float* ptr = nullptr;
+        e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            ms::set_error("decode attention (no allocation): hipGetSymbolAddress on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+
+// ms_decode_attention_nd* for callers that cannot allocate (declared in no_alloc.h): the same kernels, with the
+// workspace of the splits in `scratch` instead of two buffers of the caller.  It calls no hipMalloc, hipFree or
+// allocating library routine.  S * H * nsplit * (hd + 2) floats must fit NOALLOC_SCRATCH_FLOATS.  Nothing in
+// the scratch has to start at zero (every block writes its split's partial result, an empty split a sum
+// of zero); it keeps the last call's contents, and all calls on one GPU share it, so two calls that
+// overlap on one GPU (two streams, two threads) race: the caller orders them.
+extern "C" int MS_CAT(ms_decode_attention_noalloc_nd, MS_ATTN_ND)(
+    const void* q, const void* kpool, const void* vpool, void* out, const int* block_table, int table_stride,
+    const int* seq_pos0, int S, int H, int KV, int hd, int ps, int window, int nsplit, float scale, hipStream_t stream) {
+    MS_REQUIRE(S > 0 && H > 0 && hd > 0 && nsplit >= 1, "decode attention (no allocation): %d rows, %d heads, head size %d, %d splits",
+               S, H, hd, nsplit);
+    float* part_o = nullptr;
+    float* part_ml = nullptr;
+    if (nsplit > 1) {
+        const double need = (double)S * H * nsplit * (hd + 2);
+        MS_REQUIRE(need <= (double)NOALLOC_SCRATCH_FLOATS,
+                   "decode attention (no allocation): %d rows x %d heads x %d splits x (%d + 2) floats = %.0f exceed the scratch of %zu floats",
+                   S, H, nsplit, hd, need, NOALLOC_SCRATCH_FLOATS);
+        float* base = scratch_of_current_device();
+        if (!base) return 1;
+        part_o = base;
+        part_ml = base + (size_t)S * H * nsplit * hd;
+    }
+    return MS_CAT(ms_decode_attention_nd, MS_ATTN_ND)(q, kpool, vpool, out, part_o, part_ml, block_table, table_stride,
+                                                      seq_pos0, S, H, KV, hd, ps, window, nsplit, scale, stream);
+}
+extern "C" long MS_CAT(ms_decode_attention_noalloc_max_floats_nd, MS_ATTN_ND)() { return (long)NOALLOC_SCRATCH_FLOATS; }
 
 // The same from the partial sums of the q/k/v projection: adds them and the bias, rotates q and k
 // by the row's position, writes k and v into the row's page, and attends; a second launch merges

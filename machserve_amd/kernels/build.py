@@ -82,7 +82,8 @@ def _spec(kind: str, elem: str, nd: int | None):
 def _digest(sources, defines) -> str:
     h = hashlib.sha256()
     h.update(" ".join(FLAGS + defines).encode())
-    for f in sorted(set(sources) | {"common.cuh"}):
+    headers = {f for f in os.listdir(CSRC) if f.endswith((".cuh", ".h"))}
+    for f in sorted(set(sources) | headers):
         with open(os.path.join(CSRC, f), "rb") as fh:
             h.update(f.encode())
             h.update(fh.read())
