@@ -15,34 +15,57 @@ class DeviceCache:
 
     def __init__(self, manager: CacheManager, dtype: torch.dtype, device: torch.device):
         self.manager = manager
-        self.kpools: Dict[int, torch.Tensor] = {}
-        self.vpools: Dict[int, torch.Tensor] = {}
-        self.states: Dict[int, Dict[str, torch.Tensor]] = {}
+        # by (layer run, index among its requests); a pool has one page more than its group hands out, and a state
+        # one slot more than there are requests: rows that fill a captured step up write there
+        self._kpools: Dict[tuple, torch.Tensor] = {}
+        self._vpools: Dict[tuple, torch.Tensor] = {}
+        self._states: Dict[tuple, Dict[str, torch.Tensor]] = {}
         ps = manager.page_size
         for name, g in manager.groups.items():
-            n, kv, hd = g.pool.num_pages, g.spec.kv_heads, g.spec.head_dim
-            for layer in g.spec.layers:
-                self.kpools[layer] = torch.zeros((n, kv, ps, hd), dtype=dtype, device=device)
-                self.vpools[layer] = torch.zeros((n, kv, hd, ps), dtype=dtype, device=device)
-        for layer, req in manager.state_requests.items():
-            self.states[layer] = {k: torch.zeros((manager.max_requests, *shape), dtype=req.dtype, device=device)
-                                  for k, shape in req.shapes.items()}
+            n, kv, hd, vhd = g.pool.num_pages + 1, g.spec.kv_heads, g.spec.head_dim, g.spec.v_head_dim
+            for key in g.spec.layers:
+                self._kpools[key] = torch.zeros((n, kv, ps, hd), dtype=dtype, device=device)
+                self._vpools[key] = torch.zeros((n, kv, vhd, ps), dtype=dtype, device=device)
+        for key, req in manager.states.items():
+            self._states[key] = {k: torch.zeros((manager.max_requests + 1, *shape), dtype=req.dtype, device=device)
+                                 for k, shape in req.shapes.items()}
+        # the one-request view
+        self.kpools = {i: t for (i, j), t in self._kpools.items() if not manager.layer_requests[i][0]}
+        self.vpools = {i: t for (i, j), t in self._vpools.items() if not manager.layer_requests[i][0]}
+        self.states = {i: t for (i, j), t in self._states.items() if not manager.layer_requests[i][0]}
         manager.device = self
 
-    def binding(self, layer: int):
+    def _binding_of(self, key):
         m = self.manager
-        if layer in m.state_requests:
-            return StateBinding(self.states[layer])
-        if layer in m.layer_group:
-            src = m.layer_source.get(layer, layer)
-            return KVBinding(m.layer_group[layer], self.kpools[src], self.vpools[src])
+        if key in m.states:
+            return StateBinding(self._states[key])
+        if key in m.paged:
+            return KVBinding(m.paged[key], self._kpools[key], self._vpools[key])
+        if key in m.shared:
+            src = (m.shared[key], 0)
+            return KVBinding(m.paged[src], self._kpools[src], self._vpools[src])
         return None
 
+    def binding(self, layer: int):
+        """What the layer run's mixer asked for: one binding, or a list for a list of requests."""
+        several, reqs = self.manager.layer_requests[layer]
+        out = [self._binding_of((layer, j)) for j in range(len(reqs))]
+        return out if several else out[0]
+
     def zero_state(self, slot: int) -> None:
-        for tensors in self.states.values():
+        for tensors in self._states.values():
             for t in tensors.values():
                 t[slot].zero_()
 
+    def snapshot_states(self):
+        """Copies of every state array (empty for a model without state)."""
+        return {key: {k: t.clone() for k, t in d.items()} for key, d in self._states.items()}
+
+    def restore_states(self, saved) -> None:
+        for key, d in saved.items():
+            for k, t in d.items():
+                self._states[key][k].copy_(t)
+
     def bytes(self) -> int:
-        n = sum(t.numel() * t.element_size() for t in list(self.kpools.values()) + list(self.vpools.values()))
-        return n + sum(t.numel() * t.element_size() for d in self.states.values() for t in d.values())
+        n = sum(t.numel() * t.element_size() for t in list(self._kpools.values()) + list(self._vpools.values()))
+        return n + sum(t.numel() * t.element_size() for d in self._states.values() for t in d.values())

@@ -37,7 +37,8 @@ class GroupSpec:
     window: Optional[int]
     kv_heads: int
     head_dim: int
-    layers: List[int] = field(default_factory=list)
+    v_head_dim: int = 0      # width of a value; the key's width unless the request says otherwise
+    layers: List[Tuple[int, int]] = field(default_factory=list)  # (layer run, index among its requests)
 
 
 @dataclass
@@ -98,32 +99,44 @@ class CacheManager:
         self.max_requests = max_requests
         self.slots = _SlotsView(self.core)
         self.groups: Dict[str, _Group] = {}
-        self.layer_group: Dict[int, str] = {}
-        self.layer_source: Dict[int, int] = {}
-        self.state_requests: Dict[int, StateRequest] = {}
         specs: Dict[str, GroupSpec] = {}
+        # A layer run may ask for several things at once (pages and state, or caches of different widths): every
+        # request is kept under (layer run, index among the run's requests); a run that asked for one thing has index 0.
+        self.layer_requests: Dict[int, list] = {}
+        self.paged: Dict[Tuple[int, int], str] = {}        # -> group
+        self.shared: Dict[Tuple[int, int], int] = {}       # -> source layer run
+        self.states: Dict[Tuple[int, int], StateRequest] = {}
         for i, req in enumerate(layer_requests):
-            if isinstance(req, PagedKVRequest):
-                name = group_name(req.window)
-                if name not in specs:
-                    specs[name] = GroupSpec(name, req.window, req.kv_heads, req.head_dim)
-                g = specs[name]
-                if (g.kv_heads, g.head_dim) != (req.kv_heads, req.head_dim):
-                    # same need, other geometry: a group of its own
-                    name = f"{name}/kv{req.kv_heads}x{req.head_dim}"
-                    g = specs.setdefault(name, GroupSpec(name, req.window, req.kv_heads, req.head_dim))
-                g.layers.append(i)
-                self.layer_group[i] = name
-            elif isinstance(req, SharedKVRequest):
-                self.layer_source[i] = req.source_layer
-            elif isinstance(req, StateRequest):
-                self.state_requests[i] = req
-            elif req is not None:
-                raise CacheError(f"layer {i}: unknown cache request {req!r}")
-        for i, src in self.layer_source.items():
-            if src not in self.layer_group:
-                raise CacheError(f"layer {i} reads the cache of layer {src}, which keeps none")
-            self.layer_group[i] = self.layer_group[src]
+            several = isinstance(req, (list, tuple))
+            reqs = list(req) if several else [req]
+            self.layer_requests[i] = (several, reqs)
+            for j, r in enumerate(reqs):
+                if isinstance(r, PagedKVRequest):
+                    v_hd = r.v_head_dim or r.head_dim
+                    name = group_name(r.window)
+                    g = specs.get(name)
+                    if g is not None and (g.kv_heads, g.head_dim, g.v_head_dim) != (r.kv_heads, r.head_dim, v_hd):
+                        # same need, other geometry: a group of its own
+                        name = f"{name}/kv{r.kv_heads}x{r.head_dim}" + (f"v{v_hd}" if v_hd != r.head_dim else "")
+                        g = specs.get(name)
+                    if g is None:
+                        g = specs[name] = GroupSpec(name, r.window, r.kv_heads, r.head_dim, v_hd)
+                    g.layers.append((i, j))
+                    self.paged[(i, j)] = name
+                elif isinstance(r, SharedKVRequest):
+                    self.shared[(i, j)] = r.source_layer
+                elif isinstance(r, StateRequest):
+                    self.states[(i, j)] = r
+                elif r is not None:
+                    raise CacheError(f"layer {i}: unknown cache request {r!r}")
+        for (i, j), src in self.shared.items():
+            if (src, 0) not in self.paged or self.layer_requests[src][0]:
+                raise CacheError(f"layer {i} reads the cache of layer {src}, which keeps no single paged cache")
+        # the one-request view, as most layers have it
+        self.layer_group = {i: g for (i, j), g in self.paged.items() if not self.layer_requests[i][0]}
+        self.layer_source = {i: src for (i, j), src in self.shared.items() if not self.layer_requests[i][0]}
+        self.layer_group.update({i: self.paged[(src, 0)] for i, src in self.layer_source.items()})
+        self.state_requests = {i: r for (i, j), r in self.states.items() if not self.layer_requests[i][0]}
         for name, spec in specs.items():
             index = self.core.add_group(name, spec.window or 0, num_pages)
             self.groups[name] = _Group(spec, self.core, index)
@@ -193,7 +206,14 @@ class CacheManager:
         is owned.  Raises CacheError otherwise."""
         self.core.check()
 
-    def build_step(self, slots, counts, tokens, want_rows, heads_per_kv, rows_per_block: int, table_multiple: int = 1):
+    def build_step(self, slots, counts, tokens, want_rows, heads_per_kv, rows_per_block: int, table_multiple: int = 1,
+                   pad_rows: int = 0, axes: int = 1, explicit_positions=()):
         """The step's int32 buffer as ``(numpy array, {section: (start, size)}, {group: table width})``;
-        see ``CacheCore::build_step`` for the sections."""
-        return self.core.build_step(slots, counts, tokens, want_rows, list(heads_per_kv), rows_per_block, table_multiple)
+        see ``CacheCore::build_step`` for the sections, the rows that fill a step up and the positions."""
+        return self.core.build_step(slots, counts, tokens, want_rows, list(heads_per_kv), rows_per_block, table_multiple,
+                                    pad_rows, axes, list(explicit_positions))
+
+    @property
+    def scratch_slot(self) -> int:
+        """The state slot of rows that belong to no request (one beyond the requests' slots)."""
+        return self.core.scratch_slot()

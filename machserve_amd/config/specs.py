@@ -78,9 +78,12 @@ class LayerSpec:
 
 @dataclass(frozen=True)
 class EmbeddingSpec:
+    """Token embedding: rows of a table, times ``scale``."""
     vocab: int
     width: int
     tensors: Mapping[str, str] = field(default_factory=dict)
+    kind: str = "embedding"
+    scale: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -91,6 +94,8 @@ class HeadSpec:
     width: int
     tied: Optional[bool]
     tensors: Mapping[str, str] = field(default_factory=dict)
+    kind: str = "linear"
+    scale: float = 1.0  # the logits are multiplied by it
 
 
 @dataclass(frozen=True)

@@ -8,13 +8,13 @@
 
 namespace ms {
 
-// x[t, :] = float(table[tokens[t], :])
+// x[t, :] = float(table[tokens[t], :]) * scale
 __global__ __launch_bounds__(256) void embed_kernel(const int* __restrict__ tokens, const elem_t* __restrict__ table,
-                                                    float* __restrict__ x, int d) {
+                                                    float* __restrict__ x, int d, float scale) {
     const int t = blockIdx.x;
     const elem_t* src = table + (size_t)tokens[t] * d;
     float* dst = x + (size_t)t * d;
-    for (int c = threadIdx.x; c < d; c += 256) dst[c] = to_f32(src[c]);
+    for (int c = threadIdx.x; c < d; c += 256) dst[c] = to_f32(src[c]) * scale;
 }
 
 // r = rows ? rows[i] : i;  v = x[r, :] + sum_p partials[p, r, :] (in order);  if partials are given
@@ -266,9 +266,9 @@ __global__ __launch_bounds__(256) void rope_kv_write_quads_kernel(RopeArgs a) {
 
 using namespace ms;
 
-extern "C" int ms_embed(const int* tokens, const void* table, float* x, int T, int d, hipStream_t stream) {
+extern "C" int ms_embed(const int* tokens, const void* table, float* x, int T, int d, float scale, hipStream_t stream) {
     MS_REQUIRE(T > 0 && d > 0, "embed: empty problem T=%d d=%d", T, d);
-    hipLaunchKernelGGL(embed_kernel, dim3(T), dim3(256), 0, stream, tokens, (const elem_t*)table, x, d);
+    hipLaunchKernelGGL(embed_kernel, dim3(T), dim3(256), 0, stream, tokens, (const elem_t*)table, x, d, scale);
     return check_launch("embed");
 }
 

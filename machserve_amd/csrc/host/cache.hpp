@@ -129,6 +129,11 @@ public:
     int group_pages(int g) const { return groups_.at(g).pool.num_pages(); }
     int group_available(int g) const { return groups_.at(g).pool.available(); }
     std::vector<int> group_live_pages(int g) const { return groups_.at(g).pool.live_pages(); }
+    // A page beyond every pool (id = the pool's size) and a slot beyond the request slots (id = max_requests): never
+    // handed out.  Rows that only fill a captured step up to its size write there, so that they change nothing a
+    // request owns: neither a key nor a state.  The device arrays are one page and one slot larger for them.
+    int scratch_page(int g) const { return groups_.at(g).pool.num_pages(); }
+    int scratch_slot() const { return slots_.num_slots(); }
     int slots_available() const { return slots_.available(); }
     bool slot_is_live(int s) const { return slots_.is_live(s); }
 
@@ -242,26 +247,41 @@ public:
     // flattened.  Sections, each starting on a 16-byte boundary, in this order: tokens, positions,
     // seq_q_start, seq_q_len, seq_pos0, seq_slot, want_rows, then per group "table/<name>" [S, width]
     // and "slot_map/<name>" [T], then per entry of heads_per_kv "work/<g>" [n, 2].  `table_multiple`
-    // rounds the widths of the block tables up (captured graphs want few distinct widths).
-    py::tuple build_step(const std::vector<int>& slots, const std::vector<int>& counts, const std::vector<int>& tokens,
+    // rounds the widths of the block tables up (captured graphs want few distinct widths).  `pad_rows` appends that
+    // many requests of one row each that belong to nobody: token 0 at position 0 of the scratch slot, whose one page
+    // is the scratch page; their rows run like any other and leave no trace in what requests own.  "positions" is
+    // [T, axes]: on every axis a row's index in its request's cache, unless `explicit_positions` ([T, axes]
+    // flattened, rows of the entries only) gives the caller's own (where a row sits in the cache never follows them).
+    py::tuple build_step(const std::vector<int>& slots_in, const std::vector<int>& counts_in, const std::vector<int>& tokens_in,
                          const std::vector<int>& want_rows, const std::vector<int>& heads_per_kv, int rows_per_block,
-                         int table_multiple) const {
-        const int S = (int)slots.size();
-        if (S == 0 || counts.size() != slots.size()) throw CacheError("a step needs at least one entry");
+                         int table_multiple, int pad_rows, int axes, const std::vector<int>& explicit_positions) const {
+        const int S_real = (int)slots_in.size();
+        if (S_real == 0 || counts_in.size() != slots_in.size()) throw CacheError("a step needs at least one entry");
+        if (pad_rows < 0) throw CacheError("pad_rows must not be negative");
+        std::vector<int> slots(slots_in), counts(counts_in), tokens(tokens_in);
+        slots.insert(slots.end(), pad_rows, scratch_slot());
+        counts.insert(counts.end(), pad_rows, 1);
+        tokens.insert(tokens.end(), pad_rows, 0);
+        const int S = S_real + pad_rows;
         std::vector<int> q_start(S), pos0(S);
         int T = 0;
         for (int i = 0; i < S; ++i) {
             q_start[i] = T;
-            pos0[i] = length(slots[i]);
+            pos0[i] = i < S_real ? length(slots[i]) : 0;
             if (counts[i] < 1) throw CacheError(cat("slot ", slots[i], ": an entry needs at least one token"));
             T += counts[i];
         }
-        if ((int)tokens.size() != T) throw CacheError(cat("the step has ", T, " rows but ", tokens.size(), " tokens"));
+        if ((int)tokens.size() != T) throw CacheError(cat("the step has ", T - pad_rows, " rows but ", tokens_in.size(), " tokens"));
         std::vector<std::pair<std::string, std::vector<int32_t>>> sections;
         auto add = [&](const std::string& name, std::vector<int32_t> v) { sections.emplace_back(name, std::move(v)); };
-        std::vector<int32_t> positions(T);
+        if (axes < 1) throw CacheError(cat("positions have ", axes, " axes"));
+        if (!explicit_positions.empty() && explicit_positions.size() != (size_t)(T - pad_rows) * axes)
+            throw CacheError(cat("positions given for ", explicit_positions.size(), " numbers, the step has ", T - pad_rows, " rows of ", axes));
+        std::vector<int32_t> positions((size_t)T * axes);
         for (int i = 0; i < S; ++i)
-            for (int j = 0; j < counts[i]; ++j) positions[q_start[i] + j] = pos0[i] + j;
+            for (int j = 0; j < counts[i]; ++j)
+                for (int a = 0; a < axes; ++a) positions[(size_t)(q_start[i] + j) * axes + a] = pos0[i] + j;
+        std::copy(explicit_positions.begin(), explicit_positions.end(), positions.begin());
         add("tokens", std::vector<int32_t>(tokens.begin(), tokens.end()));
         add("positions", positions);
         add("seq_q_start", std::vector<int32_t>(q_start.begin(), q_start.end()));
@@ -270,12 +290,17 @@ public:
         add("seq_slot", std::vector<int32_t>(slots.begin(), slots.end()));
         add("want_rows", std::vector<int32_t>(want_rows.begin(), want_rows.end()));
         py::dict widths;
-        for (auto& g : groups_) {
+        for (size_t gi = 0; gi < groups_.size(); ++gi) {
+            const Group& g = groups_[gi];
             int width = 1;
-            for (int s : slots) width = std::max(width, (int)g.tables.at(s).size());
+            for (int i = 0; i < S_real; ++i) width = std::max(width, (int)g.tables.at(slots[i]).size());
             if (table_multiple > 1) width = (width + table_multiple - 1) / table_multiple * table_multiple;
             std::vector<int32_t> table((size_t)S * width, -1), slot_map(T);
-            for (int i = 0; i < S; ++i) {
+            for (int i = S_real; i < S; ++i) {
+                table[(size_t)i * width] = scratch_page((int)gi);
+                slot_map[q_start[i]] = scratch_page((int)gi) * page_size_;
+            }
+            for (int i = 0; i < S_real; ++i) {
                 const auto& t = g.tables.at(slots[i]);
                 std::copy(t.begin(), t.end(), table.begin() + (size_t)i * width);
                 for (int j = 0; j < counts[i]; ++j) {

@@ -42,6 +42,8 @@ PYBIND11_MODULE(ms_host, m) {
         .def("group_pages", &CacheCore::group_pages)
         .def("group_available", &CacheCore::group_available)
         .def("group_live_pages", &CacheCore::group_live_pages)
+        .def("scratch_page", &CacheCore::scratch_page)
+        .def("scratch_slot", &CacheCore::scratch_slot)
         .def("slots_available", &CacheCore::slots_available)
         .def("slot_is_live", &CacheCore::slot_is_live)
         .def("admit", &CacheCore::admit)
@@ -56,7 +58,9 @@ PYBIND11_MODULE(ms_host, m) {
         .def("slot_of_position", &CacheCore::slot_of_position)
         .def("live_requests", &CacheCore::live_requests)
         .def("check", &CacheCore::check)
-        .def("build_step", &CacheCore::build_step);
+        .def("build_step", &CacheCore::build_step, py::arg("slots"), py::arg("counts"), py::arg("tokens"), py::arg("want_rows"),
+             py::arg("heads_per_kv"), py::arg("rows_per_block"), py::arg("table_multiple") = 1, py::arg("pad_rows") = 0, py::arg("axes") = 1,
+             py::arg("explicit_positions") = std::vector<int>());
 
     py::register_exception<SchedulerError>(m, "SchedulerError", PyExc_ValueError);
     py::class_<PlanItem>(m, "PlanItem")

@@ -32,6 +32,9 @@ class StepEntry:
     slot: int                 # the request's state slot (from CacheManager.admit)
     tokens: Sequence[int]     # its next tokens, in order
     want: Sequence[int] = ()  # indices into ``tokens`` whose logits are wanted
+    # what the position encodings see for each token, one number per axis of the model's positions; None: on every
+    # axis the token's index in the request (where a token lies in the cache never depends on this)
+    positions: Optional[Sequence[Sequence[int]]] = None
 
 
 class _DecodeGraph:
@@ -73,6 +76,7 @@ class StepFunction:
         self.model, self.cache, self.rt = model, cache, rt
         self.rows_per_block = attention_rows_per_block
         self.heads_per_kv = model.attention_rows_per_token()
+        self.position_axes = model.position_axes() if hasattr(model, "position_axes") else 1
         # A step of few tokens is bound by its launches: it is captured into a HIP graph and replayed.
         # A decode step (one token a request), and any other step of few rows, when its shape
         # (tokens per request, wanted rows, table widths) keeps coming, as it does while the same
@@ -88,14 +92,26 @@ class StepFunction:
 
     # ------------------------------------------------------------------ context
     def _check_entries(self, entries: Sequence[StepEntry]):
-        """Validates the entries; returns their slots, token counts, flattened tokens and wanted rows."""
+        """Validates the entries; returns their slots, token counts, flattened tokens and wanted rows.
+        ``self._explicit`` is left as the entries' own positions, flattened ``[rows * axes]``, or empty if none has any."""
         if not entries:
             raise StepError("a step needs at least one entry")
         cache, vocab, limit = self.cache, self.model.vocab, self.model.spec.max_positions
         seen = set()
         slots, counts, tokens, want = [], [], [], []
+        axes = self.position_axes
+        explicit = [] if any(e.positions is not None for e in entries) else None
         for e in entries:
             n = len(e.tokens)
+            if explicit is not None:
+                base = cache.length(e.slot)
+                rows = e.positions if e.positions is not None else [[base + j] * axes for j in range(n)]
+                if len(rows) != n or any(len(r) != axes for r in rows):
+                    raise StepError(f"slot {e.slot}: positions must be {n} rows of {axes} numbers")
+                for r in rows:
+                    if min(r) < 0 or max(r) >= limit:
+                        raise StepError(f"slot {e.slot}: position {list(r)} is outside the model's {limit} positions")
+                    explicit.extend(int(v) for v in r)
             if n == 0:
                 raise StepError(f"slot {e.slot}: an entry needs at least one token")
             if e.slot in seen:
@@ -114,17 +130,19 @@ class StepFunction:
             slots.append(e.slot)
             counts.append(n)
             tokens.extend(toks)
+        self._explicit = explicit or []
         return slots, counts, tokens, want
 
-    def _context_from(self, dev: torch.Tensor, offsets, widths: Dict[str, int], host=None) -> StepContext:
+    def _context_from(self, dev: torch.Tensor, offsets, widths: Dict[str, int], host=None, sequential: bool = True) -> StepContext:
         """A step context over the device copy of a buffer laid out by ``CacheManager.build_step``."""
         def sec(k):
             start, size = offsets[k]
             return dev[start:start + size]
         S, T = offsets["seq_slot"][1], offsets["tokens"][1]
-        ctx = StepContext(n_rows=T, n_seqs=S, tokens=sec("tokens"), positions=sec("positions"),
+        ctx = StepContext(n_rows=T, n_seqs=S, tokens=sec("tokens"), positions=sec("positions").view(T, -1),
                           seq_q_start=sec("seq_q_start"), seq_q_len=sec("seq_q_len"), seq_pos0=sec("seq_pos0"),
-                          seq_slot=sec("seq_slot"), want_rows=sec("want_rows"), host=host or {}, decode_only=S == T)
+                          seq_slot=sec("seq_slot"), want_rows=sec("want_rows"), host=host or {}, decode_only=S == T,
+                          positions_sequential=sequential)
         for name, width in widths.items():
             ctx.groups[name] = GroupView(self.cache.page_size, sec(f"slot_map/{name}"), sec(f"table/{name}").view(S, width))
         for g in self.heads_per_kv:
@@ -134,13 +152,14 @@ class StepFunction:
     def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
         slots, counts, tokens, want = self._check_entries(entries)
         try:
-            host, offsets, widths = self.cache.build_step(slots, counts, tokens, want, self.heads_per_kv, self.rows_per_block)
+            host, offsets, widths = self.cache.build_step(slots, counts, tokens, want, self.heads_per_kv, self.rows_per_block,
+                                                          1, 0, self.position_axes, self._explicit)
         except CacheError as e:
             raise StepError(str(e)) from e
         dev = torch.from_numpy(host).to(self.rt.device)  # one buffer, one copy
         lists = {k: host[offsets[k][0]:offsets[k][0] + offsets[k][1]].tolist()
                  for k in ("tokens", "positions", "seq_q_start", "seq_q_len", "seq_pos0", "seq_slot", "want_rows")}
-        return self._context_from(dev, offsets, widths, lists)
+        return self._context_from(dev, offsets, widths, lists, sequential=not self._explicit)
 
     # ------------------------------------------------------------------ captured decode steps
     @staticmethod
@@ -157,19 +176,19 @@ class StepFunction:
 
     def _decode_shape(self, entries: Sequence[StepEntry], sampled: bool):
         """The buffer of a decode step (every row's logits are computed), its graph's key, and the
-        number of rows added.  The step is filled up to a bucket's size with copies of its first row,
-        so that a few graphs serve every batch size while requests end one by one: a copy writes the
-        same key and value to the same place and its logits are dropped; a decode step's time hardly
-        depends on a few rows more."""
+        number of rows added.  The step is filled up to a bucket's size, so that a few graphs serve every
+        batch size while requests end one by one, with rows that belong to no request: token 0 at position 0
+        of the cache manager's scratch slot and scratch page, so that they change no key, value or state that
+        a request owns (a mixer with state of fixed size may be captured too); their logits are dropped.  A
+        decode step's time hardly depends on a few rows more."""
         slots, counts, tokens, _ = self._check_entries(entries)
         pad = self._decode_bucket(len(slots)) - len(slots)
-        slots, counts, tokens = slots + [slots[0]] * pad, counts + [1] * pad, tokens + [tokens[0]] * pad
         try:
-            built = self.cache.build_step(slots, counts, tokens, list(range(len(slots))), self.heads_per_kv,
-                                          self.rows_per_block, self.TABLE_BUCKET)
+            built = self.cache.build_step(slots, counts, tokens, list(range(len(slots) + pad)), self.heads_per_kv,
+                                          self.rows_per_block, self.TABLE_BUCKET, pad, self.position_axes)
         except CacheError as e:
             raise StepError(str(e)) from e
-        return built, self._graph_key(counts, len(slots), built[2], sampled), pad
+        return built, self._graph_key(counts + [1] * pad, len(slots) + pad, built[2], sampled), pad
 
     def _ready(self, key: tuple, after: int) -> bool:
         """Whether the step of this shape runs from a graph: it has one, or has come ``after`` times."""
@@ -229,11 +248,17 @@ class StepFunction:
         dg.copied.record()
         if dg.graph is None:
             ctx = self._context_from(dg.dev, dg.offsets, widths)
+            # Everything is loaded and compiled before the capture: one run of the step outside it.  That run and the
+            # first replay both write the step's keys and values (the same ones, to the same places), but state of
+            # fixed size would advance twice: it is put back in between.
+            states = self.cache.device.snapshot_states() if self.cache.device is not None else None
             side = torch.cuda.Stream(device=self.rt.device)
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
-                self.model.forward(ctx)  # everything is loaded and compiled before the capture
+                self.model.forward(ctx)
             torch.cuda.current_stream().wait_stream(side)
+            if states is not None:
+                self.cache.device.restore_states(states)
             def sec(k):
                 return dg.dev[dg.offsets[k][0]:dg.offsets[k][0] + dg.offsets[k][1]]
             graph = torch.cuda.CUDAGraph()
@@ -265,7 +290,7 @@ class StepFunction:
         taken on the device: the host need not have seen them.  None if the step cannot take this
         path or its shape has not come often enough to be captured; ``OutOfPages`` before anything
         ran if the pages are not there."""
-        if not (self.use_graphs and all(len(e.tokens) == 1 for e in entries)
+        if not (self.use_graphs and all(len(e.tokens) == 1 and e.positions is None for e in entries)
                 and len({e.slot for e in entries}) == len(entries)):
             return None
         slots = [e.slot for e in entries]
@@ -325,7 +350,8 @@ class StepFunction:
                 raise OutOfPages(f"group {k}: the step needs {v} new pages, {cache.free_pages(k)} are free")
         for e in entries:
             cache.extend(e.slot, len(e.tokens))
-        if self.use_graphs and all(len(e.tokens) == 1 for e in entries) and len({e.slot for e in entries}) == len(entries):
+        graphs = self.use_graphs and all(e.positions is None for e in entries)  # a captured step takes positions from the cache
+        if graphs and all(len(e.tokens) == 1 for e in entries) and len({e.slot for e in entries}) == len(entries):
             built, key, pad = self._decode_shape(entries, False)
             if self._ready(key, self.DECODE_CAPTURE_AFTER):
                 logits, _ = self._run_graph(key, built)
@@ -342,7 +368,7 @@ class StepFunction:
                 logits = logits[torch.tensor(wanted, device=logits.device)]
             elif not borrow_logits:
                 logits = logits.clone()  # the graph's own buffer is overwritten by its next replay
-        elif self.use_graphs:
+        elif graphs:
             slots, counts, tokens, want = self._check_entries(entries)
             # block tables as wide as the next power of two of pages: a prompt that grows by a
             # portion a step keeps its shape for many steps
@@ -351,7 +377,8 @@ class StepFunction:
             while width < pages:
                 width *= 2
             try:
-                built = cache.build_step(slots, counts, tokens, want, self.heads_per_kv, self.rows_per_block, width)
+                built = cache.build_step(slots, counts, tokens, want, self.heads_per_kv, self.rows_per_block, width, 0,
+                                         self.position_axes)
             except CacheError as e:
                 raise StepError(str(e)) from e
             key = self._graph_key(counts, len(want), built[2], False)

@@ -101,12 +101,13 @@ class HipOps:
                 raise KernelError(f"{what}: {e}") from None
 
     # ------------------------------------------------------------------ elementwise
-    def embed(self, tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    def embed(self, tokens: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
         T, (V, d) = tokens.numel(), table.shape
         self._want(tokens, torch.int32, "embed tokens", T)
         self._want(table, self.dtype, "embed table")
         x = torch.empty((T, d), dtype=torch.float32, device=table.device)
-        self._check(self._core, self._core.ms_embed(_ptr(tokens), _ptr(table), _ptr(x), _c_int(T), _c_int(d), self._stream()))
+        self._check(self._core, self._core.ms_embed(_ptr(tokens), _ptr(table), _ptr(x), _c_int(T), _c_int(d), _c_float(scale),
+                                                    self._stream()))
         return x
 
     def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, rows: Optional[torch.Tensor] = None,

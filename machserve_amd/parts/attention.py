@@ -91,13 +91,14 @@ class Attention(Mixer):
             self.position.apply(q, k, ctx)
         g = self.attention_rows_per_token()
         decode = ctx.decode_only and g <= ops.DECODE_MAX_GROUP
-        if decode and self.writes_cache and (self.position is None or inv_freq is not None):
+        # the fused decode kernel rotates by the row's place in the cache: only where that is its position
+        if decode and self.writes_cache and (self.position is None or (inv_freq is not None and ctx.positions_sequential)):
             o = ops.decode_attention_fused(qkv, bias, inv_freq, view.slot_map, self.kpool, self.vpool, view.block_table,
                                            ctx.seq_pos0, s.heads, s.kv_heads, s.head_dim, view.page_size, s.window,
                                            self.scale)
             stream.add_linear(o, self.w_o)
             return
-        q = ops.rope_kv_write(qkv, bias, ctx.positions, inv_freq, view.slot_map if self.writes_cache else None,
+        q = ops.rope_kv_write(qkv, bias, ctx.position_axis(0), inv_freq, view.slot_map if self.writes_cache else None,
                               self.kpool if self.writes_cache else None, self.vpool if self.writes_cache else None,
                               s.heads, s.kv_heads, s.head_dim, view.page_size)
         if decode:

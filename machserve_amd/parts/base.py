@@ -38,10 +38,12 @@ class Runtime:
 
 @dataclass(frozen=True)
 class PagedKVRequest:
-    """A mixer's need of a paged cache: K and V per token, all keys or a window of them."""
+    """A mixer's need of a paged cache: K and V per token, all keys or a window of them.  ``v_head_dim``
+    is the width of a value where it differs from a key's ``head_dim`` (a compressed or latent cache)."""
     kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_head_dim: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -76,7 +78,7 @@ class StepContext:
     n_rows: int
     n_seqs: int
     tokens: torch.Tensor        # [T]
-    positions: torch.Tensor     # [T]
+    positions: torch.Tensor     # [T, axes]: what a position encoding encodes; one axis unless the model asks for more
     seq_q_start: torch.Tensor   # [S] first row of each request
     seq_q_len: torch.Tensor     # [S] number of its rows
     seq_pos0: torch.Tensor      # [S] position of its first row
@@ -86,6 +88,17 @@ class StepContext:
     attention_work: Dict[int, torch.Tensor] = field(default_factory=dict)  # rows per token -> [n, 2]
     host: Dict[str, object] = field(default_factory=dict)  # the same lists on the host
     decode_only: bool = False
+    # True: every row's position is, on every axis, its index in its request's cache (``seq_pos0`` onwards), so a
+    # kernel may take positions from there; False: the caller gave positions of its own for some rows
+    positions_sequential: bool = True
+
+    def position_axis(self, axis: int = 0) -> torch.Tensor:
+        """``[T]`` positions along one axis, contiguous."""
+        if self.positions.dim() == 1:
+            return self.positions
+        if self.positions.shape[1] == 1:
+            return self.positions.view(-1)
+        return self.positions[:, axis].contiguous()
 
 
 class ResidualStream:
@@ -226,6 +239,8 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
+    axes = 1  # numbers per position this encoding reads; the step's positions are [T, max over the model's encodings]
+
     def rotary_inv_freq(self) -> Optional[torch.Tensor]:
         """``[head_dim / 2]`` inverse frequencies if this is a plain rotation that the fused
         kernel can apply; None otherwise (then :meth:`apply` is called)."""
@@ -240,11 +255,13 @@ class Mixer(Part):
     """Mixes information between positions of one request (attention, or a recurrence)."""
 
     def cache_request(self):
-        """PagedKVRequest, SharedKVRequest, StateRequest or None."""
+        """PagedKVRequest, SharedKVRequest, StateRequest, None, or a list of these (pages and state together,
+        or several caches of different widths)."""
         return None
 
     def bind_cache(self, binding) -> None:
-        """Receive what the cache manager made for :meth:`cache_request`."""
+        """Receive what the cache manager made for :meth:`cache_request`: one binding, or for a list of
+        requests the list of their bindings in the same order."""
 
     def attention_rows_per_token(self) -> Optional[int]:
         """Query heads per KV head if the mixer needs attention work lists, else None."""

@@ -11,10 +11,13 @@ import torch
 
 from ..config.specs import ModelSpec
 from .base import Block, Part, ResidualStream, Runtime, StepContext, TensorDecl, require_kernel_sizes
-from .registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
+from .registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, register_embedding, register_head
 
 
+@register_embedding("embedding")
 class Embedding(Part):
+    """Rows of a table, times the spec's ``scale`` (1 for an embedding that is not scaled)."""
+
     def tensor_decls(self):
         return [TensorDecl("weight", (self.spec.vocab, self.spec.width), "matrix")]
 
@@ -22,15 +25,17 @@ class Embedding(Part):
         self.weight = t["weight"]
 
     def forward(self, tokens: torch.Tensor) -> torch.Tensor:
-        return self.rt.ops.embed(tokens, self.weight)
+        return self.rt.ops.embed(tokens, self.weight, getattr(self.spec, "scale", 1.0))
 
 
+@register_head("linear")
 class Head(Part):
-    """Output projection; tied to the embedding table when the spec says so, or when it
-    leaves it open and the checkpoint has no head tensor
-    (``crates/mach-model/src/loader.rs:1025-1033``)."""
+    """Output projection, times the spec's ``scale``; tied to the embedding table when the spec says so, or
+    when it leaves it open and the checkpoint has no head tensor
+    (``crates/mach-model/src/loader.rs:1025-1033``).  A head is built with the model's embedding part as
+    its third argument and has ``forward(h) -> float32 logits`` and ``vocab`` in its spec."""
 
-    def __init__(self, spec, rt, embedding: Embedding):
+    def __init__(self, spec, rt, embedding):
         super().__init__(spec, rt)
         self.embedding = embedding
         self.weight = None
@@ -49,7 +54,11 @@ class Head(Part):
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         w = self.weight if self.weight is not None else self.embedding.weight
-        return self.rt.ops.linear(h, w, None, out_f32=True)
+        logits = self.rt.ops.linear(h, w, None, out_f32=True)
+        scale = getattr(self.spec, "scale", 1.0)
+        if scale != 1.0:
+            logits *= scale
+        return logits
 
 
 class DecoderModel:
@@ -57,7 +66,7 @@ class DecoderModel:
         spec.validate()
         self.spec, self.rt = spec, rt
         require_kernel_sizes(rt, "output head", [("width", spec.embedding.width)])
-        self.embedding = Embedding(spec.embedding, rt)
+        self.embedding = EMBEDDINGS.build(spec.embedding, rt)
         self.blocks: List[Block] = []
         for layer in spec.layers:
             block_cls = BLOCKS.get(layer.block)
@@ -65,7 +74,7 @@ class DecoderModel:
                                          NORMS.build(layer.mixer_norm, rt), NORMS.build(layer.feed_forward_norm, rt)))
         self.order = list(spec.order)
         self.final_norm = NORMS.build(spec.final_norm, rt)
-        self.head = Head(spec.head, rt, self.embedding)
+        self.head = HEADS.build(spec.head, rt, self.embedding)
         self._bindings, self._rebind = [], False
 
     # ------------------------------------------------------------------ structure
@@ -84,15 +93,19 @@ class DecoderModel:
         what a run reads never depends on how the tokens were cut into steps.  A layer that
         reads another layer's cache reads that of the layer's latest earlier run."""
         from .base import SharedKVRequest
-        out = []
-        for p, i in enumerate(self.order):
-            req = self.blocks[i].mixer.cache_request()
+
+        def placed(req, p, i):
             if isinstance(req, SharedKVRequest):
                 earlier = [q for q in range(p) if self.order[q] == req.source_layer]
                 if not earlier:
                     raise ValueError(f"layer {i} reads the cache of layer {req.source_layer}, which has not run before it")
-                req = SharedKVRequest(earlier[-1])
-            out.append(req)
+                return SharedKVRequest(earlier[-1])
+            return req
+
+        out = []
+        for p, i in enumerate(self.order):
+            req = self.blocks[i].mixer.cache_request()
+            out.append([placed(r, p, i) for r in req] if isinstance(req, (list, tuple)) else placed(req, p, i))
         return out
 
     def bind_cache(self, device_cache) -> None:
@@ -114,6 +127,10 @@ class DecoderModel:
             raise ValueError("the mixers' attention kernels take blocks of different numbers of rows: "
                              + ", ".join(f"{name} (head size {hd}): {u}" for u, name, hd in sorted(units)))
         return next(iter(units))[0] if units else None
+
+    def position_axes(self) -> int:
+        """Numbers per position of a step: the most that any position encoding of the model reads."""
+        return max([getattr(p, "axes", 1) for p in self.parts()] + [1])
 
     @property
     def vocab(self) -> int:

@@ -23,8 +23,8 @@ class EmulatedOps:
     def _r(self, t):  # round to the element type, as a kernel's store does
         return t.to(self.dtype)
 
-    def embed(self, tokens, table):
-        return table[tokens.long()].float()
+    def embed(self, tokens, table, scale=1.0):
+        return table[tokens.long()].float() * scale
 
     SKINNY_ROWS = 64
     DECODE_MAX_GROUP = 16

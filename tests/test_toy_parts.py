@@ -14,11 +14,13 @@ from plain import qwen2_plain as P
 
 from machserve_amd.config import (AttentionSpec, EmbeddingSpec, GatedMlpSpec, HeadSpec, LayerSpec, ModelSpec, NormSpec,
                                   RotarySpec, register_architecture)
-from machserve_amd.parts import (FeedForward, Mixer, PositionEncoding, StateRequest, TensorDecl, register_feed_forward,
-                                 register_mixer, register_position_encoding)
+from machserve_amd.parts import (FeedForward, Head, Mixer, PagedKVRequest, PositionEncoding, StateRequest, TensorDecl,
+                                 register_feed_forward, register_head, register_mixer, register_position_encoding)
 
 WIDTH, HEADS, KV, HD, INTER, VOCAB = 48, 3, 1, 16, 80, 90
 EXPERTS, EXPERT_INTER = 3, 24
+VHD = 8                              # width of a value in the toy latent mixer; its keys are HD wide
+EMB_SCALE, HEAD_SCALE = 1.5, 0.5
 
 
 @dataclass(frozen=True)
@@ -94,10 +96,119 @@ class PositionScale(PositionEncoding):
     attention part must take the unfused path."""
 
     def apply(self, q, k, ctx):
-        f = (1.0 + ctx.positions.float() / 64.0)[:, None, None]
+        f = (1.0 + ctx.position_axis(0).float() / 64.0)[:, None, None]
         q *= f
         if k is not None:
             k *= f
+
+
+def two_axis_factor(positions, hd):
+    """[T, 1, hd]: the first half of a head is scaled by 1 + p0 / 64, the second by 1 + p1 / 32."""
+    p = positions.float()
+    return torch.cat([(1.0 + p[:, 0:1] / 64.0).expand(-1, hd // 2), (1.0 + p[:, 1:2] / 32.0).expand(-1, hd - hd // 2)], 1)[:, None, :]
+
+
+@register_position_encoding("toy_two_axes")
+class TwoAxes(PositionEncoding):
+    """A position is a pair of numbers; each scales one half of every head."""
+    axes = 2
+
+    def apply(self, q, k, ctx):
+        f = two_axis_factor(ctx.positions, q.shape[-1])
+        q *= f
+        if k is not None:
+            k *= f
+
+
+@dataclass(frozen=True)
+class LatentSpec:
+    kind: str
+    width: int
+    heads: int
+    key_dim: int
+    value_dim: int
+    position: object
+    tensors: Mapping[str, str] = field(default_factory=dict)
+
+
+@register_mixer("toy_latent")
+class LatentAttention(Mixer):
+    """One key/value head whose values are narrower than its keys, and beside the pages a state of fixed size
+    (how many tokens the request has had), which damps the output: it asks the cache manager for both at
+    once.  Its attention is written with ordinary tensor operations; it reads the step's host lists."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        from machserve_amd.parts import POSITION_ENCODINGS
+        self.position = POSITION_ENCODINGS.build(spec.position, rt)
+
+    def sub_parts(self):
+        return [self.position]
+
+    def tensor_decls(self):
+        sp = self.spec
+        return [TensorDecl("q", (sp.heads * sp.key_dim, sp.width)), TensorDecl("k", (sp.key_dim, sp.width)),
+                TensorDecl("v", (sp.value_dim, sp.width)), TensorDecl("o", (sp.width, sp.heads * sp.value_dim))]
+
+    def load(self, t):
+        self.w = {k: v.float() for k, v in t.items()}
+
+    def cache_request(self):
+        return [PagedKVRequest(1, self.spec.key_dim, None, v_head_dim=self.spec.value_dim), StateRequest({"count": (1,)})]
+
+    def bind_cache(self, bindings):
+        kv, state = bindings
+        self.group, self.kpool, self.vpool, self.count = kv.group, kv.kpool, kv.vpool, state.tensors["count"]
+
+    def forward(self, h, stream, ctx):
+        sp, x = self.spec, h.float()
+        T = x.shape[0]
+        q = (x @ self.w["q"].t()).view(T, sp.heads, sp.key_dim)
+        k = (x @ self.w["k"].t()).view(T, 1, sp.key_dim)
+        v = (x @ self.w["v"].t())
+        self.position.apply(q, k, ctx)
+        view = ctx.groups[self.group]
+        ps = view.page_size
+        where = view.slot_map.long()
+        self.kpool[where // ps, 0, where % ps, :] = k[:, 0].to(self.kpool.dtype)
+        self.vpool[where // ps, 0, :, where % ps] = v.to(self.vpool.dtype)
+        out = torch.empty((T, sp.heads, sp.value_dim), dtype=torch.float32, device=x.device)
+        for s, (slot, q0, n, p0) in enumerate(zip(ctx.host["seq_slot"], ctx.host["seq_q_start"], ctx.host["seq_q_len"], ctx.host["seq_pos0"])):
+            pages = view.block_table[s, :-(-(p0 + n) // ps)].long()
+            keys = self.kpool[pages, 0].reshape(-1, sp.key_dim).float()[:p0 + n]
+            vals = self.vpool[pages, 0].transpose(1, 2).reshape(-1, sp.value_dim).float()[:p0 + n]
+            scores = torch.einsum("thd,sd->ths", q[q0:q0 + n], keys) * sp.key_dim ** -0.5
+            seen = torch.arange(p0 + n, device=x.device)[None, :] <= (p0 + torch.arange(n, device=x.device))[:, None]
+            scores = scores.masked_fill(~seen[:, None, :], float("-inf"))
+            count = self.count[slot] + torch.arange(1, n + 1, device=x.device, dtype=torch.float32)
+            out[q0:q0 + n] = torch.softmax(scores, -1) @ vals / (1.0 + 0.01 * count)[:, None, None]
+            self.count[slot] = count[-1]
+        stream.add(out.reshape(T, -1) @ self.w["o"].t())
+
+
+@dataclass(frozen=True)
+class BiasedHeadSpec:
+    kind: str
+    vocab: int
+    width: int
+    tied: bool
+    scale: float
+    tensors: Mapping[str, str] = field(default_factory=dict)
+
+
+@register_head("toy_biased")
+class BiasedHead(Head):
+    """The framework's head, and a bias on every logit: another head is a registered class and a spec."""
+
+    def tensor_decls(self):
+        return super().tensor_decls() + [TensorDecl("bias", (self.spec.vocab,), "vector")]
+
+    def load(self, t):
+        super().load(t)
+        self.bias = t["bias"]
+
+    def forward(self, h):
+        return super().forward(h) + self.bias
 
 
 @dataclass
@@ -128,9 +239,13 @@ class ToyConfig:
             layer(1, RunningMeanSpec("toy_running_mean", WIDTH, {"w": "l1.mean.w"})),
             layer(2, att(2, RotarySpec("toy_position_scale", HD, 0.0), window=9)),
             layer(3, att(3, RotarySpec("rotary", HD, 1e4), kv_source=0)),
+            layer(4, LatentSpec("toy_latent", WIDTH, HEADS, HD, VHD, RotarySpec("toy_two_axes", HD, 0.0),
+                                {k: f"l4.lat.{k}" for k in ("q", "k", "v", "o")})),
         ]
-        return ModelSpec("ToyForCausalLM", EmbeddingSpec(VOCAB, WIDTH, {"weight": "emb"}), tuple(layers),
-                         order=(0, 1, 2, 1, 3), final_norm=norm("nf"), head=HeadSpec(VOCAB, WIDTH, True), max_positions=512)
+        return ModelSpec("ToyForCausalLM", EmbeddingSpec(VOCAB, WIDTH, {"weight": "emb"}, scale=EMB_SCALE), tuple(layers),
+                         order=(0, 1, 2, 1, 3, 4), final_norm=norm("nf"),
+                         head=BiasedHeadSpec("toy_biased", VOCAB, WIDTH, True, HEAD_SCALE, {"bias": "head.bias"}),
+                         max_positions=512)
 
 
 register_architecture("ToyForCausalLM", ToyConfig)
@@ -141,7 +256,9 @@ def toy_tensors(seed=0):
     r = lambda *s: torch.randn(*s, generator=g) * 0.2
     t = {"emb": r(VOCAB, WIDTH), "nf": 1 + r(WIDTH) * 0.2, "l1.mean.w": r(WIDTH, WIDTH),
          "l2.moe.router": r(EXPERTS, WIDTH) * 5, "l2.moe.w1": r(EXPERTS, EXPERT_INTER, WIDTH), "l2.moe.w2": r(EXPERTS, WIDTH, EXPERT_INTER)}
-    for i in range(4):
+    t["head.bias"] = r(VOCAB)
+    t["l4.lat.q"], t["l4.lat.k"], t["l4.lat.v"], t["l4.lat.o"] = r(HEADS * HD, WIDTH), r(HD, WIDTH), r(VHD, WIDTH), r(WIDTH, HEADS * VHD)
+    for i in range(5):
         t[f"l{i}.n1"], t[f"l{i}.n2"] = 1 + r(WIDTH) * 0.2, 1 + r(WIDTH) * 0.2
         if i != 2:  # layer 2 has the routed feed-forward
             t[f"l{i}.ff.gate.weight"], t[f"l{i}.ff.up.weight"], t[f"l{i}.ff.down.weight"] = r(INTER, WIDTH), r(INTER, WIDTH), r(WIDTH, INTER)
@@ -153,12 +270,28 @@ def toy_tensors(seed=0):
     return t
 
 
+def second_axis(n0, n1):
+    """The second number of the positions n0 .. n1 - 1 that the tests give the toy model: a row of a picture
+    three tokens wide, say."""
+    return [j // 3 for j in range(n0, n1)]
+
+
 def plain_toy(t, toks):
     """The toy model over a whole sequence with the plain parts."""
     T = len(toks)
     pos = torch.arange(T)
-    x = t["emb"][torch.tensor(toks)]
+    pos2 = torch.stack([pos, torch.tensor(second_axis(0, T))], 1)
+    x = t["emb"][torch.tensor(toks)] * EMB_SCALE
     kv0 = {}
+
+    def latent(xn):
+        q = (xn @ t["l4.lat.q"].t()).view(T, HEADS, HD) * two_axis_factor(pos2, HD)
+        k = (xn @ t["l4.lat.k"].t()).view(T, 1, HD) * two_axis_factor(pos2, HD)
+        v = (xn @ t["l4.lat.v"].t()).view(T, 1, VHD)
+        scores = torch.einsum("thd,sd->ths", q, k[:, 0]) * HD ** -0.5
+        scores = scores.masked_fill(~torch.tril(torch.ones(T, T, dtype=torch.bool))[:, None, :], float("-inf"))
+        o = torch.softmax(scores, -1) @ v[:, 0] / (1.0 + 0.01 * torch.arange(1, T + 1, dtype=torch.float32))[:, None, None]
+        return o.reshape(T, -1) @ t["l4.lat.o"].t()
 
     def attention(i, xn, kind):
         q = P.linear(xn, t[f"l{i}.att.q.weight"], t[f"l{i}.att.q.bias"]).view(T, HEADS, HD)
@@ -178,9 +311,11 @@ def plain_toy(t, toks):
         o = P.attention(q, k, v, window=9 if i == 2 else None)
         return P.linear(o.reshape(T, -1), t[f"l{i}.att.o.weight"])
 
-    for i in (0, 1, 2, 1, 3):
+    for i in (0, 1, 2, 1, 3, 4):
         xn = P.rms_norm(x, t[f"l{i}.n1"], 1e-5)
-        if i == 1:
+        if i == 4:
+            x = x + latent(xn)
+        elif i == 1:
             # the layer runs twice with the same weights; each run has a state of its own
             mean = torch.cumsum(xn, 0) / torch.arange(1, T + 1, dtype=torch.float32)[:, None]
             x = x + mean @ t["l1.mean.w"].t()
@@ -193,7 +328,7 @@ def plain_toy(t, toks):
             x = x + torch.stack([t["l2.moe.w2"][e] @ row for row, e in zip(y, choice)])
             continue
         x = x + P.swiglu(xn, t[f"l{i}.ff.gate.weight"], t[f"l{i}.ff.up.weight"], t[f"l{i}.ff.down.weight"])
-    return P.linear(P.rms_norm(x, t["nf"], 1e-5), t["emb"])
+    return P.linear(P.rms_norm(x, t["nf"], 1e-5), t["emb"]) * HEAD_SCALE + t["head.bias"]
 
 
 def _check(device, ops, dtype=torch.float32):
@@ -202,7 +337,10 @@ def _check(device, ops, dtype=torch.float32):
     t = toy_tensors()
     lm = load_model(config=config_from_dict({"architectures": ["ToyForCausalLM"]}), tensors=t, dtype=dtype,
                     device=device, page_size=16, num_pages=12, max_requests=3, ops=ops)
-    assert sorted(lm.cache.groups) == ["full", "window9"] and lm.cache.state_requests.keys() == {1, 3}
+    assert sorted(lm.cache.groups) == ["full", f"full/kv1x{HD}v{VHD}", "window9"] and lm.cache.state_requests.keys() == {1, 3}
+    assert lm.step.position_axes == 2
+    kv, st = lm.device_cache.binding(5)      # the latent layer asked for pages and a state at once
+    assert kv.kpool.shape[-1] == HD and kv.vpool.shape[-2] == VHD and st.tensors["count"].shape == (3 + 1, 1)
     assert not lm.step.use_graphs, "a mixer that reads host lists must keep the step function out of graphs"
     gen = torch.Generator().manual_seed(1)
     seqs = [torch.randint(0, VOCAB, (n,), generator=gen).tolist() for n in (40, 23)]
@@ -216,7 +354,8 @@ def _check(device, ops, dtype=torch.float32):
         entries = []
         for r in range(2):
             n = cuts[r][step]
-            entries.append(StepEntry(slots[r], seqs[r][fed[r]:fed[r] + n], list(range(n))))
+            positions = [[a, b] for a, b in zip(range(fed[r], fed[r] + n), second_axis(fed[r], fed[r] + n))]
+            entries.append(StepEntry(slots[r], seqs[r][fed[r]:fed[r] + n], list(range(n)), positions))
         logits = lm.step(entries)
         k = 0
         for r in range(2):
@@ -231,6 +370,103 @@ def _check(device, ops, dtype=torch.float32):
     lm.cache.release(slots[0])
     s = lm.cache.admit()
     assert s == slots[0] and all(lm.device_cache.states[p]["sum"][s].abs().max() == 0 for p in (1, 3))
+
+
+# ---------------------------------------------------------------------------- a toy model that may be captured
+
+@register_mixer("toy_running_mean_on_device")
+class DeviceRunningMean(RunningMean):
+    """The same running mean, reading nothing but device memory from the step: such a mixer may say
+    ``graph_safe`` and is then captured into graphs, filled up with rows that belong to no request (they
+    update the scratch slot's state, nobody's), and launched a step ahead like the framework's own attention."""
+    graph_safe = True
+
+    def forward(self, h, stream, ctx):
+        x = h.float()
+        T, dev = x.shape[0], x.device
+        rows = torch.arange(T, device=dev)
+        seq = torch.searchsorted(ctx.seq_q_start.long(), rows, right=True) - 1      # the request of every row
+        slot, q0 = ctx.seq_slot.long()[seq], ctx.seq_q_start.long()[seq]
+        earlier = ((seq[:, None] == seq[None, :]) & (rows[None, :] <= rows[:, None])).float()
+        run = earlier @ x + self.state["sum"][slot]
+        cnt = self.state["count"][slot] + (rows - q0 + 1).float()[:, None]
+        last = (ctx.seq_q_start + ctx.seq_q_len - 1).long()
+        self.state["sum"].index_copy_(0, ctx.seq_slot.long(), run[last])
+        self.state["count"].index_copy_(0, ctx.seq_slot.long(), cnt[last])
+        stream.add((run / cnt) @ self.w.float().t())
+
+
+@dataclass
+class GraphToyConfig:
+    @classmethod
+    def from_dict(cls, raw):
+        return cls()
+
+    def to_spec(self):
+        base = ToyConfig().to_spec()
+        mean = LayerSpec("prenorm", RunningMeanSpec("toy_running_mean_on_device", WIDTH, {"w": "l1.mean.w"}), base.layers[1].feed_forward,
+                         base.layers[1].mixer_norm, base.layers[1].feed_forward_norm)
+        return ModelSpec("GraphToyForCausalLM", EmbeddingSpec(VOCAB, WIDTH, {"weight": "emb"}), (base.layers[0], mean),
+                         order=(0, 1, 0), final_norm=base.final_norm, head=HeadSpec(VOCAB, WIDTH, True), max_positions=512)
+
+
+register_architecture("GraphToyForCausalLM", GraphToyConfig)
+
+
+def plain_graph_toy(t, toks):
+    T = len(toks)
+    pos = torch.arange(T)
+    x = t["emb"][torch.tensor(toks)]
+    for i in (0, 1, 0):
+        xn = P.rms_norm(x, t[f"l{i}.n1"], 1e-5)
+        if i == 1:
+            x = x + (torch.cumsum(xn, 0) / torch.arange(1, T + 1, dtype=torch.float32)[:, None]) @ t["l1.mean.w"].t()
+        else:
+            q = P.rope(P.linear(xn, t["l0.att.q.weight"], t["l0.att.q.bias"]).view(T, HEADS, HD), pos, 1e4)
+            k = P.rope(P.linear(xn, t["l0.att.k.weight"], t["l0.att.k.bias"]).view(T, KV, HD), pos, 1e4)
+            v = P.linear(xn, t["l0.att.v.weight"]).view(T, KV, HD)
+            x = x + P.linear(P.attention(q, k, v).reshape(T, -1), t["l0.att.o.weight"])
+        xn = P.rms_norm(x, t[f"l{i}.n2"], 1e-5)
+        x = x + P.swiglu(xn, t[f"l{i}.ff.gate.weight"], t[f"l{i}.ff.up.weight"], t[f"l{i}.ff.down.weight"])
+    return P.linear(P.rms_norm(x, t["nf"], 1e-5), t["emb"])
+
+
+def graph_toy_tensors():
+    t = toy_tensors()
+    keep = ("emb", "nf", "l0.", "l1.")
+    return {k: v for k, v in t.items() if k.startswith(keep)}
+
+
+def _generate_graph_toy(device, ops, n_new):
+    from machserve_amd.config import config_from_dict
+    from machserve_amd.engine import Engine, load_model
+    t = graph_toy_tensors()
+    lm = load_model(config=config_from_dict({"architectures": ["GraphToyForCausalLM"]}), tensors=t, dtype=torch.float32,
+                    device=device, page_size=16, num_pages=24, max_requests=4, ops=ops)
+    gen = torch.Generator().manual_seed(3)
+    prompts = [torch.randint(0, VOCAB, (n,), generator=gen).tolist() for n in (7, 19, 12)]
+    eng = Engine(lm, max_batch_tokens=64)
+    got = eng.generate(prompts, max_new=n_new)
+    for p, g in zip(prompts, got):
+        seq = list(p)
+        for tok in g:   # greedy: every generated token is the plain model's most likely one, by a clear margin or a tie's lowest index
+            logits = plain_graph_toy(t, seq)[-1]
+            assert tok == P.argmax_first(logits) or logits[tok] >= logits.max() - 2e-4 * (1 + logits.abs().max()), len(seq)
+            seq.append(tok)
+    return lm
+
+
+def test_toy_model_with_state_on_the_device_on_the_cpu_stand_ins():
+    _generate_graph_toy("cpu", EmulatedOps(), 12)
+
+
+@pytest.mark.gpu
+def test_a_mixer_with_state_is_captured_filled_up_and_launched_ahead():
+    """Three requests decode in captured steps of four rows (one belongs to nobody) that are launched a step
+    ahead: the state of the requests is what the plain model's is, token for token, for 60 tokens."""
+    lm = _generate_graph_toy("cuda:0", None, 60)
+    assert lm.step.use_graphs and len(lm.step._graphs) >= 1
+    assert any(k[0] == (1, 1, 1, 1) for k in lm.step._graphs), "a step of three requests is captured as one of four rows"
 
 
 def test_toy_model_on_the_cpu_stand_ins():
