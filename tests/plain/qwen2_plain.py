@@ -64,7 +64,16 @@ def rope(x: torch.Tensor, positions: torch.Tensor, theta: float) -> torch.Tensor
     return torch.cat([a * c - b * s, a * s + b * c], dim=-1)
 
 
-def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int | None = None) -> torch.Tensor:
+def same(x: torch.Tensor) -> torch.Tensor:
+    return x
+
+
+def to_bf16_and_back(x: torch.Tensor) -> torch.Tensor:
+    """What storing a value in bfloat16 does to it (round to nearest even, crates/mach-model/src/fp16.rs:84-94)."""
+    return x.to(torch.bfloat16).to(x.dtype)
+
+
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int | None = None, rounded=same) -> torch.Tensor:
     """Causal grouped-query attention over a whole sequence.
 
     ``q`` is ``[T, H, hd]``, ``k``/``v`` are ``[T, KV, hd]``.  Query head ``h`` reads
@@ -86,7 +95,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int | N
             lo = 0 if window is None else max(0, p - window + 1)
             scores = (k[lo:p + 1, kv, :] @ q[p, h, :]) * scale
             e = torch.exp(scores - scores.max())
-            out[p, h, :] = (e[:, None] * v[lo:p + 1, kv, :]).sum(dim=0) / e.sum()
+            # (a reduced-precision engine rounds the probabilities that multiply the values, not those it sums)
+            out[p, h, :] = (rounded(e)[:, None] * v[lo:p + 1, kv, :]).sum(dim=0) / e.sum()
     return out
 
 
@@ -95,16 +105,16 @@ def silu(x: torch.Tensor) -> torch.Tensor:
     return x / (1.0 + torch.exp(-x))
 
 
-def swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
+def swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, rounded=same) -> torch.Tensor:
     """``down( silu(gate(x)) * up(x) )``: the activation is on the gate branch.
 
     crates/mach-model/src/ref_model.rs:299-309, crates/mach-model/src/kernels.rs:131-140,
     tools/ref_llama.py:120-123.
     """
-    return linear(silu(linear(x, w_gate)) * linear(x, w_up), w_down)
+    return linear(rounded(silu(linear(x, w_gate)) * linear(x, w_up)), w_down)
 
 
-def attention_block(x, w, prefix, positions, sizes, window=None):
+def attention_block(x, w, prefix, positions, sizes, window=None, rounded=same):
     """q/k/v projections with optional bias, rotation of q and k, attention, output
     projection without bias.  crates/mach-model/src/batched.rs:3566-3679, 4022-4031;
     tools/ref_llama.py:100-119.
@@ -114,9 +124,9 @@ def attention_block(x, w, prefix, positions, sizes, window=None):
     q = linear(x, w[prefix + "q_proj.weight"], w.get(prefix + "q_proj.bias"))
     k = linear(x, w[prefix + "k_proj.weight"], w.get(prefix + "k_proj.bias"))
     v = linear(x, w[prefix + "v_proj.weight"], w.get(prefix + "v_proj.bias"))
-    q = rope(q.view(T, H, hd), positions, sizes["theta"])
-    k = rope(k.view(T, KV, hd), positions, sizes["theta"])
-    o = attention(q, k, v.view(T, KV, hd), window)
+    q = rounded(rope(q.view(T, H, hd), positions, sizes["theta"]))
+    k = rounded(rope(k.view(T, KV, hd), positions, sizes["theta"]))
+    o = rounded(attention(q, k, rounded(v.view(T, KV, hd)), window, rounded))
     return linear(o.reshape(T, H * hd), w[prefix + "o_proj.weight"])
 
 
@@ -131,8 +141,12 @@ def layer_windows(sizes) -> list:
     return [sizes["sliding_window"] if i >= sizes["max_window_layers"] else None for i in range(L)]
 
 
-def forward(weights: dict, sizes: dict, tokens, compute=torch.float32, start_pos: int = 0) -> torch.Tensor:
-    """Logits ``[T, vocab]`` at every position of one whole sequence.
+def forward(weights: dict, sizes: dict, tokens, compute=torch.float32, start_pos: int = 0, rounded=same) -> torch.Tensor:
+    """Logits ``[T, vocab]`` at every position of one whole sequence.  ``rounded`` is applied wherever a
+    reduced-precision run of the same formulas stores a value in its element type: the inputs of every matrix
+    product (the norms' outputs, the attention output, SiLU(gate) * up), q, and the keys and values of the
+    cache, and the probabilities that multiply the values; the stream, the sums, the softmax and its
+    statistics stay as computed.  The default rounds nothing.
 
     Pre-norm blocks ``x += attn(norm(x)); x += mlp(norm(x))``, final norm, head =
     ``lm_head.weight`` when the tensor exists, else the embedding table.
@@ -146,11 +160,11 @@ def forward(weights: dict, sizes: dict, tokens, compute=torch.float32, start_pos
     windows = layer_windows(sizes)
     for i in range(sizes["layers"]):
         p = f"model.layers.{i}."
-        xn = rms_norm(x, w[p + "input_layernorm.weight"], sizes["eps"])
-        x = x + attention_block(xn, w, p + "self_attn.", positions, sizes, windows[i])
-        xn = rms_norm(x, w[p + "post_attention_layernorm.weight"], sizes["eps"])
-        x = x + swiglu(xn, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
-    xf = rms_norm(x, w["model.norm.weight"], sizes["eps"])
+        xn = rounded(rms_norm(x, w[p + "input_layernorm.weight"], sizes["eps"]))
+        x = x + attention_block(xn, w, p + "self_attn.", positions, sizes, windows[i], rounded)
+        xn = rounded(rms_norm(x, w[p + "post_attention_layernorm.weight"], sizes["eps"]))
+        x = x + swiglu(xn, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"], rounded)
+    xf = rounded(rms_norm(x, w["model.norm.weight"], sizes["eps"]))
     head = w["lm_head.weight"] if "lm_head.weight" in w and not sizes.get("tied", False) else w["model.embed_tokens.weight"]
     return linear(xf, head)
 
