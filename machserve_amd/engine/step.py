@@ -47,6 +47,10 @@ class _DecodeGraph:
         self.sampled = None  # int32 [2, B] when the graph also samples: tokens, bits of the logprobs
         self.copied = torch.cuda.Event()  # the last upload of `pinned` has finished
 
+    def held_bytes(self) -> int:
+        """Device memory this captured step holds for good: its buffer and its results."""
+        return sum(t.numel() * t.element_size() for t in (self.dev, self.logits, self.sampled) if t is not None)
+
 
 @dataclass
 class LaunchedDecode:
@@ -64,6 +68,11 @@ class LaunchedDecode:
 class StepFunction:
     TABLE_BUCKET = 8        # captured block tables are this many pages wide, or a multiple
     MAX_GRAPHS = 256        # captured steps kept; the one unused longest goes first
+    # ... and the most memory they may hold for good between them: each keeps its step buffer and its results (the
+    # logits [rows, vocabulary] in 32-bit are nearly all of it: 39 MB at 64 rows of a 152k vocabulary).  What a
+    # captured step needs only while it runs comes from one pool that all captures share, since they run one
+    # after another on one stream.  This reserve is device memory beside the weights and the page pools.
+    MAX_GRAPH_BYTES = 2 << 30
     CAPTURE_MAX_ROWS = 320  # a larger step keeps the device busy longer than the host needs to launch it (and replays slower)
     # A capture costs 7 ms; a replayed step is 0.9 ms shorter than a launched one with a few requests, 0.3 to
     # 0.4 ms with 64 requests or a few hundred rows.  While requests end one by one most shapes last a few
@@ -86,6 +95,7 @@ class StepFunction:
         self.use_graphs = (use_graphs and rt.device.type == "cuda"
                            and all(getattr(b.mixer, "graph_safe", False) for b in getattr(model, "blocks", [])))
         self._graphs: "OrderedDict[tuple, _DecodeGraph]" = OrderedDict()
+        self._graph_pool = None  # the memory pool that all captures share
         self._seen: Dict[tuple, int] = {}
         self._results: Dict[int, list] = {}  # pinned buffers for the samples, three per batch size, in turn
         self._launches = 0
@@ -262,7 +272,9 @@ class StepFunction:
             def sec(k):
                 return dg.dev[dg.offsets[k][0]:dg.offsets[k][0] + dg.offsets[k][1]]
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
                 dg.logits = self.model.forward(ctx)
                 if sampling is not None:
                     dg.sampled = self.rt.ops.sample_packed(
@@ -271,10 +283,14 @@ class StepFunction:
                         also_tokens=sec("tokens"))
             dg.graph = graph
             self._graphs[key] = dg
-            while len(self._graphs) > self.MAX_GRAPHS:
+            while len(self._graphs) > 1 and (len(self._graphs) > self.MAX_GRAPHS or self.graph_bytes() > self.MAX_GRAPH_BYTES):
                 self._graphs.popitem(last=False)
         dg.graph.replay()
         return (dg.sampled if sampling is not None else dg.logits), dg
+
+    def graph_bytes(self) -> int:
+        """Device memory that the captured steps hold for good between them."""
+        return sum(g.held_bytes() for g in self._graphs.values())
 
     def decode_and_sample(self, entries: Sequence[StepEntry], temperatures, top_ks, top_ps, states):
         """A decode-only step (one token per request) with sampling inside the captured graph: one

@@ -181,13 +181,19 @@ def test_captured_steps_are_dropped_and_captured_again(dirs):
         eng.step_pipelined()
         step += 1
         assert step < 2000
-    assert len(st._graphs) <= 2
+    assert len(st._graphs) <= 2 and 0 < st.graph_bytes() <= 2 * 4 * (sizes["vocab"] * 4 + 4096)
     again = [k for k in set(captures) if captures.count(k) > 1]
     assert dropped and again, f"a shape must have been dropped and captured again ({len(captures)} captures, {len(dropped)} dropped)"
     done = eng.scheduler.finished
     for rid, (_, prompt, max_new) in zip(ids, reqs):
         assert done[rid].generated == P.greedy_generate(w, sizes, prompt, max_new), f"request {rid}"
     eng.loaded.cache.check()
+    # the same limit by bytes: with room for one step's results only, one captured step is kept
+    st.MAX_GRAPHS, st.MAX_GRAPH_BYTES = 256, 1
+    for n in (3, 9):
+        eng.add(random_prompt(n, sizes["vocab"], 400 + n), 20)
+    eng.run()
+    assert len(st._graphs) == 1
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
