@@ -2,19 +2,37 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--dtype bf16|f32]
                     [--shape 0.5b|1.5b|7b] [--batch B] [--context C] [--page-size P]
+                    [--no-points] [--no-kernels] [--more-shapes]
 
 Default run: Qwen2.5-0.5B layer sizes with random weights (synthetic token ids), 8 requests
 that each hold a 2,048-token context, K decode steps through the whole engine (scheduler,
-step function, sampler).  One JSON line: ``value`` is decoded tokens a second at batch 8;
-``prefill`` is one 2,048-token prompt in one step; ``roofline`` prices the decode step's
-mandatory bytes (every weight once, the live requests' cache) against 8 TB/s;
-``points`` holds decode at batch 1 and 64.
+step function, sampler), timed three times in a row; the median window is reported.  One JSON
+line: ``value`` is decoded tokens a second at batch 8; ``prefill`` is one 2,048-token prompt in
+one step; ``roofline`` prices the decode step's mandatory bytes (every weight once, the live
+requests' cache) against 8 TB/s; ``points`` holds decode at batch 1 and 64, decode at longer
+contexts and a longer prefill (``points_detail``: their times and fractions of the published
+peak); ``launches_per_step`` counts the kernels of a decode step; ``measured_peaks`` is what the
+box itself gives a device-to-device copy and a loop of matrix instructions; ``kernels`` breaks
+the decode step and the prefill down by kind of kernel (time a step, GB/s or TFLOP/s, fraction
+of the published and of the measured peak), from a second run of the same work under
+``rocprofv3 --kernel-trace`` whose dispatches are matched, in order, with the operations that
+the step issues.
+
+Method of the reference: time per step over a fixed number of steps after a warm-up
+(``crates/mach-model/examples/lctx_bench.rs:64-89``, ``docs/benchmark-protocol.md:43-75``).
 """
 from __future__ import annotations
 
 import argparse
+import csv
+import glob
 import json
+import os
+import shutil
+import statistics
+import subprocess
 import sys
+import tempfile
 import time
 
 PEAK_HBM_GBS = 8000.0
@@ -29,8 +47,6 @@ QWEN25_05B = {
     "max_position_embeddings": 32768, "rms_norm_eps": 1e-6, "rope_theta": 1000000.0, "tie_word_embeddings": True,
     "hidden_act": "silu", "use_sliding_window": False,
 }
-
-
 # the two larger configurations of the same architecture (random weights, same distribution)
 QWEN25_15B = dict(QWEN25_05B, hidden_size=1536, num_hidden_layers=28, num_attention_heads=12, num_key_value_heads=2,
                   intermediate_size=8960)
@@ -56,6 +72,136 @@ def prefill_flops(cfg, T):
     return gemm + attn
 
 
+# ------------------------------------------------------------------------------------ the operations of a step, by kind
+
+PRODUCT_OPS = {  # name -> positions of (rows operand, weight) among the arguments
+    "linear_split": (0, 1), "linear": (0, 1), "linear_residual": (0, 1), "linear_residual_prenorm": (0, 1),
+    "linear_swiglu": (0, 1), "linear_swiglu_scaled": (0, 3), "linear_split_normed": (0, 4), "linear_swiglu_normed": (0, 4),
+}
+OTHER_OPS = {"embed": "embedding", "rmsnorm": "norm", "add_partials": "norm", "rope_kv_write": "rotation and cache write",
+             "paged_attention": "attention", "decode_attention_fused": "attention", "decode_attention": "attention",
+             "sample": "sampling", "sample_packed": "sampling", "top_logprobs": "sampling", "logit_edit": "sampling"}
+
+
+class Recorder:
+    """Wraps the kernel boundary's methods: while ``on()`` says so, every outermost call is listed with its kind,
+    the kernels it launched, and for a matrix product the bytes of its weight and its floating-point operations."""
+
+    def __init__(self, ops, vocab, on):
+        self.ops, self.calls, self.depth, self.on = ops, [], 0, on
+        for name in list(PRODUCT_OPS) + list(OTHER_OPS):
+            setattr(ops, name, self._wrap(name, getattr(ops, name), vocab))
+
+    def _wrap(self, name, inner, vocab):
+        def call(*a, **kw):
+            if self.depth or not self.on():
+                return inner(*a, **kw)
+            self.depth += 1
+            before = self.ops.launch_count()
+            try:
+                out = inner(*a, **kw)
+            finally:
+                self.depth -= 1
+            launched = self.ops.launch_count() - before
+            kind, nbytes, flops = OTHER_OPS.get(name), 0, 0
+            if name in PRODUCT_OPS:
+                rows, w = a[PRODUCT_OPS[name][0]], a[PRODUCT_OPS[name][1]]
+                kind = "head" if w.shape[0] >= vocab else "products"
+                nbytes, flops = w.numel() * w.element_size(), 2 * rows.shape[0] * w.numel()
+            self.calls.append([kind, launched, nbytes, flops])
+            return out
+        return call
+
+
+def trace_rows(folder):
+    """(start, end, name) of every dispatch of the engine's own kernels in a rocprofv3 kernel trace, in order."""
+    rows = []
+    for path in glob.glob(os.path.join(folder, "**", "*kernel_trace.csv"), recursive=True):
+        with open(path, newline="") as f:
+            for r in csv.DictReader(f):
+                if "ms::" in r["Kernel_Name"]:
+                    rows.append((int(r["Start_Timestamp"]), int(r["End_Timestamp"]), r["Kernel_Name"]))
+    rows.sort()
+    return rows
+
+
+def account(calls, rows, n_steps, peak_of, measured_of, extra):
+    """Per kind of kernel: launches and microseconds a step, and with the kind's bytes or operations its rate and the
+    fractions of the published and of the measured peak.  ``calls`` lists one step's operations in order; ``rows``
+    ends with the dispatches of ``n_steps`` such steps."""
+    per_launch = [c for c in calls for _ in range(c[1])]
+    L = len(per_launch)
+    if L == 0 or len(rows) < n_steps * L:
+        return {"error": f"{len(rows)} traced dispatches for {n_steps} steps of {L} launches"}
+    rows = rows[-n_steps * L:]
+    kinds = {}
+    for i, (start, end, _) in enumerate(rows):
+        k = kinds.setdefault(per_launch[i % L][0], {"launches": 0, "us": 0.0})
+        k["us"] += (end - start) / 1e3 / n_steps
+    for c in calls:
+        k = kinds.setdefault(c[0], {"launches": 0, "us": 0.0})
+        k["launches"] += c[1]
+        k["bytes"] = k.get("bytes", 0) + c[2]
+        k["flops"] = k.get("flops", 0) + c[3]
+    for name, (nbytes, flops) in extra.items():
+        if name in kinds:
+            kinds[name]["bytes"], kinds[name]["flops"] = nbytes, flops
+    out = {}
+    for name, k in kinds.items():
+        rec = {"launches": k["launches"], "us": round(k["us"], 2)}
+        unit = peak_of.get(name)
+        work = k.get("bytes", 0) if unit == "GB/s" else k.get("flops", 0)
+        if unit and work and k["us"] > 0:
+            rate = work / (k["us"] * 1e-6) / (1e9 if unit == "GB/s" else 1e12)
+            peak = PEAK_HBM_GBS if unit == "GB/s" else peak_of["flops_peak"] / 1e12
+            rec.update({"rate": round(rate, 1), "unit": unit if unit == "GB/s" else "TFLOP/s", "frac": round(rate / peak, 4)})
+            if measured_of.get(unit):
+                rec["frac_of_measured"] = round(rate / measured_of[unit], 4)
+        out[name] = rec
+    span = sum((rows[(s + 1) * L - 1][1] - rows[s * L][0]) for s in range(n_steps)) / 1e3 / n_steps
+    busy = sum(k["us"] for k in kinds.values())
+    out["all"] = {"launches": L, "us_in_kernels": round(busy, 2), "us_first_to_last": round(span, 2),
+                  "us_between_kernels": round(span - busy, 2)}
+    return out
+
+
+def measured_peaks(dtype_name):
+    """What the box gives: a device-to-device copy of 1 GiB (bytes read plus written over the time) and a loop of
+    nothing but matrix instructions of the run's element type."""
+    import ctypes
+    import torch
+    from machserve_amd.kernels import build
+    out = {}
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0")
+    dst = torch.empty_like(src)
+    best = 1e9
+    for _ in range(5):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        dst.copy_(src)
+        b.record()
+        b.synchronize()
+        best = min(best, a.elapsed_time(b))
+    out["copy_GBs"] = round(2 * (1 << 30) / (best * 1e-3) / 1e9, 1)
+    del src, dst
+    lib = ctypes.CDLL(build.ensure_library("probe", dtype_name))
+    blocks, iters = 4096, 2048 if dtype_name == "bf16" else 1024
+    buf = torch.empty(blocks * 256, dtype=torch.float32, device="cuda:0")
+    flops = ctypes.c_double(0.0)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    best = 1e9
+    for _ in range(4):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        if lib.ms_probe_mfma(ctypes.c_void_p(buf.data_ptr()), blocks, iters, ctypes.byref(flops), stream) != 0:
+            return out
+        b.record()
+        b.synchronize()
+        best = min(best, a.elapsed_time(b))
+    out["mfma_TFLOPs"] = round(flops.value / (best * 1e-3) / 1e12, 1)
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -67,9 +213,13 @@ def main() -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
     ap.add_argument("--shape", default="0.5b", choices=sorted(SHAPES), help="layer sizes (default: the 0.5B configuration)")
     ap.add_argument("--page-size", type=int, default=64)
-    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--no-points", action="store_true", help="skip the further points and the prefill")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the break-down by kind of kernel (a second run under rocprofv3)")
+    ap.add_argument("--more-shapes", action="store_true", help="add decode and prefill points of the 1.5B and 7B layer sizes")
     ap.add_argument("--sync-steps", action="store_true", help="wait for each decode step's tokens before the next is launched")
-    ap.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiles)")
+    ap.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for profiles)")
+    ap.add_argument("--prefill-tokens", type=int, default=None, help="tokens of the prefill (default: the context)")
+    ap.add_argument("--record-calls", default=None, help=argparse.SUPPRESS)  # file that receives one step's operations (the traced run)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -81,30 +231,43 @@ def main() -> int:
     from machserve_amd.sampling import SamplingParams
     from machserve_amd.weights import random_tensor_dict
 
-    shape_name, shape = SHAPES[args.shape]
-    raw = dict(shape)
-    full_layers = raw["num_hidden_layers"]
-    if args.layers:
-        raw["num_hidden_layers"] = args.layers
-    cfg = config_from_dict(raw)
     dt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
-    tensors = random_tensor_dict(cfg, 0, dt, device="cuda:0")
-    ctx, page = args.context, args.page_size
+    page = args.page_size
     gen = torch.Generator().manual_seed(1)
+    models = {}
 
-    def prompts(n, length):
+    def model_of(shape):
+        if shape not in models:
+            raw = dict(SHAPES[shape][1])
+            full = raw["num_hidden_layers"]
+            if args.layers and shape == args.shape:
+                raw["num_hidden_layers"] = args.layers
+            cfg = config_from_dict(raw)
+            models.clear()  # one model's weights at a time
+            torch.cuda.empty_cache()
+            models[shape] = (cfg, random_tensor_dict(cfg, 0, dt, device="cuda:0"), full)
+        return models[shape]
+
+    def prompts(cfg, n, length):
         return [torch.randint(0, cfg.vocab_size, (length,), generator=gen).tolist() for _ in range(n)]
 
-    def make_engine(batch, budget):
-        per_req = -(-(ctx + args.warmup + args.steps + 2 * batch + 96) // page)
-        lm = load_model(config=cfg, tensors=tensors, dtype=dt, page_size=page, num_pages=batch * per_req + 4,
-                        max_requests=batch)
+    recording = [False]
+    recorders = []
+
+    def make_engine(shape, batch, budget, ctx, windows=1):
+        cfg, tensors, _ = model_of(shape)
+        per_req = -(-(ctx + args.warmup + windows * args.steps + 2 * batch + 96) // page)
+        lm = load_model(config=cfg, tensors=tensors, dtype=dt, page_size=page, num_pages=batch * per_req + 4, max_requests=batch)
+        if args.record_calls and not recorders:
+            recorders.append(Recorder(lm.rt.ops, cfg.vocab_size, lambda: recording[0]))
         return Engine(lm, max_batch_tokens=budget, max_running=batch)
 
-    def decode_run(batch):
-        eng = make_engine(batch, 4096)
-        for p in prompts(batch, ctx):
-            eng.add(p, args.warmup + args.steps + 2 * batch + 88, SamplingParams())  # early ones decode while later ones prefill
+    def decode_run(shape, batch, ctx, windows=3):
+        """(tokens a second, milliseconds a step) of the median of ``windows`` timed runs of ``--steps`` decode steps."""
+        cfg = model_of(shape)[0]
+        eng = make_engine(shape, batch, 4096, ctx, windows)
+        for p in prompts(cfg, batch, ctx):
+            eng.add(p, args.warmup + windows * args.steps + 2 * batch + 88, SamplingParams())  # early ones decode while later ones prefill
         while any(not r.decoding for r in eng.scheduler.running) or eng.scheduler.waiting:
             eng.step()
         # the engine's own loop (Engine.run): a step is launched while the tokens of the step before
@@ -112,48 +275,94 @@ def main() -> int:
         step = eng.step if args.sync_steps else eng.step_pipelined
         # the engine captures a decode step into a graph once its shape has come a number of times:
         # that happens before the warm-up, not in the timed steps
+        recording[0] = bool(args.record_calls)  # the capture issues the step's operations once: they are listed then
         for _ in range(eng.loaded.step.DECODE_CAPTURE_AFTER + 2):
             step()
         for _ in range(args.warmup):
             step()
-        torch.cuda.synchronize()
-        before, seen = eng.steps, 0
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            em, _ = step()
-            seen += len(em)
-        torch.cuda.synchronize()
-        dt_s = time.perf_counter() - t0
-        assert eng.steps - before == args.steps, "exactly the timed steps ran on the device"
-        assert batch * (args.steps - 1) <= seen <= batch * args.steps  # the first call may have had nothing before it
+        times = []
+        for _ in range(windows):
+            torch.cuda.synchronize()
+            before, seen = eng.steps, 0
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                em, _ = step()
+                seen += len(em)
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            assert eng.steps - before == args.steps, "exactly the timed steps ran on the device"
+            assert batch * (args.steps - 1) <= seen <= batch * args.steps  # the first call may have had nothing before it
+        recording[0] = False
         del eng
         torch.cuda.empty_cache()
+        dt_s = statistics.median(times)
         return batch * args.steps / dt_s, dt_s / args.steps * 1e3
 
-    def prefill_run():
-        eng = make_engine(1, ctx)
+    def prefill_run(shape, tokens):
+        cfg = model_of(shape)[0]
+        eng = make_engine(shape, 1, tokens, tokens)
         times = []
         for rep in range(4):
-            eng.add(prompts(1, ctx)[0], 1, SamplingParams())
+            eng.add(prompts(cfg, 1, tokens)[0], 1, SamplingParams())
             torch.cuda.synchronize()
+            recording[0] = bool(args.record_calls) and rep == 3
+            if recording[0] and recorders:
+                del recorders[0].calls[:]
             t0 = time.perf_counter()
             em, done = eng.step()
             torch.cuda.synchronize()
+            recording[0] = False
             times.append(time.perf_counter() - t0)
             assert len(em) == 1 and len(done) == 1
         del eng
         torch.cuda.empty_cache()
         return min(times[1:])
 
-    nums = model_numbers(cfg, dt.itemsize)
+    def decode_bytes(cfg, batch, ctx, windows):
+        nums = model_numbers(cfg, dt.itemsize)
+        mean_ctx = ctx + args.warmup + windows * args.steps / 2
+        return nums["weight_bytes"] + batch * mean_ctx * nums["kv_bytes_per_token"]
+
+    def decode_point(shape, batch, ctx):
+        tok_s, ms = decode_run(shape, batch, ctx)
+        rate = decode_bytes(model_of(shape)[0], batch, ctx, 3) / (ms * 1e-3) / 1e9
+        return tok_s, {"ms": round(ms, 4), "GBs": round(rate, 1), "frac": round(rate / PEAK_HBM_GBS, 4)}
+
+    def prefill_point(shape, tokens):
+        t = prefill_run(shape, tokens)
+        fl = prefill_flops(model_of(shape)[0], tokens)
+        return tokens / t, {"ms": round(t * 1e3, 3), "TFLOPs": round(fl / t / 1e12, 1), "frac": round(fl / t / PEAK_FLOPS[args.dtype], 4)}
+
+    shape_name = SHAPES[args.shape][0]
+    cfg, _, full_layers = model_of(args.shape)
+    ctx = args.context
+    prefill_tokens = args.prefill_tokens or ctx
+
+    def save_calls(kind):
+        """The traced run's list of one step's operations: the last graph's worth for decoding, the last step's for prefill."""
+        calls = recorders[0].calls if recorders else []
+        if kind == "decode":  # the capture ran the step's operations once under recording: the last such run
+            ends = [i for i, c in enumerate(calls) if c[0] == "sampling"]
+            starts = [i for i, c in enumerate(calls) if c[0] == "embedding"]
+            if ends and starts:
+                first = max(s for s in starts if s < ends[-1])
+                calls = calls[first:ends[-1] + 1]
+        with open(args.record_calls, "w") as f:
+            json.dump(calls, f)
+
     if args.prefill_only:
-        t = prefill_run()
-        print(json.dumps({"prefill": {"value": round(ctx / t, 1), "tokens": ctx, "ms": round(t * 1e3, 3),
-                                      "frac": round(prefill_flops(cfg, ctx) / t / PEAK_FLOPS[args.dtype], 4)}}))
+        tok_s, rec = prefill_point(args.shape, prefill_tokens)
+        if args.record_calls:
+            save_calls("prefill")
+        print(json.dumps({"prefill": {"value": round(tok_s, 1), "tokens": prefill_tokens, **rec}}))
         return 0
-    tok_s, ms = decode_run(args.batch)
-    step_bytes = nums["weight_bytes"] + args.batch * (ctx + args.warmup + args.steps / 2) * nums["kv_bytes_per_token"]
-    achieved = step_bytes / (ms * 1e-3) / 1e9
+    if args.record_calls:  # the traced run: one window, nothing else
+        decode_run(args.shape, args.batch, ctx, windows=1)
+        save_calls("decode")
+        return 0
+
+    tok_s, ms = decode_run(args.shape, args.batch, ctx)
+    achieved = decode_bytes(cfg, args.batch, ctx, 3) / (ms * 1e-3) / 1e9
     out = {
         "metric": f"decode tok/s at batch {args.batch}, {ctx}-token contexts ({shape_name} shape)",
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -165,25 +374,94 @@ def main() -> int:
             "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
             "tied_head": bool(cfg.tie_word_embeddings), "rope_theta": cfg.rope_theta, "rms_eps": cfg.rms_norm_eps,
-            "page_size": page, "prefill_tokens": ctx, "sampling": "greedy",
+            "page_size": page, "prefill_tokens": prefill_tokens, "sampling": "greedy",
             "stepping": "one at a time" if args.sync_steps else "launched one step ahead",
         },
+        "timed": "median of three windows of `steps` steps",
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
     }
+    peaks = measured_peaks(args.dtype)
+    out["measured_peaks"] = peaks
+    if peaks.get("copy_GBs"):
+        out["roofline"]["frac_of_measured_copy"] = round(achieved / peaks["copy_GBs"], 4)
     if not args.no_points:
-        t = prefill_run()
-        fl = prefill_flops(cfg, ctx)
-        out["prefill"] = {"value": round(ctx / t, 1), "tokens": ctx, "ms": round(t * 1e3, 3),
-                          "frac": round(fl / t / PEAK_FLOPS[args.dtype], 4)}
-        b1, _ = decode_run(1)
-        b64, _ = decode_run(64)
-        out["points"] = {"decode_b1": round(b1, 1), "decode_b64": round(b64, 1)}
+        p_tok_s, p = prefill_point(args.shape, prefill_tokens)
+        out["prefill"] = {"value": round(p_tok_s, 1), "tokens": prefill_tokens, "ms": p["ms"], "frac": p["frac"]}
+        points, detail = {}, {}
+        for name, batch, c in (("decode_b1", 1, ctx), ("decode_b64", 64, ctx), ("decode_b8_ctx8192", 8, 8192),
+                               ("decode_b8_ctx32000", 8, 32000)):
+            if c + 4 * args.steps + 300 > cfg.max_position_embeddings:
+                continue
+            v, detail[name] = decode_point(args.shape, batch, c)
+            points[name] = round(v, 1)
+        v, detail["prefill_8192"] = prefill_point(args.shape, 8192)
+        points["prefill_8192"] = round(v, 1)
         if args.dtype == "bf16" and cfg.num_hidden_layers == full_layers and args.shape == "0.5b" and ctx == 2048:
-            out["vs_reference"] = {"decode_b64_ctx2048": round(b64 / REF_DECODE_B64_CTX2048, 2),
-                                   "prefill_2048": round(ctx / t / REF_PREFILL_2048, 2)}
+            out["vs_reference"] = {"decode_b64_ctx2048": round(points["decode_b64"] / REF_DECODE_B64_CTX2048, 2),
+                                   "prefill_2048": round(p_tok_s / REF_PREFILL_2048, 2)}
+        if args.more_shapes:
+            for shape, runs in (("1.5b", (("decode_b8", 8, 512), ("decode_b64", 64, 2048))), ("7b", (("decode_b1", 1, 2048), ("decode_b64", 64, 2048)))):
+                if shape == args.shape:
+                    continue
+                for name, batch, c in runs:
+                    v, detail[f"{shape}_{name}_ctx{c}"] = decode_point(shape, batch, c)
+                    points[f"{shape}_{name}_ctx{c}"] = round(v, 1)
+                v, detail[f"{shape}_prefill_2048"] = prefill_point(shape, 2048)
+                points[f"{shape}_prefill_2048"] = round(v, 1)
+            model_of(args.shape)
+        out["points"], out["points_detail"] = points, detail
+    models.clear()
+    torch.cuda.empty_cache()
+    if not args.no_kernels:
+        out["kernels"] = kernels_by_kind(args, cfg, dt, peaks, ctx, prefill_tokens)
+        if isinstance(out["kernels"].get("decode"), dict) and "all" in out["kernels"]["decode"]:
+            out["launches_per_step"] = out["kernels"]["decode"]["all"]["launches"]
     print(json.dumps(out))
     return 0
+
+
+def kernels_by_kind(args, cfg, dt, peaks, ctx, prefill_tokens):
+    """The decode step and the prefill again under ``rocprofv3 --kernel-trace``, in processes of their own; their
+    dispatches are matched in order with the operations that the traced run lists for one step."""
+    prof = shutil.which("rocprofv3") or ("/opt/rocm/bin/rocprofv3" if os.path.exists("/opt/rocm/bin/rocprofv3") else None)
+    if prof is None:
+        return {"error": "rocprofv3 not found"}
+    me = os.path.abspath(__file__)
+    base = [sys.executable, me, "--steps", str(args.steps), "--warmup", str(args.warmup), "--batch", str(args.batch), "--context", str(ctx),
+            "--dtype", args.dtype, "--shape", args.shape, "--page-size", str(args.page_size)] + (["--layers", str(args.layers)] if args.layers else [])
+    nums = model_numbers(cfg, dt.itemsize)
+    measured = {"GB/s": peaks.get("copy_GBs"), "TFLOP/s": peaks.get("mfma_TFLOPs")}
+    out = {}
+    env = dict(os.environ, TMPDIR=tempfile.gettempdir())
+    for kind in ("decode", "prefill"):
+        with tempfile.TemporaryDirectory() as tmp:
+            calls_file = os.path.join(tmp, "calls.json")
+            cmd = [prof, "--kernel-trace", "--output-format", "csv", "-d", os.path.join(tmp, "trace"), "--"] + base + ["--record-calls", calls_file]
+            if kind == "prefill":
+                cmd += ["--prefill-only", "--prefill-tokens", str(prefill_tokens)]
+            try:
+                r = subprocess.run(cmd, capture_output=True, text=True, timeout=420, cwd=tmp, env=env)
+                if r.returncode != 0 or not os.path.exists(calls_file):
+                    out[kind] = {"error": f"the traced run ended with {r.returncode}: {r.stderr[-300:]}"}
+                    continue
+                with open(calls_file) as f:
+                    calls = json.load(f)
+                rows = trace_rows(os.path.join(tmp, "trace"))
+            except (subprocess.TimeoutExpired, OSError, ValueError) as e:
+                out[kind] = {"error": f"{type(e).__name__}: {e}"}
+                continue
+            if kind == "decode":
+                mean_ctx = ctx + args.warmup + args.steps / 2
+                peak_of = {"products": "GB/s", "head": "GB/s", "attention": "GB/s"}
+                extra = {"attention": (args.batch * mean_ctx * nums["kv_bytes_per_token"], 0)}
+                out[kind] = account(calls, rows, args.steps, peak_of, measured, extra)
+            else:
+                T = prefill_tokens
+                peak_of = {"products": "TFLOP/s", "attention": "TFLOP/s", "head": "GB/s", "flops_peak": PEAK_FLOPS[args.dtype]}
+                extra = {"attention": (0, cfg.num_hidden_layers * 4.0 * cfg.num_attention_heads * cfg.head_dim * (T * (T + 1) / 2))}
+                out[kind] = account(calls, rows, 1, peak_of, measured, extra)
+    return out
 
 
 if __name__ == "__main__":

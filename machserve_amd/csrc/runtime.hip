@@ -7,6 +7,7 @@
 namespace ms {
 
 static thread_local char g_error[512] = "";
+static long g_launches = 0;  // kernels this library has launched (asked for by the benchmark's launch count)
 
 void set_error(const char* fmt, ...) {
     va_list ap;
@@ -16,6 +17,7 @@ void set_error(const char* fmt, ...) {
 }
 
 int check_launch(const char* what) {
+    ++g_launches;
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_error("%s: launch failed: %s", what, hipGetErrorString(e));
@@ -27,6 +29,9 @@ int check_launch(const char* what) {
 }  // namespace ms
 
 extern "C" const char* ms_last_error() { return ms::g_error; }
+
+// Kernels launched by this library so far (every launch goes through check_launch).
+extern "C" long ms_launch_count() { return ms::g_launches; }
 
 // 1 for the bfloat16 build, 0 for the 32-bit build.
 extern "C" int ms_elem_is_bf16() { return ms::kBf16 ? 1 : 0; }

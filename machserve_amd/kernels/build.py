@@ -67,6 +67,8 @@ def _hipcc() -> str:
 def _sources_of(kind: str):
     if kind == "core":
         return list(CORE_SOURCES)
+    if kind == "probe":  # the benchmark's measurement of the matrix cores; nothing on the product path loads it
+        return ["runtime.hip", "probe.hip"]
     return ["runtime.hip", "attention.hip"]
 
 
@@ -212,6 +214,7 @@ def build_all(force: bool = True, workers: int = 4) -> list:
     jobs = []
     for elem in ELEM_DEFINE:
         jobs.append(("core", elem, None))
+        jobs.append(("probe", elem, None))
         for nd in ATTENTION_TILES:
             jobs.append(("attention", elem, nd))
     with ThreadPoolExecutor(max_workers=workers) as pool:

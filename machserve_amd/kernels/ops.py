@@ -56,6 +56,7 @@ class HipOps:
         self.device = torch.device(device)
         self._index = self.device.index if self.device.index is not None else torch.cuda.current_device()
         self.elem = "bf16" if dtype == torch.bfloat16 else "f32"
+        self._libs: list = []
         self._core = self._load(build.ensure_library("core", self.elem))
         self._attn = {}
         # what the library plans for a product depends on its sizes alone: asked once per size
@@ -67,7 +68,13 @@ class HipOps:
         except OSError as e:
             raise KernelError(f"cannot load {path}: {e}") from None
         lib.ms_last_error.restype = ctypes.c_char_p
+        lib.ms_launch_count.restype = ctypes.c_long
+        self._libs.append(lib)
         return lib
+
+    def launch_count(self) -> int:
+        """Kernels launched so far by the libraries this object has loaded."""
+        return sum(int(lib.ms_launch_count()) for lib in self._libs)
 
     def _stream(self):
         """torch's current stream on this object's device as a raw handle."""
