@@ -36,7 +36,7 @@ import tempfile
 import time
 
 PEAK_HBM_GBS = 8000.0
-PEAK_FLOPS = {"bf16": 2.5e15, "f32": 157.3e12}
+PEAK_FLOPS = {"bf16": 2.5e15, "f16": 2.5e15, "f32": 157.3e12}
 # the reference's own numbers for this model on its hardware (RX 7900 XTX, fp16)
 REF_DECODE_B64_CTX2048 = 4777.0   # README.md:15, docs/benchmark-protocol.md:74-75
 REF_PREFILL_2048 = 2048 / 0.289   # README.md:18
@@ -210,7 +210,7 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (named in config)")
-    ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
     ap.add_argument("--shape", default="0.5b", choices=sorted(SHAPES), help="layer sizes (default: the 0.5B configuration)")
     ap.add_argument("--page-size", type=int, default=64)
     ap.add_argument("--no-points", action="store_true", help="skip the further points and the prefill")
@@ -231,7 +231,7 @@ def main() -> int:
     from machserve_amd.sampling import SamplingParams
     from machserve_amd.weights import random_tensor_dict
 
-    dt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    dt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[args.dtype]
     page = args.page_size
     gen = torch.Generator().manual_seed(1)
     models = {}

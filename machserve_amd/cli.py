@@ -12,7 +12,7 @@ top_p, seed, presence_penalty, frequency_penalty, max_new, eos, stop.
 
     python -m machserve_amd --model DIR --prompt-ids 1,2,3 --max-new 16
     python -m machserve_amd --random-config config.json --seed 0 --prompt-file prompts.txt
-    python -m machserve_amd random-weights --config config.json --seed 0 --out DIR [--dtype f32|bf16]
+    python -m machserve_amd random-weights --config config.json --seed 0 --out DIR [--dtype f32|bf16|f16]
     python -m machserve_amd doctor
 """
 from __future__ import annotations
@@ -66,11 +66,11 @@ def random_weights(argv) -> int:
     ap.add_argument("--config", required=True, help="config.json of the architecture")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--out", required=True, help="folder to write")
-    ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"], help="dtype the tensors are stored in")
+    ap.add_argument("--dtype", default="f32", choices=["f32", "bf16", "f16"], help="dtype the tensors are stored in")
     args = ap.parse_args(argv)
     with open(args.config) as f:
         raw = json.load(f)
-    out = write_random_model(raw, args.seed, args.out, torch.float32 if args.dtype == "f32" else torch.bfloat16)
+    out = write_random_model(raw, args.seed, args.out, {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[args.dtype])
     print(out)
     return 0
 
@@ -86,7 +86,7 @@ def main(argv=None) -> int:
     ap.add_argument("--model", default=_env("MACH_MODEL"), help="folder with config.json and model.safetensors")
     ap.add_argument("--random-config", help="config.json to build random weights from instead of --model")
     ap.add_argument("--weights-seed", type=int, default=0, help="seed of the random weights")
-    ap.add_argument("--dtype", default=_env("MACH_DTYPE", "bf16"), help="bf16 | f32")
+    ap.add_argument("--dtype", default=_env("MACH_DTYPE", "bf16"), help="bf16 | f16 | f32 (MACH_DTYPE of the reference: f16 | f32)")
     ap.add_argument("--prompt-ids", action="append", default=[], help="token ids of one prompt, comma separated")
     ap.add_argument("--prompt-file", help="one prompt a line, token ids separated by spaces or commas")
     ap.add_argument("--max-new", type=int, default=16)

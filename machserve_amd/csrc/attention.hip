@@ -34,7 +34,7 @@ namespace ms {
 constexpr int ND = MS_ATTN_ND;
 constexpr int HDT = ND * 16;             // head size of the tile
 constexpr int NKS = (HDT + 31) / 32;     // K steps of 32 over the head size
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
 constexpr int BKV = ND <= 8 ? 64 : 32;
 constexpr int EPC = 8;
 // LDS has 64 banks of 4 bytes: the 16-byte reads of K fragments (row l % 16, chunk l / 16) are free of
@@ -50,7 +50,7 @@ constexpr int NTP = (NT + 1) / 2;        // pairs of score tiles = K steps of th
 constexpr int K_LD = HDT + KPAD, V_LD = BKV + VPAD;
 constexpr int ROWS_PER_BLOCK = 64;
 constexpr float NEG_BIG = -1e30f;
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
 constexpr int MAX_KEY_GROUPS = ND <= 4 ? 4 : 2;  // groups of four waves that may share a block's keys
 #else
 constexpr int MAX_KEY_GROUPS = 2;
@@ -78,7 +78,7 @@ struct AttnArgs {
 };
 
 __device__ __forceinline__ float exp_f(float x) {
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
     return __expf(x);
 #else
     return expf(x);
@@ -86,7 +86,7 @@ __device__ __forceinline__ float exp_f(float x) {
 }
 
 __device__ __forceinline__ float exp2_f(float x) {
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
     return __builtin_amdgcn_exp2f(x);
 #else
     return exp2f(x);
@@ -99,7 +99,7 @@ __device__ __forceinline__ float exp2_f(float x) {
 // and a causal prompt's last rows see every key: more groups cut that chain.
 // Waves per SIMD the compiler has to leave room for: with the small bfloat16 tiles two blocks of a CU
 // overlap one's LDS traffic with the other's arithmetic, if the registers allow them.
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
 template <int KG> constexpr int attention_waves_per_simd() { return ND <= 4 ? (KG == 1 ? 3 : 4) : 1; }
 #else
 template <int KG> constexpr int attention_waves_per_simd() { return 1; }

@@ -1,15 +1,19 @@
 // Shared definitions of the gfx950 kernels: element type of this build, MFMA wrappers,
 // wave reductions and the error channel of the extern "C" entry points.
 //
-// One library is built per element type: MS_ELEM_BF16 (bfloat16 storage, 32-bit
-// accumulation) or MS_ELEM_F32 (everything in true 32-bit; its matrix products use the
+// One library is built per element type: MS_ELEM_BF16 or MS_ELEM_F16 (bfloat16 or half-precision
+// storage, 32-bit accumulation; MS_ELEM_HALF is defined for both: they share every tile and
+// schedule) or MS_ELEM_F32 (everything in true 32-bit; its matrix products use the
 // full-precision v_mfma_f32_16x16x4_f32, never a reduced-precision mode).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#if defined(MS_ELEM_BF16) == defined(MS_ELEM_F32)
-#error "define exactly one of MS_ELEM_BF16, MS_ELEM_F32"
+#if (defined(MS_ELEM_BF16) + defined(MS_ELEM_F16) + defined(MS_ELEM_F32)) != 1
+#error "define exactly one of MS_ELEM_BF16, MS_ELEM_F16, MS_ELEM_F32"
+#endif
+#if defined(MS_ELEM_BF16) || defined(MS_ELEM_F16)
+#define MS_ELEM_HALF 1
 #endif
 
 namespace ms {
@@ -17,35 +21,42 @@ namespace ms {
 constexpr int WAVE = 64;
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 // ---- element type ---------------------------------------------------------------
-#ifdef MS_ELEM_BF16
+#if defined(MS_ELEM_BF16)
 typedef __bf16 elem_t;
-constexpr bool kBf16 = true;
+#elif defined(MS_ELEM_F16)
+typedef _Float16 elem_t;
 #else
 typedef float elem_t;
-constexpr bool kBf16 = false;
+#endif
+#ifdef MS_ELEM_HALF
+constexpr bool kHalf = true;  // two-byte elements
+typedef elem_t half8_t __attribute__((ext_vector_type(8)));
+typedef elem_t half4_t __attribute__((ext_vector_type(4)));
+#else
+constexpr bool kHalf = false;
 #endif
 
 __device__ __forceinline__ float to_f32(float v) { return v; }
 __device__ __forceinline__ float to_f32(__bf16 v) { return (float)v; }
+__device__ __forceinline__ float to_f32(_Float16 v) { return (float)v; }
 
-// Round-to-nearest-even conversion of the compiler's own __bf16 cast.
+// Round-to-nearest-even conversion of the compiler's own casts.
 template <typename T> __device__ __forceinline__ T from_f32(float v);
 template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
 template <> __device__ __forceinline__ __bf16 from_f32<__bf16>(float v) { return (__bf16)v; }
+template <> __device__ __forceinline__ _Float16 from_f32<_Float16>(float v) { return (_Float16)v; }
 
 // A fragment is 8 consecutive elements along the reduction dimension of one row of an
 // operand: for lane l of a wave, row l % 16 and elements (l / 16) * 8 .. + 8 of a chunk of
 // 32.  Both operands of a product use the same split, so the sum over the chunk is
 // complete whatever order the hardware takes the elements in.
 struct alignas(16) Frag {
-#ifdef MS_ELEM_BF16
-    bf16x8_t v;
+#ifdef MS_ELEM_HALF
+    half8_t v;
 #else
     float v[8];
 #endif
@@ -53,8 +64,8 @@ struct alignas(16) Frag {
 
 __device__ __forceinline__ Frag frag_zero() {
     Frag f;
-#ifdef MS_ELEM_BF16
-    for (int i = 0; i < 8; ++i) f.v[i] = (__bf16)0.0f;
+#ifdef MS_ELEM_HALF
+    for (int i = 0; i < 8; ++i) f.v[i] = (elem_t)0.0f;
 #else
     for (int i = 0; i < 8; ++i) f.v[i] = 0.0f;
 #endif
@@ -64,8 +75,8 @@ __device__ __forceinline__ Frag frag_zero() {
 // Load 8 consecutive elements (16-byte aligned for bf16, 32-byte for float).
 __device__ __forceinline__ Frag frag_load(const elem_t* p) {
     Frag f;
-#ifdef MS_ELEM_BF16
-    f.v = *reinterpret_cast<const bf16x8_t*>(p);
+#ifdef MS_ELEM_HALF
+    f.v = *reinterpret_cast<const half8_t*>(p);
 #else
     const f32x4* q = reinterpret_cast<const f32x4*>(p);
     f32x4 a = q[0], b = q[1];
@@ -76,8 +87,8 @@ __device__ __forceinline__ Frag frag_load(const elem_t* p) {
 }
 
 __device__ __forceinline__ void frag_store(elem_t* p, const Frag& f) {
-#ifdef MS_ELEM_BF16
-    *reinterpret_cast<bf16x8_t*>(p) = f.v;
+#ifdef MS_ELEM_HALF
+    *reinterpret_cast<half8_t*>(p) = f.v;
 #else
     f32x4* q = reinterpret_cast<f32x4*>(p);
     f32x4 a = {f.v[0], f.v[1], f.v[2], f.v[3]}, b = {f.v[4], f.v[5], f.v[6], f.v[7]};
@@ -88,8 +99,10 @@ __device__ __forceinline__ void frag_store(elem_t* p, const Frag& f) {
 // acc[16x16] += A[16 rows x 32] * B[16 cols x 32]^T, both given as fragments.
 // Result layout: lane l holds rows (l / 16) * 4 + i (i = 0..3) of column l % 16.
 __device__ __forceinline__ void mma_16x16x32(f32x4& acc, const Frag& a, const Frag& b) {
-#ifdef MS_ELEM_BF16
+#if defined(MS_ELEM_BF16)
     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
+#elif defined(MS_ELEM_F16)
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.v, b.v, acc, 0, 0, 0);
 #else
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v[i], b.v[i], acc, 0, 0, 0);

@@ -223,9 +223,9 @@ __global__ __launch_bounds__(256) void rope_kv_write_quads_kernel(RopeArgs a) {
         return r;
     };
     auto store_quad = [](elem_t* o, const f32x4& v) {
-#ifdef MS_ELEM_BF16
-        bf16x4_t b = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
-        *reinterpret_cast<bf16x4_t*>(o) = b;
+#ifdef MS_ELEM_HALF
+        half4_t b = {(elem_t)v[0], (elem_t)v[1], (elem_t)v[2], (elem_t)v[3]};
+        *reinterpret_cast<half4_t*>(o) = b;
 #else
         *reinterpret_cast<f32x4*>(o) = v;
 #endif
@@ -281,7 +281,7 @@ extern "C" int ms_rmsnorm(float* x, const float* partials, int n_partials, int T
     MS_REQUIRE(d * sizeof(float) <= 60000, "rmsnorm: width %d exceeds the row buffer", d);
     MS_REQUIRE(n_partials == 0 || partials, "rmsnorm: %d partial sums without a buffer", n_partials);
     const size_t ps = (size_t)T * d, smem = (size_t)d * sizeof(float);
-    const bool f32_out = out_f32 || !kBf16;
+    const bool f32_out = out_f32 || !kHalf;
     const int groups = d % 4 == 0 ? (d <= 1024 ? 1 : (d <= 2048 ? 2 : (d <= 4096 ? 4 : 0))) : 0;
     const bool aligned = (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(partials)) % 16 == 0;
     if (groups && aligned && n_partials <= 16) {

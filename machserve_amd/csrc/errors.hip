@@ -1,5 +1,7 @@
 // Error channel of the extern "C" entry points: a refused call returns non-zero and
-// leaves its reason here.  Role of `check` in crates/mach-kernel-sys/src/hip.rs:370.
+// leaves its reason here; and the count of kernels launched.  Role of `check` in
+// crates/mach-kernel-sys/src/hip.rs:370.  (Memory, streams and graph capture are torch's: the
+// entry points take raw pointers and a stream.)
 #include "common.cuh"
 #include <cstdarg>
 #include <cstdio>
@@ -33,5 +35,5 @@ extern "C" const char* ms_last_error() { return ms::g_error; }
 // Kernels launched by this library so far (every launch goes through check_launch).
 extern "C" long ms_launch_count() { return ms::g_launches; }
 
-// 1 for the bfloat16 build, 0 for the 32-bit build.
-extern "C" int ms_elem_is_bf16() { return ms::kBf16 ? 1 : 0; }
+// Bytes of an element of this build: 2 (bfloat16 or half precision) or 4.
+extern "C" int ms_elem_bytes() { return (int)sizeof(ms::elem_t); }

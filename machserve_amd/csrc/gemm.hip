@@ -22,7 +22,7 @@
 
 namespace ms {
 
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
 constexpr int EPC = 8;   // elements per 16-byte chunk
 constexpr int KPAD = 16;  // row padding in elements: rows of 96 (BK 32) or 160 (BK 64) bytes
 #else
@@ -47,7 +47,7 @@ struct EpiArgs {
 };
 
 __device__ __forceinline__ float silu_f(float g) {
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
     return g / (1.0f + __expf(-g));
 #else
     return g / (1.0f + expf(-g));
@@ -59,7 +59,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
                                                    int M, int N, int K, EpiArgs ep) {
     static_assert(WM * WN == 4, "four waves");
     static_assert(BK % 32 == 0, "K step in MFMA steps of 32");
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
     constexpr bool DIRECT = BK == 64;
 #else
     constexpr bool DIRECT = false;
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
             *reinterpret_cast<u32x4*>(&Ws[buf][at(row, my_chunk)]) = rw[i];
         }
     };
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
     // One K step of both tiles straight into LDS buffer `buf`: lane l of a wave's load lands at the wave's
     // base + 16 l.  Written in assembly: of a load that it knows to write LDS the compiler makes every later
     // LDS read wait (vmcnt(0)), and nothing would be in flight during the multiplications; the waits are
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
         }
     };
     if constexpr (DIRECT && STAGES > 2) {
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
         // A block that is alone on its CU (few tiles: one tile of rows under a weight of a few hundred column
         // tiles) has nobody to hide its loads behind, and with one step in flight every step costs a trip to
         // memory.  Here STAGES - 1 steps are in flight: the loads of step kt + STAGES - 1 go out before step
@@ -248,7 +248,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
         }
 #endif
     } else if constexpr (DIRECT) {
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
         if (nk == 1 && partial) {
             load_global_tail(k_begin);
             store_lds(0);
@@ -391,7 +391,7 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
                            A, W, M, N, K, ep);                                                                        \
         return check_launch("gemm " #BM_ "x" #BN_ "x" #BK_);                                                          \
     } while (0)
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
     const int forced = g_gemm_config;
     if (forced == 1) MS_GEMM(128, 128, 2, 2, 32);
     if (forced == 2) MS_GEMM(128, 128, 2, 2, 64);
@@ -434,7 +434,7 @@ static constexpr int g_force_splits = 0;
 #endif
 
 static int plan_tiled_splits(int M, int N, int K) {
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
     const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
     if (b128 >= 300 && g_force_splits == 0) return 1;
     // More than six slices cost more in the consumer's sums than they gain here (with very few tiles - a
@@ -504,7 +504,7 @@ extern "C" int ms_linear_swiglu(const void* a, const void* w, void* out, int M, 
 
 // Whether ms_linear_swiglu_scaled takes this shape: bfloat16, one tile of rows, whole K steps of 64.
 extern "C" int ms_swiglu_scaled_takes(int M, int I, int K) {
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
     (void)I;
     return M >= 1 && M <= 64 && K % 64 == 0 && K >= 256;
 #else
@@ -517,7 +517,7 @@ extern "C" int ms_swiglu_scaled_takes(int M, int I, int K) {
 // divided by the row's root mean square, 1 / sqrt(sum_p row_ss[p, row] / K + eps), before the activation.
 extern "C" int ms_linear_swiglu_scaled(const void* a, const float* row_ss, int ss_parts, float eps, const void* w, void* out, int M, int I,
                                        int K, hipStream_t stream) {
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
     MS_REQUIRE(ms_swiglu_scaled_takes(M, I, K), "gated product with row factors: M=%d K=%d is not taken", M, K);
     MS_REQUIRE(row_ss && ss_parts >= 1, "gated product with row factors: the rows' sums of squares are missing");
     MS_REQUIRE((reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0, "gemm: operands must be 16-byte aligned");
@@ -542,7 +542,7 @@ extern "C" int ms_tiled_partials(int M, int N, int K) { return plan_tiled_splits
 // layer sizes, 8 to 64 rows).  The choice changes the order of the sums, so results differ in rounding.
 extern "C" int ms_prefers_tiled(int M, int N, int K) {
     if (M > 64) return 1;
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
     // Above 32 rows the tiled kernel, with K cut over enough blocks, beats the few-rows kernel for every
     // weight (0.5B q/k/v projection at 64 rows: 9.7 us few-rows, 4.9 us tiled in seven slices).
     if (M > 32) return 1;

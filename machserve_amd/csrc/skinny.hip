@@ -37,7 +37,7 @@ struct SkinnyArgs {
 };
 
 __device__ __forceinline__ float silu_sk(float g) {
-#ifdef MS_ELEM_BF16
+#ifdef MS_ELEM_HALF
     return g / (1.0f + __expf(-g));
 #else
     return g / (1.0f + expf(-g));
@@ -412,7 +412,7 @@ struct SkinnyPlan { int wn, ksi, ksb, k_per_wave; };
 // Columns per wave in units of 16: with more than 32 rows and enough columns to keep every CU busy,
 // a wave takes 64 columns, so that the rows it re-reads (from L2, they are shared by all waves)
 // weigh no more than the weights it streams.
-static int skinny_nt(int M, int N) { return (kBf16 && M > 32 && N >= 4096) ? 4 : 2; }  // 32-bit fragments are twice as large
+static int skinny_nt(int M, int N) { return (kHalf && M > 32 && N >= 4096) ? 4 : 2; }  // 32-bit fragments are twice as large
 
 #ifdef MS_MEASURE  // switches for measurements, in no library that serves
 static int g_force_ksi = 0;  // waves along K inside a block (1 = four column waves)
@@ -462,7 +462,7 @@ static int launch_skinny(const SkinnyArgs& a, const SkinnyPlan& p, hipStream_t s
     MS_REQUIRE(a.K % 8 == 0, "skinny product: the reduction size K=%d must be a multiple of 8", a.K);
     if (a.M <= 16) return launch_skinny_mt<1, 2, EPI>(a, p, stream);
     if (a.M <= 32) return launch_skinny_mt<2, 2, EPI>(a, p, stream);
-    if constexpr (kBf16) {
+    if constexpr (kHalf) {
         if (skinny_nt(a.M, a.N) == 4) {
             if (a.M <= 48) return launch_skinny_mt<3, 4, EPI>(a, p, stream);
             return launch_skinny_mt<4, 4, EPI>(a, p, stream);

@@ -14,17 +14,17 @@ from ..parts import DecoderModel, Runtime
 from ..weights import Checkpoint, TensorDict, load_weights
 from .step import StepFunction
 
-DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
-          "f32": torch.float32}
+DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float16": torch.float16, "fp16": torch.float16,
+          "f16": torch.float16, "half": torch.float16, "float32": torch.float32, "fp32": torch.float32, "f32": torch.float32}
 
 
 def parse_dtype(name) -> torch.dtype:
     if isinstance(name, torch.dtype):
-        if name in (torch.bfloat16, torch.float32):
+        if name in (torch.bfloat16, torch.float16, torch.float32):
             return name
     elif name in DTYPES:
         return DTYPES[name]
-    raise ValueError(f"dtype {name!r}: choose bfloat16 or float32")
+    raise ValueError(f"dtype {name!r}: choose bfloat16, float16 or float32")
 
 
 @dataclass

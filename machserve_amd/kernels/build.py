@@ -23,8 +23,8 @@ CSRC = os.path.normpath(CSRC)
 ARCH = "gfx950"
 FLAGS = ["-O3", f"--offload-arch={ARCH}", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
          "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
-ELEM_DEFINE = {"bf16": "MS_ELEM_BF16", "f32": "MS_ELEM_F32"}
-CORE_SOURCES = ["runtime.hip", "gemm.hip", "skinny.hip", "elementwise.hip", "sampling.hip"]
+ELEM_DEFINE = {"bf16": "MS_ELEM_BF16", "f16": "MS_ELEM_F16", "f32": "MS_ELEM_F32"}
+CORE_SOURCES = ["errors.hip", "gemm.hip", "skinny.hip", "elementwise.hip", "sampling.hip"]
 ATTENTION_TILES = (1, 2, 3, 4, 6, 8, 12, 16)  # head-size tiles in units of 16
 
 _lock = threading.Lock()
@@ -68,8 +68,8 @@ def _sources_of(kind: str):
     if kind == "core":
         return list(CORE_SOURCES)
     if kind == "probe":  # the benchmark's measurement of the matrix cores; nothing on the product path loads it
-        return ["runtime.hip", "probe.hip"]
-    return ["runtime.hip", "attention.hip"]
+        return ["errors.hip", "probe.hip"]
+    return ["errors.hip", "attention.hip"]
 
 
 def _spec(kind: str, elem: str, nd: int | None):

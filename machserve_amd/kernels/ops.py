@@ -45,17 +45,20 @@ def _stream():
 
 
 class HipOps:
-    """Kernels of one element type: ``torch.bfloat16`` (serving) or ``torch.float32`` (true 32-bit)."""
+    """Kernels of one element type: ``torch.bfloat16`` or ``torch.float16`` (serving; the same kernels with the
+    other two-byte type, the reference's own fast precision, ``crates/mach-model/src/config.rs:3-11``) or
+    ``torch.float32`` (true 32-bit)."""
+    ELEMS = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}
 
     def __init__(self, dtype: torch.dtype, device: str = "cuda:0"):
-        if dtype not in (torch.bfloat16, torch.float32):
-            raise KernelError(f"no kernels for element type {dtype}; bfloat16 and float32 are built")
+        if dtype not in self.ELEMS:
+            raise KernelError(f"no kernels for element type {dtype}; bfloat16, float16 and float32 are built")
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible: the HIP kernels have no CPU fallback")
         self.dtype = dtype
         self.device = torch.device(device)
         self._index = self.device.index if self.device.index is not None else torch.cuda.current_device()
-        self.elem = "bf16" if dtype == torch.bfloat16 else "f32"
+        self.elem = self.ELEMS[dtype]
         self._libs: list = []
         self._core = self._load(build.ensure_library("core", self.elem))
         self._attn = {}

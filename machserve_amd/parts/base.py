@@ -105,9 +105,9 @@ class ResidualStream:
     """The 32-bit residual stream ``x [T, width]`` and what is still to be added to it.
 
     ``add_linear`` does not launch its product at once but when the stream is next read.  With
-    few rows the product leaves partial sums (``pending``) that the reading norm adds in its
-    own kernel (``normed``), which saves a pass over the stream; with many rows the product
-    adds to the stream in its epilogue.
+    few rows the product leaves partial sums (``pending``) that a reading norm may add in its
+    own kernel, which saves a pass over the stream; with many rows the product adds to the
+    stream in its epilogue.  A reader that knows nothing of this calls ``value()``.
     """
 
     def __init__(self, x: torch.Tensor, ops):
@@ -126,14 +126,15 @@ class ResidualStream:
         self.flush()
         self.x += y.to(self.x.dtype)
 
-    def _launch_deferred(self) -> None:
+    def launch_deferred(self) -> None:
+        """Launch the product that ``add_linear`` left, if any; its sum may stay pending as partial sums."""
         if self.deferred is not None:
             a, w = self.deferred
             self.deferred = None
             self.pending = self.ops.linear_residual(a, w, self.x)
 
     def flush(self) -> None:
-        self._launch_deferred()
+        self.launch_deferred()
         if self.pending is not None:
             self.ops.add_partials(self.x, self.pending)
             self.pending = None
@@ -142,66 +143,26 @@ class ResidualStream:
         self.flush()
         return self.x
 
-    def normed_linear_split(self, weight: torch.Tensor, eps: float, w: torch.Tensor) -> torch.Tensor:
-        """``rmsnorm(x) @ w.T`` as float32 ``[P, T, N]`` partial sums, the norm folded into the product
-        where the kernels take the shape."""
-        self._launch_deferred()
-        T, K = self.x.shape
-        P = 0 if self.pending is None else self.pending.shape[0]
-        if self.ops.norm_folds_into(T, w.shape[0], K, P):
-            out, x_new = self.ops.linear_split_normed(self.x, self.pending, weight, eps, w)
-            if x_new is not None:
-                self.x, self.pending = x_new, None
-            return out
-        return self.ops.linear_split(self.normed(weight, eps), w)
-
-    def normed_linear_swiglu(self, weight: torch.Tensor, eps: float, w_gate_up: torch.Tensor, intermediate: int) -> torch.Tensor:
-        """``silu(h @ gate.T) * (h @ up.T)`` for ``h = rmsnorm(x)``, the norm folded in where possible."""
-        if self.deferred is not None and self.pending is None:
-            # a product that is still to be added: where the kernels can, it leaves what the norm needs beside its
-            # sum, and the gated product applies the norm's factor to its own finished sums
-            a, w = self.deferred
-            takes = getattr(self.ops, "prenorm_swiglu_takes", None)
-            if takes is not None and takes(a.shape[0], w.shape[0], w.shape[1], w_gate_up.shape[0]):
-                self.deferred = None
-                hn, row_ss = self.ops.linear_residual_prenorm(a, w, self.x, weight)
-                return self.ops.linear_swiglu_scaled(hn, row_ss, eps, w_gate_up, intermediate)
-        self._launch_deferred()
-        T, K = self.x.shape
-        P = 0 if self.pending is None else self.pending.shape[0]
-        if self.ops.norm_folds_into(T, w_gate_up.shape[0], K, P):
-            out, x_new = self.ops.linear_swiglu_normed(self.x, self.pending, weight, eps, w_gate_up, intermediate)
-            if x_new is not None:
-                self.x, self.pending = x_new, None
-            return out
-        return self.ops.linear_swiglu(self.normed(weight, eps), w_gate_up, intermediate)
-
-    def normed(self, weight: torch.Tensor, eps: float, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """``rmsnorm(x) * weight`` of the stream with everything added (of its ``rows`` if given),
-        in the element type."""
-        self._launch_deferred()
-        h = self.ops.rmsnorm(self.x, weight, eps, rows, False, self.pending)
-        if rows is None:
-            self.pending = None  # the kernel wrote the sum back
-        return h
-
 
 class PendingNorm:
     """The normalised stream, not yet computed: a part that starts with a product over it (``takes_pending_norm``)
-    gets this instead of a tensor and lets the product's kernel apply the norm; ``tensor()`` runs
-    the norm by itself."""
+    gets this instead of a tensor, so that a norm whose kernels can do so is applied inside the product.  This base
+    form runs the norm by itself and then the plain product; a norm with fused forms of its own returns a subclass
+    from ``Norm.pending``."""
 
-    def __init__(self, stream: ResidualStream, weight: torch.Tensor, eps: float):
-        self.stream, self.weight, self.eps = stream, weight, eps
+    def __init__(self, norm: "Norm", stream: ResidualStream):
+        self.norm, self.stream = norm, stream
 
     def tensor(self) -> torch.Tensor:
-        return self.stream.normed(self.weight, self.eps)
+        return self.norm.forward(self.stream)
 
     def linear_split(self, w: torch.Tensor) -> torch.Tensor:
-        return self.stream.normed_linear_split(self.weight, self.eps, w)
+        """``norm(x) @ w.T`` as float32 ``[P, T, N]`` partial sums."""
+        return self.stream.ops.linear_split(self.tensor(), w)
 
     def linear_swiglu(self, w_gate_up: torch.Tensor, intermediate: int) -> torch.Tensor:
-        return self.stream.normed_linear_swiglu(self.weight, self.eps, w_gate_up, intermediate)
+        """``silu(h @ gate.T) * (h @ up.T)`` for ``h = norm(x)``."""
+        return self.stream.ops.linear_swiglu(self.tensor(), w_gate_up, intermediate)
 
 
 def require_kernel_sizes(rt: "Runtime", what: str, reductions=(), head_dim: Optional[int] = None) -> None:

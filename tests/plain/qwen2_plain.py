@@ -73,6 +73,11 @@ def to_bf16_and_back(x: torch.Tensor) -> torch.Tensor:
     return x.to(torch.bfloat16).to(x.dtype)
 
 
+def to_f16_and_back(x: torch.Tensor) -> torch.Tensor:
+    """What storing a value in half precision does to it (round to nearest even, crates/mach-model/src/fp16.rs:9-60)."""
+    return x.to(torch.float16).to(x.dtype)
+
+
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int | None = None, rounded=same) -> torch.Tensor:
     """Causal grouped-query attention over a whole sequence.
 

@@ -11,7 +11,7 @@ from gpu_util import DEV, assert_close
 from plain import qwen2_plain as P
 
 pytestmark = pytest.mark.gpu
-DTYPES = [torch.float32, torch.bfloat16]
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
 
 
 def ops_for(dtype):
@@ -98,7 +98,7 @@ def test_linear_many_rows_cut_along_k(dtype, M, N, K):
     ops = ops_for(dtype)
     a, w = rnd((M, K), dtype, 41), rnd((N, K), dtype, 42, K ** -0.5)
     parts = ops.linear_split(a.to(DEV), w.to(DEV))
-    assert parts.shape[1:] == (M, N) and (dtype == torch.bfloat16 or parts.shape[0] == 1)
+    assert parts.shape[1:] == (M, N) and (dtype != torch.float32 or parts.shape[0] == 1)
     assert_close(parts.sum(0), P.linear(a.double(), w.double()), torch.float32 if dtype == torch.float32 else dtype)
     assert ops.linear_split(a.to(DEV), w.to(DEV), allow_partials=False).shape[0] == 1
 
@@ -192,7 +192,7 @@ def test_residual_product_prepares_the_norm_for_the_gated_product(dtype, M, N, K
     assert_close(ss.sum(0), (xd.cpu().double() ** 2).sum(1), torch.float32, "sums of squares")
     g, u = rnd((I, N), dtype, 55, N ** -0.5 * 3), rnd((I, N), dtype, 56, N ** -0.5)
     takes = ops.prenorm_swiglu_takes(M, N, K, 2 * ((I + 15) // 16) * 16)
-    assert takes == (dtype == torch.bfloat16 and N % 64 == 0 and N >= 256 and not ops._tiled(M, N, K))
+    assert takes == (dtype != torch.float32 and N % 64 == 0 and N >= 256 and not ops._tiled(M, N, K))
     if takes:
         h = P.rms_norm(x_new.float(), nw, eps)
         ref = P.silu(P.linear(h.double(), g.double())) * P.linear(h.double(), u.double())

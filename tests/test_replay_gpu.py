@@ -17,6 +17,7 @@ LENGTHS = {"A": [5, 17, 33, 90], "B": [1, 9, 40, 100], "C": [3, 64, 130, 47]}
 
 
 BF16_ROUNDED_TOL = 1.5e-2   # against the plain model that rounds where the engine rounds (see ``check``)
+F16_TOL, F16_ROUNDED_TOL = 3e-2 / 8, 1.5e-2 / 8   # half precision has three bits of mantissa more than bfloat16
 
 
 def logit_tol(dtype, ref):
@@ -26,6 +27,8 @@ def logit_tol(dtype, ref):
     input, cache in bfloat16): 8 bits of mantissa, ~2^-8 per rounding, a few dozen roundings
     adding up like a random walk."""
     scale = ref.abs().max().item()
+    if dtype == torch.float16:
+        return F16_TOL * scale
     return (2e-5 + 2e-5 * scale) if dtype == torch.float32 else (3e-2 * scale)
 
 
@@ -55,8 +58,9 @@ class Ref:
 def plain_ref(w, sizes, prompt, dtype):
     if dtype == torch.float32:
         return Ref(P.forward(w, sizes, prompt))
-    ww = {k: v.to(torch.bfloat16).float() if v.dim() == 2 else v for k, v in w.items()}  # the matrices are stored in bfloat16
-    return Ref(P.forward(ww, sizes, prompt), P.forward(ww, sizes, prompt, rounded=P.to_bf16_and_back))
+    ww = {k: v.to(dtype).float() if v.dim() == 2 else v for k, v in w.items()}  # the matrices are stored in the element type
+    stored = P.to_bf16_and_back if dtype == torch.bfloat16 else P.to_f16_and_back
+    return Ref(P.forward(ww, sizes, prompt), P.forward(ww, sizes, prompt, rounded=stored))
 
 
 def plain_logits(models, which, dtype, i):
@@ -94,8 +98,10 @@ def check(got, ref, dtype, what):
     elif ref.rounded is not None:
         scale = ref.rounded.abs().max().item()
         err = (got - ref.rounded).abs().max().item()
-        WORST["bf16 vs rounded"] = max(WORST.get("bf16 vs rounded", 0.0), err / scale)
-        assert err <= BF16_ROUNDED_TOL * scale, f"{what}: {err:.3e} from the plain model with the engine's roundings, allowed {BF16_ROUNDED_TOL * scale:.3e}"
+        WORST[f"{dtype} vs rounded"] = max(WORST.get(f"{dtype} vs rounded", 0.0), err / scale)
+        WORST[f"{dtype} vs plain"] = max(WORST.get(f"{dtype} vs plain", 0.0), (got - ref.logits).abs().max().item() / ref.logits.abs().max().item())
+        bound = (BF16_ROUNDED_TOL if dtype == torch.bfloat16 else F16_ROUNDED_TOL) * scale
+        assert err <= bound, f"{what}: {err:.3e} from the plain model with the engine's roundings, allowed {bound:.3e}"
 
 
 def run_cuts(lm, prompt, cuts):
@@ -111,7 +117,7 @@ def run_cuts(lm, prompt, cuts):
     return torch.cat(out)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("which", ["A", "B", "C"])
 def test_whole_prompts(models, which, dtype):
     lm = engine(models, which, dtype, 16)
@@ -142,7 +148,7 @@ def changing_cuts(n):
     return out
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("which", ["A", "B", "C"])
 def test_portions_of_changing_size(models, which, dtype):
     lm = engine(models, which, dtype, 16)
@@ -151,7 +157,7 @@ def test_portions_of_changing_size(models, which, dtype):
               f"{which} prompt {i} in portions")
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("which", ["A", "B", "C"])
 def test_mixed_with_page_reuse(models, which, dtype):
     """Requests arrive one after another; every step carries a portion of the newest beside
@@ -369,7 +375,7 @@ def _four_mode_trace(prompts, page):
     return steps, wanted, peak
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("which", ["A", "B", "C"])
 def test_the_four_ways_through_the_program(models, which, dtype, tmp_path):
     """``bin/trace_run`` itself, fed the four ways of cutting as one stream of steps, with a pool of exactly the
@@ -382,7 +388,7 @@ def test_the_four_ways_through_the_program(models, which, dtype, tmp_path):
     total = sum(-(-len(p) // page) * page for p in prompts)
     assert peak < 2 * total, "the pool is far smaller than what the trace writes in all"
     root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..")
-    name = "float32" if dtype == torch.float32 else "bfloat16"
+    name = {torch.float32: "float32", torch.bfloat16: "bfloat16", torch.float16: "float16"}[dtype]
     r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", d, "--dtype", name, "--out", str(tmp_path),
                         "--max-tokens", str(peak)], input="\n".join(json.dumps(s) for s in steps) + "\n",
                        capture_output=True, text=True, timeout=600)
@@ -399,4 +405,4 @@ def test_the_four_ways_through_the_program(models, which, dtype, tmp_path):
 
 
 def test_zz_report_worst_bfloat16_error():
-    print("largest bfloat16 error against the plain model with the engine's roundings, in units of the logits' scale:", WORST)
+    print("largest errors of the reduced-precision runs, in units of the logits' scale:", WORST)
