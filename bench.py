@@ -119,10 +119,43 @@ def trace_rows(folder):
     for path in glob.glob(os.path.join(folder, "**", "*kernel_trace.csv"), recursive=True):
         with open(path, newline="") as f:
             for r in csv.DictReader(f):
-                if "ms::" in r["Kernel_Name"]:
+                if "ms::" in r["Kernel_Name"] or "_ZN2ms" in r["Kernel_Name"]:  # (some names come without being demangled)
                     rows.append((int(r["Start_Timestamp"]), int(r["End_Timestamp"]), r["Kernel_Name"]))
     rows.sort()
     return rows
+
+
+def by_name(rows, n):
+    """The dispatches ``rows[-n:]`` by kernel name: (name, calls, mean microseconds, total microseconds), longest total first."""
+    names = {}
+    for start, end, name in rows[-n:]:
+        k = names.setdefault(name, [0, 0.0])
+        k[0] += 1
+        k[1] += (end - start) / 1e3
+    return sorted(((nm, c, t / c, t) for nm, (c, t) in names.items()), key=lambda r: -r[3])
+
+
+def write_summary(path, title, command, kinds, names, n_steps):
+    """A short text summary of one traced run: what it ran, the kinds of kernels, the kernels by name."""
+    lines = [f"# {title}", "", "Command (on an MI355X, from the repository root; the summary is written by the command itself):", "",
+             f"    {command}", "",
+             "The work is run a second time under `rocprofv3 --kernel-trace`; the dispatches of the last steps are matched, in order, with",
+             "the operations one step issues.  Times are the kernels' own durations as the profiler reports them.", "",
+             "| kind of kernel | launches a step | us a step | rate | of the published peak | of what the box gives |", "|---|---|---|---|---|---|"]
+    for kind, r in kinds.items():
+        if kind == "all" or not isinstance(r, dict):
+            continue
+        rate = f"{r['rate']} {r['unit']}" if "rate" in r else ""
+        lines.append(f"| {kind} | {r['launches']} | {r['us']} | {rate} | {r.get('frac', '')} | {r.get('frac_of_measured', '')} |")
+    if isinstance(kinds.get("all"), dict):
+        a = kinds["all"]
+        lines += ["", f"All: {a['launches']} launches a step, {a['us_in_kernels']} us inside kernels, {a['us_first_to_last']} us from the first "
+                      f"kernel's start to the last one's end under the profiler (which slows the replay of a captured step)."]
+    lines += ["", f"| kernel | calls in {n_steps} step{'s' if n_steps != 1 else ''} | mean us | total us |", "|---|---|---|---|"]
+    for nm, c, mean, total in names[:14]:
+        lines.append(f"| `{nm[:110]}` | {c} | {mean:.2f} | {total:.1f} |")
+    with open(path, "w") as f:
+        f.write("\n".join(lines) + "\n")
 
 
 def account(calls, rows, n_steps, peak_of, measured_of, extra):
@@ -219,6 +252,8 @@ def main() -> int:
     ap.add_argument("--sync-steps", action="store_true", help="wait for each decode step's tokens before the next is launched")
     ap.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for profiles)")
     ap.add_argument("--prefill-tokens", type=int, default=None, help="tokens of the prefill (default: the context)")
+    ap.add_argument("--profile-out", default=None, help="folder that receives a summary of the traced runs, one text file for the decode "
+                    "step and one for the prefill (kinds of kernels, and the kernels by name)")
     ap.add_argument("--record-calls", default=None, help=argparse.SUPPRESS)  # file that receives one step's operations (the traced run)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -456,11 +491,21 @@ def kernels_by_kind(args, cfg, dt, peaks, ctx, prefill_tokens):
                 peak_of = {"products": "GB/s", "head": "GB/s", "attention": "GB/s"}
                 extra = {"attention": (args.batch * mean_ctx * nums["kv_bytes_per_token"], 0)}
                 out[kind] = account(calls, rows, args.steps, peak_of, measured, extra)
+                n_steps, title = args.steps, f"decode step, batch {args.batch}, {ctx}-token contexts"
             else:
                 T = prefill_tokens
                 peak_of = {"products": "TFLOP/s", "attention": "TFLOP/s", "head": "GB/s", "flops_peak": PEAK_FLOPS[args.dtype]}
                 extra = {"attention": (0, cfg.num_hidden_layers * 4.0 * cfg.num_attention_heads * cfg.head_dim * (T * (T + 1) / 2))}
                 out[kind] = account(calls, rows, 1, peak_of, measured, extra)
+                n_steps, title = 1, f"prefill of one {T}-token prompt in one step"
+            if args.profile_out and "all" in out[kind]:
+                os.makedirs(args.profile_out, exist_ok=True)
+                shape = SHAPES[args.shape][0]
+                name = (f"decode_b{args.batch}" + (f"_ctx{ctx}" if ctx != 2048 else "") if kind == "decode" else f"prefill_{T}")
+                name += ("" if args.shape == "0.5b" else "_" + args.shape) + ("" if args.dtype == "bf16" else "_" + args.dtype)
+                command = "python bench.py " + " ".join(a for a in sys.argv[1:])
+                write_summary(os.path.join(args.profile_out, name + ".md"), f"{title} ({shape} shape, {args.dtype}, random weights)", command,
+                              out[kind], by_name(rows, n_steps * out[kind]["all"]["launches"]), n_steps)
     return out
 
 
