@@ -412,7 +412,14 @@ struct SkinnyPlan { int wn, ksi, ksb, k_per_wave; };
 // Columns per wave in units of 16: with more than 32 rows and enough columns to keep every CU busy,
 // a wave takes 64 columns, so that the rows it re-reads (from L2, they are shared by all waves)
 // weigh no more than the weights it streams.
-static int skinny_nt(int M, int N) { return (kHalf && M > 32 && N >= 4096) ? 4 : 2; }  // 32-bit fragments are twice as large
+// Under at most 32 rows and a narrow output a wave takes 16 columns only: a CU that streams a weight alone gets
+// little more than its share of the chip's rate, so a small weight wants as many blocks as it can be cut into
+// (`pairs`: the gated product needs gate and up tiles side by side).
+static int skinny_nt(int M, int N, bool pairs = false) {
+    if (kHalf && M > 32 && N >= 4096) return 4;  // 32-bit fragments are twice as large
+    if (!pairs && M <= 32 && N <= 2048) return 1;
+    return 2;
+}
 
 #ifdef MS_MEASURE  // switches for measurements, in no library that serves
 static int g_force_ksi = 0;  // waves along K inside a block (1 = four column waves)
@@ -421,8 +428,8 @@ static int g_max_ksb = 0;    // most blocks along K
 static constexpr int g_force_ksi = 0, g_max_ksb = 0;
 #endif
 
-static SkinnyPlan plan_skinny(int M, int N, int K, bool allow_partials) {
-    const int NT = skinny_nt(M, N);
+static SkinnyPlan plan_skinny(int M, int N, int K, bool allow_partials, bool pairs = false) {
+    const int NT = skinny_nt(M, N, pairs);
     const int col_waves = ceil_div(N, 16 * NT);
     const int slices = ceil_div(K, KSTEP);  // slices of 128 along K: one wave iteration each
     int want = max(1, min(ceil_div(4096, col_waves), slices));  // waves wanted along K
@@ -460,6 +467,12 @@ template <int EPI>
 static int launch_skinny(const SkinnyArgs& a, const SkinnyPlan& p, hipStream_t stream) {
     MS_REQUIRE(a.M > 0 && a.M <= 64, "skinny product: M=%d must be in 1..64", a.M);
     MS_REQUIRE(a.K % 8 == 0, "skinny product: the reduction size K=%d must be a multiple of 8", a.K);
+    if constexpr (EPI != SK_SWIGLU) {
+        if (skinny_nt(a.M, a.N) == 1) {
+            if (a.M <= 16) return launch_skinny_mt<1, 1, EPI>(a, p, stream);
+            return launch_skinny_mt<2, 1, EPI>(a, p, stream);
+        }
+    }
     if (a.M <= 16) return launch_skinny_mt<1, 2, EPI>(a, p, stream);
     if (a.M <= 32) return launch_skinny_mt<2, 2, EPI>(a, p, stream);
     if constexpr (kHalf) {
@@ -537,7 +550,7 @@ extern "C" int ms_linear_skinny(const void* a, const void* w, float* out, int M,
 extern "C" int ms_linear_swiglu_skinny(const void* a, const void* w, void* out, int M, int I, int K, hipStream_t stream) {
     const int n = 2 * ceil_div(I, 16) * 16;
     SkinnyArgs args{(const elem_t*)a, (const elem_t*)w, out, M, n, K, 0, I};
-    return launch_skinny<SK_SWIGLU>(args, plan_skinny(M, n, K, false), stream);
+    return launch_skinny<SK_SWIGLU>(args, plan_skinny(M, n, K, false, true), stream);
 }
 
 // Whether ms_linear_norm_skinny / ms_linear_swiglu_norm_skinny should be given this shape.
@@ -579,7 +592,7 @@ extern "C" int ms_linear_residual_skinny(const void* a, const void* w, float* x,
 extern "C" int ms_skinny_prenorm_parts(int M, int N, int K) {
     if (M < 1 || M > 32 || K % 8) return 0;
     const SkinnyPlan p = plan_skinny(M, N, K, true);
-    return p.ksb == 1 ? ceil_div(N, 32) : 0;
+    return p.ksb == 1 ? ceil_div(N, 16 * skinny_nt(M, N)) : 0;
 }
 
 // x[M, N] += a w^T as ms_linear_residual_skinny does, and beside it hn[M, N] = x * norm_w in the element type and
@@ -590,6 +603,10 @@ extern "C" int ms_linear_residual_prenorm_skinny(const void* a, const void* w, f
     MS_REQUIRE(norm_w && hn && ss_part, "few-rows product that prepares the norm: its outputs are missing");
     const SkinnyPlan p = plan_skinny(M, N, K, true);
     SkinnyArgs args{(const elem_t*)a, (const elem_t*)w, x, M, N, K, 0, 0, norm_w, (elem_t*)hn, ss_part};
+    if (skinny_nt(M, N) == 1) {
+        if (M <= 16) return launch_skinny_mt<1, 1, SK_RESIDUAL_PRENORM>(args, p, stream);
+        return launch_skinny_mt<2, 1, SK_RESIDUAL_PRENORM>(args, p, stream);
+    }
     if (M <= 16) return launch_skinny_mt<1, 2, SK_RESIDUAL_PRENORM>(args, p, stream);
     return launch_skinny_mt<2, 2, SK_RESIDUAL_PRENORM>(args, p, stream);
 }
