@@ -476,7 +476,7 @@ def kernels_by_kind(args, cfg, dt, peaks, ctx, prefill_tokens):
             if kind == "prefill":
                 cmd += ["--prefill-only", "--prefill-tokens", str(prefill_tokens)]
             try:
-                r = subprocess.run(cmd, capture_output=True, text=True, timeout=420, cwd=tmp, env=env)
+                r = subprocess.run(cmd, capture_output=True, text=True, timeout=150, cwd=tmp, env=env)
                 if r.returncode != 0 or not os.path.exists(calls_file):
                     out[kind] = {"error": f"the traced run ended with {r.returncode}: {r.stderr[-300:]}"}
                     continue
