@@ -538,7 +538,7 @@ struct DecodeTile {
 
 template <bool FUSED>
 __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
-    __shared__ float sm_o[3][HDT][16];  // also the staging area of the fused prologue: (g + 2) * hd floats
+    __shared__ __align__(32) float sm_o[3][HDT][16];  // also the staging area of the fused prologue: (g + 2) * hd sums and g * hd elements
     __shared__ float sm_m[3][16], sm_l[3][16];
     __shared__ float cs[HDT / 2], sn[HDT / 2], knew[HDT], vnew[HDT];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -628,6 +628,37 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
             }
         }
     };
+    // The fused prologue stages this KV head's share of the step's row: its g query heads, its key, its
+    // value, (g + 2) * hd columns, four per thread at a time.  What the first four need from memory
+    // (the bias and the first two partial sums) is asked for here, before anything else: nothing of it
+    // depends on the row's position, and the row's query is what the block waits for in the end.
+    const int width = FUSED ? (g + 2) * hd : 0;
+    const size_t pstride = FUSED ? (size_t)gridDim.x * a.stride : 0;
+    const float* row0 = FUSED ? a.qkv + (size_t)s * a.stride : nullptr;
+    const float* bias = FUSED && a.bias ? a.bias : row0;  // without a bias: finite values, times zero
+    const float bias_on = FUSED && a.bias ? 1.f : 0.f;
+    auto column = [&](int c) {
+        c = min(c, width - 1);
+        const int qcol = kvh * g * hd, kcol = a.H * hd + kvh * hd, vcol = (a.H + a.KV) * hd + kvh * hd;
+        return c < g * hd ? qcol + c : (c < (g + 1) * hd ? kcol + c - g * hd : vcol + c - (g + 1) * hd);
+    };
+    int col_e[4];
+    float bias_e[4], part_e[2][4], freq_e = 0.f;
+    int slot = -1;
+    if constexpr (FUSED) {
+        const size_t p1 = (size_t)min(1, a.n_partials - 1) * pstride;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            col_e[u] = column(tid + u * 256);
+            bias_e[u] = bias[col_e[u]];
+            part_e[0][u] = row0[col_e[u]];
+            part_e[1][u] = row0[p1 + col_e[u]];
+        }
+        freq_e = (a.inv_freq ? a.inv_freq : row0)[min(tid, hd / 2 - 1)];
+        slot = a.slot_map[s];
+        __builtin_amdgcn_sched_barrier(0);  // the loads stay up here
+    }
+
     // The first tile depends on nothing the prologue computes: it is requested before the prologue
     // so that its latency hides behind it.
     DecodeTile next;
@@ -638,94 +669,98 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
     Frag qf[NKS];
     if constexpr (FUSED) {
         const int half = hd / 2;
-        const size_t pstride = (size_t)gridDim.x * a.stride;
-        const float* row0 = a.qkv + (size_t)s * a.stride;
-        // stage this KV head's share of the row: its g query heads, its key, its value
-        float* rowv = &sm_o[0][0][0];
-        const int qcol = kvh * g * hd, kcol = a.H * hd + kvh * hd, vcol = (a.H + a.KV) * hd + kvh * hd;
-        // four columns per thread at a time, all of their loads asked for before the first is used
-        const float* bias = a.bias ? a.bias : row0;  // without a bias: finite values, times zero
-        const float bias_on = a.bias ? 1.f : 0.f;
-        const int width = (g + 2) * hd;
-        for (int c0 = tid; c0 < width; c0 += 4 * 256) {
+        float* rowv = &sm_o[0][0][0];                                   // (g + 2) * hd sums, then ...
+        elem_t* qrot = reinterpret_cast<elem_t*>(rowv + (g + 2) * hd);  // ... the g rotated queries, rounded
+        // the angles, while the sums are on their way
+        if (tid < half) {
+            float c = 1.f, sv = 0.f;
+            if (a.inv_freq) sincosf((float)pos * freq_e, &sv, &c);
+            cs[tid] = c;
+            sn[tid] = sv;
+        }
+        // Further partial sums, eight at a time, all of their loads asked for before the first is added: the
+        // sums were written by the kernel before this one, and one load after the other would be as many trips
+        // to them (beyond the last partial sum: the last one again, not added).
+        auto add_partials = [&](int first, const int (&col)[4], float (&v)[4]) {
+            constexpr int NB = 8;
+            for (int p0 = first; p0 < a.n_partials; p0 += NB) {
+                float t[NB][4];
+#pragma unroll
+                for (int q = 0; q < NB; ++q) {
+                    const size_t po = (size_t)min(p0 + q, a.n_partials - 1) * pstride;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) t[q][u] = row0[po + col[u]];
+                }
+#pragma unroll
+                for (int q = 0; q < NB; ++q)
+                    if (p0 + q < a.n_partials) {
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) v[u] += t[q][u];
+                    }
+            }
+        };
+        {
+            float v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = bias_e[u] * bias_on + part_e[0][u] + (a.n_partials > 1 ? part_e[1][u] : 0.f);
+            add_partials(2, col_e, v);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (tid + u * 256 < width) rowv[tid + u * 256] = v[u];
+        }
+        for (int c0 = tid + 4 * 256; c0 < width; c0 += 4 * 256) {  // more than 1,024 columns: many large heads
             int col[4];
             float v[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                const int c = min(c0 + u * 256, width - 1);
-                col[u] = c < g * hd ? qcol + c : (c < (g + 1) * hd ? kcol + c - g * hd : vcol + c - (g + 1) * hd);
+                col[u] = column(c0 + u * 256);
                 v[u] = bias[col[u]] * bias_on;
             }
-            // Several partial sums at a time, all of their loads asked for before the first is added: the sums
-            // were written by the kernel before this one, and one load after the other would be as many trips
-            // to them (beyond the last partial sum: the last one again, not added).  Two at a time when there
-            // are no more (a few-rows projection), eight otherwise (a projection cut along K).
-            auto add_partials = [&](auto batch) {
-                constexpr int NB = decltype(batch)::value;
-                for (int p0 = 0; p0 < a.n_partials; p0 += NB) {
-                    float t[NB][4];
-#pragma unroll
-                    for (int q = 0; q < NB; ++q) {
-                        const size_t po = (size_t)min(p0 + q, a.n_partials - 1) * pstride;
-#pragma unroll
-                        for (int u = 0; u < 4; ++u) t[q][u] = row0[po + col[u]];
-                    }
-#pragma unroll
-                    for (int q = 0; q < NB; ++q)
-                        if (p0 + q < a.n_partials) {
-#pragma unroll
-                            for (int u = 0; u < 4; ++u) v[u] += t[q][u];
-                        }
-                }
-            };
-            if (a.n_partials <= 2) add_partials(std::integral_constant<int, 2>{});
-            else add_partials(std::integral_constant<int, 8>{});
+            add_partials(0, col, v);
 #pragma unroll
             for (int u = 0; u < 4; ++u)
                 if (c0 + u * 256 < width) rowv[c0 + u * 256] = v[u];
         }
-        if (tid < half) {
-            float c = 1.f, sv = 0.f;
-            if (a.inv_freq) sincosf((float)pos * a.inv_freq[tid], &sv, &c);
-            cs[tid] = c;
-            sn[tid] = sv;
-        }
         __syncthreads();
-        // the row's own key (rotated) and value, rounded as the page holds them
+        // Rotation, one pair (d, d + hd / 2) of a query head or of the key per thread at a time; the row's
+        // own key and value are rounded as the page holds them, and one block writes them there (nobody
+        // reads them in this launch).
         {
-            const float* kv_ = rowv + g * hd;
-            const float* vv_ = rowv + (g + 1) * hd;
-            const int slot = a.slot_map[s];
-            const int page = slot / ps, off = slot % ps;
-            for (int d = tid; d < hd; d += 256) {
-                const int j = d < half ? d : d - half;
-                const float x0 = kv_[j], x1 = kv_[j + half];
-                const elem_t ke = from_f32<elem_t>(d < half ? x0 * cs[j] - x1 * sn[j] : x0 * sn[j] + x1 * cs[j]);
-                const elem_t ve = from_f32<elem_t>(vv_[d]);
-                knew[d] = to_f32(ke);
-                vnew[d] = to_f32(ve);
-                if (sp == 0 && slot >= 0) {  // one block writes the page; nobody reads it in this launch
-                    const_cast<elem_t*>(a.kpool)[(((size_t)page * a.KV + kvh) * ps + off) * hd + d] = ke;
-                    const_cast<elem_t*>(a.vpool)[(((size_t)page * a.KV + kvh) * hd + d) * ps + off] = ve;
+            const int page = slot >= 0 ? slot / ps : 0, off = slot >= 0 ? slot % ps : 0;
+            const bool writes = sp == 0 && slot >= 0;
+            elem_t* kdst = const_cast<elem_t*>(a.kpool) + (((size_t)page * a.KV + kvh) * ps + off) * hd;
+            elem_t* vdst = const_cast<elem_t*>(a.vpool) + ((size_t)page * a.KV + kvh) * hd * ps + off;
+            const float inv_half = 1.0f / (float)half;
+            for (int i = tid; i < (g + 1) * half; i += 256) {
+                const int row = (int)(((float)i + 0.5f) * inv_half), j = i - row * half;  // i < 17 * 128: exact
+                const float x0 = rowv[row * hd + j], x1 = rowv[row * hd + j + half];
+                const elem_t r0 = from_f32<elem_t>(x0 * cs[j] - x1 * sn[j]), r1 = from_f32<elem_t>(x0 * sn[j] + x1 * cs[j]);
+                if (row < g) {
+                    qrot[row * hd + j] = r0;
+                    qrot[row * hd + j + half] = r1;
+                } else {
+                    knew[j] = to_f32(r0);
+                    knew[j + half] = to_f32(r1);
+                    if (writes) {
+                        kdst[j] = r0;
+                        kdst[j + half] = r1;
+                    }
                 }
             }
+            const float* vv_ = rowv + (g + 1) * hd;
+            for (int d = tid; d < hd; d += 256) {
+                const elem_t ve = from_f32<elem_t>(vv_[d]);
+                vnew[d] = to_f32(ve);
+                if (writes) vdst[(size_t)d * ps] = ve;
+            }
         }
+        __syncthreads();
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
             const int d0 = ks * 32 + grp * 8;
-            if (valid && d0 < hd) {
-                const float* qh = rowv + r16 * hd;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int d = d0 + e, j = d < half ? d : d - half;
-                    const float x0 = qh[j], x1 = qh[j + half];
-                    qf[ks].v[e] = from_f32<elem_t>(d < half ? x0 * cs[j] - x1 * sn[j] : x0 * sn[j] + x1 * cs[j]);
-                }
-            } else {
-                qf[ks] = frag_zero();
-            }
+            qf[ks] = (valid && d0 < hd) ? frag_load(qrot + r16 * hd + d0) : frag_zero();
         }
-        __syncthreads();  // knew / vnew are complete, and the staging area is free again
+        __syncthreads();  // the staging area is free again: the waves hand their results over through it
     } else {
         const elem_t* qrow = a.q + ((size_t)s * a.H + head) * hd;
 #pragma unroll
