@@ -34,6 +34,11 @@ struct SkinnyArgs {
     const float* norm_w;  // [N]
     elem_t* hn;           // [M, N]: (stream + product) * norm_w, not yet divided by the root mean square
     float* ss_part;       // [column waves, M]: each column wave's share of the rows' sums of squares
+    // SK_SWIGLU of rows that came in multiplied by a norm's weight only (at most 16 rows): both products of a
+    // row are multiplied by 1 / sqrt(sum over parts of row_ss[part, row] / K + ss_eps) before the activation
+    const float* row_ss;  // [ss_parts, M] or null
+    int ss_parts;
+    float ss_eps;
 };
 
 __device__ __forceinline__ float silu_sk(float g) {
@@ -44,8 +49,15 @@ __device__ __forceinline__ float silu_sk(float g) {
 #endif
 }
 
+// A block of eight waves puts two on every SIMD; with more than 128 registers a wave a CU then holds one
+// block, and a grid of more blocks than CUs (the gated product: 304 for 9,728 columns) runs in two rounds
+// although every block only waits for its one trip to memory.  One row tile under at most 32 columns a wave
+// fits 128 registers where nothing of the residual stream is held beside the sums: two blocks a CU.
 template <int MT, int NT, int WN, int KSI, int EPI>
-__global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a) {
+constexpr int skinny_waves_per_simd() { return (WN * KSI == 8 && MT == 1 && NT <= 2 && EPI <= SK_SWIGLU) ? 4 : 1; }
+
+template <int MT, int NT, int WN, int KSI, int EPI>
+__global__ __launch_bounds__(64 * WN * KSI, (skinny_waves_per_simd<MT, NT, WN, KSI, EPI>())) void gemm_skinny_kernel(SkinnyArgs a) {
     __shared__ float red[(KSI > 1 ? (KSI - 1) : 1) * WN * NT * 4 * 64];  // one row tile of every slice at a time
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wn = wave % WN, wk = wave / WN;
@@ -59,6 +71,22 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
     for (int i = 0; i < MT; ++i)
 #pragma unroll
         for (int j = 0; j < NT; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    // SK_SWIGLU with row factors: the rows' sums of squares come in parts (written by the kernel before this
+    // one).  The block's waves share them out: lane (row, q) of wave w adds parts 4 w + q, 4 w + q + 4 W, ...
+    // (W waves), the first two of them asked for here with everything else; the four q of a row are added by
+    // shuffles, the waves' shares through LDS in wave order.  The order depends on the number of parts only.
+    constexpr bool FACTORS = EPI == SK_SWIGLU && MT == 1;
+    __shared__ float ss_red[FACTORS ? WN * KSI : 1][16];
+    float ss_early[2] = {0.f, 0.f};
+    if constexpr (FACTORS) {
+        if (a.row_ss) {
+            const int share = wave * 4 + grp, row = min(r16, a.M - 1);
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+                ss_early[u] = a.row_ss[(size_t)min(share + u * 4 * WN * KSI, a.ss_parts - 1) * a.M + row];
+        }
+    }
 
     // SK_RESIDUAL: the stream's values are asked for now, with everything else, not after the sums
     constexpr bool ADDS = EPI == SK_RESIDUAL || EPI == SK_RESIDUAL_PRENORM;
@@ -153,6 +181,18 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
         }
     }
 
+    if constexpr (FACTORS) {
+        if (a.row_ss) {
+            constexpr int W = WN * KSI;
+            const int share = wave * 4 + grp, row = min(r16, a.M - 1);
+            float sq = (share < a.ss_parts ? ss_early[0] : 0.f) + (share + 4 * W < a.ss_parts ? ss_early[1] : 0.f);
+            for (int p = share + 8 * W; p < a.ss_parts; p += 4 * W) sq += a.row_ss[(size_t)p * a.M + row];  // a very wide stream
+            sq += __shfl_xor(sq, 16, WAVE);
+            sq += __shfl_xor(sq, 32, WAVE);
+            if (grp == 0) ss_red[wave][r16] = sq;
+            if constexpr (KSI == 1) __syncthreads();  // with slices of K the barrier of their sum serves
+        }
+    }
     // sum the K slices of the block in slice order: slice 0 keeps its sums and adds 1, 2, ...;
     // one 16-row tile per round keeps the LDS buffer small
     if constexpr (KSI > 1) {
@@ -185,6 +225,18 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
         static_assert(NT % 2 == 0, "gate and up tiles come in pairs");
         if (!owner) return;
         elem_t* out = reinterpret_cast<elem_t*>(a.out);
+        float f[4] = {1.f, 1.f, 1.f, 1.f};  // of the rows this lane holds
+        if constexpr (FACTORS) {
+            if (a.row_ss) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float sq = 0.f;
+#pragma unroll
+                    for (int w = 0; w < WN * KSI; ++w) sq += ss_red[w][grp * 4 + e];
+                    f[e] = 1.0f / sqrtf(sq / (float)a.K + a.ss_eps);
+                }
+            }
+        }
 #pragma unroll
         for (int i = 0; i < MT; ++i)
 #pragma unroll
@@ -194,7 +246,7 @@ __global__ __launch_bounds__(64 * WN * KSI) void gemm_skinny_kernel(SkinnyArgs a
                 for (int e = 0; e < 4; ++e) {
                     const int row = i * 16 + grp * 4 + e;
                     if (row < a.M && col < a.n_out)
-                        out[(size_t)row * a.n_out + col] = from_f32<elem_t>(silu_sk(acc[i][j][e]) * acc[i][j + 1][e]);
+                        out[(size_t)row * a.n_out + col] = from_f32<elem_t>(silu_sk(acc[i][j][e] * f[e]) * (acc[i][j + 1][e] * f[e]));
                 }
             }
     } else if constexpr (EPI == SK_RESIDUAL_PRENORM) {
@@ -550,6 +602,29 @@ extern "C" int ms_linear_skinny(const void* a, const void* w, float* out, int M,
 extern "C" int ms_linear_swiglu_skinny(const void* a, const void* w, void* out, int M, int I, int K, hipStream_t stream) {
     const int n = 2 * ceil_div(I, 16) * 16;
     SkinnyArgs args{(const elem_t*)a, (const elem_t*)w, out, M, n, K, 0, I};
+    return launch_skinny<SK_SWIGLU>(args, plan_skinny(M, n, K, false, true), stream);
+}
+
+// Whether ms_linear_swiglu_scaled_skinny takes this shape, and is the faster of the two forms for it: one
+// tile of rows, and so few waves that all of them are on the chip at once (sixteen a CU), each
+// waiting for its one trip to memory.  (0.5B gate/up, 304 blocks: 9.9 us tiled with three K steps in flight,
+// which multiplies 64-row tiles of padding and ends in a long epilogue; the walk over K there is bound by
+// its own instructions, not by memory.)
+extern "C" int ms_swiglu_scaled_skinny_takes(int M, int I, int K) {
+    if (!kHalf || M < 1 || M > 16 || K % 8) return 0;
+    const int n = 2 * ceil_div(I, 16) * 16;
+    const SkinnyPlan p = plan_skinny(M, n, K, false, true);
+    return ceil_div(n, 32 * p.wn) * p.wn * p.ksi <= 4096;  // sixteen waves a CU
+}
+
+// ms_linear_swiglu_skinny for rows that came in multiplied by a norm's weight only: both products of a row are
+// divided by the row's root mean square, 1 / sqrt(sum_p row_ss[p, row] / K + eps), before the activation.
+extern "C" int ms_linear_swiglu_scaled_skinny(const void* a, const float* row_ss, int ss_parts, float eps, const void* w, void* out,
+                                              int M, int I, int K, hipStream_t stream) {
+    MS_REQUIRE(ms_swiglu_scaled_skinny_takes(M, I, K), "few-rows gated product with row factors: M=%d I=%d K=%d is not taken", M, I, K);
+    MS_REQUIRE(row_ss && ss_parts >= 1, "few-rows gated product with row factors: the rows' sums of squares are missing");
+    const int n = 2 * ceil_div(I, 16) * 16;
+    SkinnyArgs args{(const elem_t*)a, (const elem_t*)w, out, M, n, K, 0, I, nullptr, nullptr, nullptr, row_ss, ss_parts, eps};
     return launch_skinny<SK_SWIGLU>(args, plan_skinny(M, n, K, false, true), stream);
 }
 

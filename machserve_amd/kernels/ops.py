@@ -258,7 +258,8 @@ class HipOps:
         first leaves ``x * norm_w`` and the rows' sums of squares beside the sum, the second divides its
         finished sums by the root mean square (:meth:`linear_residual_prenorm`, :meth:`linear_swiglu_scaled`)."""
         return (not self._tiled(M, N, K) and self._plan("ms_skinny_prenorm_parts", M, N, K) > 0
-                and bool(self._plan("ms_swiglu_scaled_takes", M, n_gate_up // 2, N)))
+                and bool(self._plan("ms_swiglu_scaled_takes", M, n_gate_up // 2, N)
+                         or self._plan("ms_swiglu_scaled_skinny_takes", M, n_gate_up // 2, N)))
 
     def linear_residual_prenorm(self, a: torch.Tensor, w: torch.Tensor, x: torch.Tensor, norm_w: torch.Tensor):
         """``x += a @ w.T`` in place; returns ``(x * norm_w`` in the element type, float32 ``[parts, M]`` whose sum
@@ -284,9 +285,10 @@ class HipOps:
             raise KernelError(f"linear_swiglu_scaled: interleaved weight has {N} rows for intermediate size {intermediate}")
         self._want(row_ss, torch.float32, "linear_swiglu_scaled sums of squares", row_ss.shape[0], M)
         out = torch.empty((M, intermediate), dtype=self.dtype, device=hn.device)
-        self._check(self._core, self._core.ms_linear_swiglu_scaled(
-            _ptr(hn), _ptr(row_ss), _c_int(row_ss.shape[0]), _c_float(eps), _ptr(w_gate_up), _ptr(out), _c_int(M),
-            _c_int(intermediate), _c_int(K), self._stream()))
+        few_rows = bool(self._plan("ms_swiglu_scaled_skinny_takes", M, intermediate, K))
+        fn = self._core.ms_linear_swiglu_scaled_skinny if few_rows else self._core.ms_linear_swiglu_scaled
+        self._check(self._core, fn(_ptr(hn), _ptr(row_ss), _c_int(row_ss.shape[0]), _c_float(eps), _ptr(w_gate_up), _ptr(out),
+                                   _c_int(M), _c_int(intermediate), _c_int(K), self._stream()))
         return out
 
     def linear_swiglu(self, a: torch.Tensor, w_gate_up: torch.Tensor, intermediate: int) -> torch.Tensor:

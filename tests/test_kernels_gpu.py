@@ -172,7 +172,8 @@ def test_products_with_the_norm_folded_in(dtype, M, N, K, NP):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K,I", [(8, 896, 896, 4864), (1, 896, 896, 4864), (20, 320, 264, 203), (32, 256, 128, 100),
-                                     (5, 1000, 200, 50), (16, 1536, 904, 120)])
+                                     (5, 1000, 200, 50), (16, 1536, 904, 120), (3, 64, 72, 65536), (13, 2048, 136, 40),
+                                     (17, 896, 896, 4864)])
 def test_residual_product_prepares_the_norm_for_the_gated_product(dtype, M, N, K, I):
     """x += a w^T leaves x * norm_w and the rows' sums of squares beside the sum; the gated product of those rows
     divides its finished sums by the root mean square: together rmsnorm(x + a w^T) through gate and up."""
@@ -192,7 +193,8 @@ def test_residual_product_prepares_the_norm_for_the_gated_product(dtype, M, N, K
     assert_close(ss.sum(0), (xd.cpu().double() ** 2).sum(1), torch.float32, "sums of squares")
     g, u = rnd((I, N), dtype, 55, N ** -0.5 * 3), rnd((I, N), dtype, 56, N ** -0.5)
     takes = ops.prenorm_swiglu_takes(M, N, K, 2 * ((I + 15) // 16) * 16)
-    assert takes == (dtype != torch.float32 and N % 64 == 0 and N >= 256 and not ops._tiled(M, N, K))
+    # the tiled form wants whole K steps of 64; at most 16 rows go to the few-rows form, which takes any K
+    assert takes == (dtype != torch.float32 and ((N % 64 == 0 and N >= 256) or M <= 16) and not ops._tiled(M, N, K))
     if takes:
         h = P.rms_norm(x_new.float(), nw, eps)
         ref = P.silu(P.linear(h.double(), g.double())) * P.linear(h.double(), u.double())
