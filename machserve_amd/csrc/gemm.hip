@@ -558,8 +558,9 @@ extern "C" int ms_prefers_tiled(int M, int N, int K) {
     }
     if (N >= 1024) {
         // a projection of the width (q/k/v, output): from 16 rows, or 8 if it is not small (batch 32: 1.40 ->
-        // 1.36 ms a step; 0.5B q/k/v at 8 rows is faster in the few-rows kernel)
-        return M >= 16 || (M >= 8 && nk >= 2e6);
+        // 1.36 ms a step; 0.5B q/k/v at 8 rows is faster in the few-rows kernel); a large weight (the 1.5B down
+        // projection: 27 MB) from one row on (1.5B decode step at batch 1 and 4: 1.5 % shorter)
+        return M >= 16 || (M >= 8 && nk >= 2e6) || nk >= 10e6;
     }
     // a narrow output with a long K (a down projection): the tiled kernel cuts K over many blocks
     return M >= 32 && K >= 4096;
