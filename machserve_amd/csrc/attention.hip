@@ -538,6 +538,8 @@ struct DecodeTile {
 
 template <bool FUSED>
 __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
+    arguments_now(a.q, a.kpool, a.vpool, a.out, a.part_o, a.part_ml, a.block_table, a.seq_pos0, a.table_stride, a.H, a.KV, a.hd,
+                  a.ps, a.window, a.nsplit, a.scale, a.qkv, a.bias, a.inv_freq, a.slot_map, a.n_partials, a.stride);
     __shared__ __align__(32) float sm_o[3][HDT][16];  // also the staging area of the fused prologue: (g + 2) * hd sums and g * hd elements
     __shared__ float sm_m[3][16], sm_l[3][16];
     __shared__ float cs[HDT / 2], sn[HDT / 2], knew[HDT], vnew[HDT];
@@ -934,6 +936,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
 // is computed from those, so that the kernel waits for memory once.
 __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                           elem_t* __restrict__ out, int hd, int nsplit) {
+    arguments_now(part_o, part_ml, out, hd, nsplit);
     constexpr int BATCH = 8;
     const size_t row = blockIdx.x;  // (request, head)
     const int lane = threadIdx.x;

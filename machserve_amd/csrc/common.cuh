@@ -121,6 +121,19 @@ __device__ __forceinline__ uint32_t opaque(uint32_t x) {
     return x;
 }
 
+// A kernel's arguments are read through the scalar cache, which is empty when the kernel starts: every read is a
+// trip to memory (about 0.4 us), and the compiler asks for an argument only where it is first needed, behind
+// the branches and the waits that come before: one trip after the other (four in the fused decode attention).
+// Naming the arguments here, first thing in a kernel, makes one request of them all.
+template <typename T>
+__device__ __forceinline__ void argument_now(T v) {
+    asm volatile("" ::"s"(v));
+}
+template <typename... T>
+__device__ __forceinline__ void arguments_now(T... v) {
+    (argument_now(v), ...);
+}
+
 // ---- reductions -----------------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -11,6 +11,7 @@ namespace ms {
 // x[t, :] = float(table[tokens[t], :]) * scale
 __global__ __launch_bounds__(256) void embed_kernel(const int* __restrict__ tokens, const elem_t* __restrict__ table,
                                                     float* __restrict__ x, int d, float scale) {
+    arguments_now(tokens, table, x, d, scale);
     const int t = blockIdx.x;
     const elem_t* src = table + (size_t)tokens[t] * d;
     float* dst = x + (size_t)t * d;
@@ -56,6 +57,7 @@ __global__ __launch_bounds__(256) void rmsnorm_wide_kernel(float* __restrict__ x
                                                            size_t partial_stride, const int* __restrict__ rows,
                                                            const float* __restrict__ w, OutT* __restrict__ out, int d,
                                                            float eps, int n_more) {
+    arguments_now(x, partials, partial_stride, rows, w, out, d, eps, n_more);
     __shared__ float scratch[4];
     const int i = blockIdx.x, ng = d / 4;
     const size_t r = rows ? rows[i] : i;

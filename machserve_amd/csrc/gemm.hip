@@ -58,6 +58,8 @@ template <int BM, int BN, int WM, int WN, int BK, int EPI, int STAGES = 2, bool 
 __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A, const elem_t* __restrict__ W,
                                                    int M, int N, int K, EpiArgs ep) {
     static_assert(WM * WN == 4, "four waves");
+    arguments_now(A, W, M, N, K, ep.out, ep.bias, ep.ldo, ep.n_out, ep.k_per_split, ep.split_stride);
+    if constexpr (SCALED) arguments_now(ep.row_ss, ep.ss_parts, ep.ss_eps);
     static_assert(BK % 32 == 0, "K step in MFMA steps of 32");
 #ifdef MS_ELEM_HALF
     constexpr bool DIRECT = BK == 64;

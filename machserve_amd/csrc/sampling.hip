@@ -45,6 +45,7 @@ constexpr int ARGMAX_CHUNKS = 64;
 // a block writes the maximum of its chunk and the smallest index that holds it.
 __global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ logits, int vocab,
                                                              float* __restrict__ part_val, int* __restrict__ part_idx) {
+    arguments_now(logits, vocab, part_val, part_idx);
     __shared__ float s_v[4];
     __shared__ int s_i[4];
     const int r = blockIdx.x, ch = blockIdx.y, tid = threadIdx.x;
@@ -82,6 +83,8 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
 }
 
 __global__ __launch_bounds__(ST) void sample_kernel(SampleArgs a) {
+    arguments_now(a.logits, a.temperature, a.top_k, a.top_p, a.state, a.out_token, a.out_logprob, a.vocab, a.part_val, a.part_idx,
+                  a.also_token);
     __shared__ float scratch[ST / WAVE];
     __shared__ float seg[ST], seg_pref[ST];
     __shared__ float s_u;

@@ -58,6 +58,9 @@ constexpr int skinny_waves_per_simd() { return (WN * KSI == 8 && MT == 1 && NT <
 
 template <int MT, int NT, int WN, int KSI, int EPI>
 __global__ __launch_bounds__(64 * WN * KSI, (skinny_waves_per_simd<MT, NT, WN, KSI, EPI>())) void gemm_skinny_kernel(SkinnyArgs a) {
+    arguments_now(a.A, a.W, a.out, a.M, a.N, a.K, a.k_per_wave);
+    if constexpr (EPI == SK_SWIGLU) arguments_now(a.n_out, a.row_ss, a.ss_parts, a.ss_eps);
+    if constexpr (EPI == SK_RESIDUAL_PRENORM) arguments_now(a.norm_w, a.hn, a.ss_part);
     __shared__ float red[(KSI > 1 ? (KSI - 1) : 1) * WN * NT * 4 * 64];  // one row tile of every slice at a time
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wn = wave % WN, wk = wave / WN;
@@ -330,6 +333,7 @@ struct SkinnyNormArgs {
 
 template <int NT, int KSI, int EPI, int NP>
 __global__ __launch_bounds__(64 * KSI) void gemm_skinny_norm_kernel(SkinnyNormArgs a) {
+    arguments_now(a.x, a.partials, a.partial_stride, a.norm_w, a.x_out, a.W, a.out, a.M, a.N, a.K, a.k_per_wave, a.n_out, a.eps);
     static_assert(KSI > 1, "the slices of K are waves of one block");
     __shared__ float red[(KSI - 1) * NT * 4 * 64];
     __shared__ float ss_part[KSI][16];
