@@ -73,7 +73,9 @@ def test_rmsnorm(dtype, T, d, eps):
                                    # the tiled kernel's K steps: one partial step, one whole, two whole, whole + partial
                                    (70, 100, 40), (130, 64, 64), (100, 96, 128), (513, 1200, 136), (2048, 1152, 904),
                                    # few tiles, whole K steps: four LDS buffers in turn, with four, five, seven and nineteen steps
-                                   (64, 200, 256), (48, 264, 320), (40, 130, 448), (100, 72, 1216)])
+                                   (64, 200, 256), (48, 264, 320), (40, 130, 448), (100, 72, 1216),
+                                   # so many tiles that tiles of 128x160 save a round: whole tiles, and ragged rows and columns
+                                   (1024, 9728, 136), (1000, 9700, 264)])
 def test_linear(dtype, M, N, K):
     ops = ops_for(dtype)
     a, w = rnd((M, K), dtype, 5), rnd((N, K), dtype, 6, K ** -0.5)
@@ -204,7 +206,9 @@ def test_residual_product_prepares_the_norm_for_the_gated_product(dtype, M, N, K
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,I,K", [(1, 16, 8), (9, 160, 64), (70, 328, 192), (200, 4864, 896), (64, 4864, 896), (33, 264, 136),
-                                   (64, 328, 256), (50, 1000, 576)])
+                                   (64, 328, 256), (50, 1000, 576),
+                                   # tiles of 128x160 (five pairs of gate and up tiles): whole, and ragged at both edges
+                                   (2048, 4864, 896), (1000, 4850, 200)])
 def test_linear_swiglu(dtype, M, I, K):
     from machserve_amd.kernels import interleave_gate_up
     ops = ops_for(dtype)
