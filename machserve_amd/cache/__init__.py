@@ -14,8 +14,8 @@ _host = ensure_host_module()
 BlockPool, SlotPool, CacheCore = _host.BlockPool, _host.SlotPool, _host.CacheCore
 CacheError, OutOfPages = _host.CacheError, _host.OutOfPages
 
-from .manager import CacheManager, GroupSpec, KVBinding, StateBinding, group_name  # noqa: E402
+from .manager import CacheManager, GroupSpec, KVBinding, StateBinding, group_name, pages_by_need  # noqa: E402
 from .device import DeviceCache  # noqa: E402
 
 __all__ = ["BlockPool", "CacheCore", "CacheError", "OutOfPages", "SlotPool", "CacheManager", "GroupSpec", "KVBinding",
-           "StateBinding", "group_name", "DeviceCache"]
+           "StateBinding", "group_name", "pages_by_need", "DeviceCache"]

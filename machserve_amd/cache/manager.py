@@ -89,10 +89,28 @@ class _SlotsView:
         return self._core.slot_is_live(slot)
 
 
+def pages_by_need(max_tokens: int, max_requests: int, portion: int, page_size: int):
+    """A rule for :class:`CacheManager`'s ``num_pages``: a group of all keys gets the pages of ``max_tokens``
+    tokens; a window group only what its requests can hold at a time, which is, for each of ``max_requests``
+    requests, the pages that ``window + portion - 1`` consecutive keys touch (``portion``: the most tokens of one
+    request that a step brings), and never more than the group of all keys would get.  The scheduler refuses a
+    request by the same count (``csrc/host/scheduler.hpp``, ``SchedulerCore::add``)."""
+    full = max(1, -(-max_tokens // page_size))
+
+    def rule(group: "GroupSpec") -> int:
+        if group.window is None:
+            return full
+        per_request = -(-(group.window + portion - 1) // page_size) + 1
+        return max(1, min(full, max_requests * per_request))
+    return rule
+
+
 class CacheManager:
-    def __init__(self, layer_requests, page_size: int, num_pages: int, max_requests: int):
+    def __init__(self, layer_requests, page_size: int, num_pages, max_requests: int):
         """``layer_requests[p]`` is the cache request of the p-th layer run of a step (see
-        ``parts.base`` and ``DecoderModel.cache_requests``); "layer" below means such a run."""
+        ``parts.base`` and ``DecoderModel.cache_requests``); "layer" below means such a run.
+        ``num_pages``: pages of every group's pool; or a dict from group name to pages (a group it
+        does not name is an error); or a rule ``GroupSpec -> pages`` (see :func:`pages_by_need`)."""
         from ..parts.base import PagedKVRequest, SharedKVRequest, StateRequest
         self.core = CacheCore(page_size, max_requests)
         self.page_size = page_size
@@ -137,8 +155,17 @@ class CacheManager:
         self.layer_source = {i: src for (i, j), src in self.shared.items() if not self.layer_requests[i][0]}
         self.layer_group.update({i: self.paged[(src, 0)] for i, src in self.layer_source.items()})
         self.state_requests = {i: r for (i, j), r in self.states.items() if not self.layer_requests[i][0]}
+        if isinstance(num_pages, dict):
+            unknown = sorted(set(num_pages) - set(specs))
+            missing = sorted(set(specs) - set(num_pages))
+            if unknown or missing:
+                raise CacheError(f"num_pages names groups {unknown} that the model has not and lacks {missing}; "
+                                 f"the model's groups are {sorted(specs)}")
         for name, spec in specs.items():
-            index = self.core.add_group(name, spec.window or 0, num_pages)
+            pages = num_pages[name] if isinstance(num_pages, dict) else num_pages(spec) if callable(num_pages) else num_pages
+            if isinstance(pages, bool) or not isinstance(pages, int) or pages < 1:
+                raise CacheError(f"group {name}: {pages!r} pages; a pool needs at least one")
+            index = self.core.add_group(name, spec.window or 0, pages)
             self.groups[name] = _Group(spec, self.core, index)
         self._names = list(self.groups)
         self.device = None  # filled by DeviceCache

@@ -44,6 +44,8 @@ class AttentionSpec:
     ``window``: number of most recent keys a row may see (None = all).
     ``kv_source``: index of another layer whose cache this layer reads instead of
     writing its own (None = own cache).
+    ``scale``: what the scores are multiplied by before the softmax (None = ``head_dim ** -0.5``,
+    ``crates/mach-model/src/config.rs:231-234``).
     """
     kind: str
     hidden: int
@@ -54,6 +56,7 @@ class AttentionSpec:
     window: Optional[int] = None
     kv_source: Optional[int] = None
     tensors: Mapping[str, str] = field(default_factory=dict)
+    scale: Optional[float] = None
 
 
 @dataclass(frozen=True)
@@ -68,7 +71,9 @@ class GatedMlpSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One block: which arrangement, and the specs of the parts it arranges."""
+    """One pre-norm block: the specs of the four parts it arranges.  ``block`` names the registered arrangement,
+    which builds its parts from the fields it reads; another arrangement brings a spec class of its own (any object
+    with ``block`` and the fields that arrangement reads)."""
     block: str
     mixer: object
     feed_forward: object
@@ -116,11 +121,11 @@ class ModelSpec:
             if not 0 <= i < n:
                 raise ConfigError(f"order names layer {i}, but there are {n} layers")
         for i, layer in enumerate(self.layers):
-            src = getattr(layer.mixer, "kv_source", None)
+            src = getattr(getattr(layer, "mixer", None), "kv_source", None)
             if src is not None:
                 if not 0 <= src < n or src == i:
                     raise ConfigError(f"layer {i}: kv_source {src} is not another layer")
-                if getattr(self.layers[src].mixer, "kv_source", None) is not None:
+                if getattr(getattr(self.layers[src], "mixer", None), "kv_source", None) is not None:
                     raise ConfigError(f"layer {i}: kv_source {src} itself reads another layer's cache")
                 if self.order.index(src) > self.order.index(i):
                     raise ConfigError(f"layer {i} reads the cache of layer {src}, which runs later")

@@ -1130,7 +1130,13 @@ extern "C" int MS_CAT(ms_decode_attention_noalloc_nd, MS_ATTN_ND)(
     return MS_CAT(ms_decode_attention_nd, MS_ATTN_ND)(q, kpool, vpool, out, part_o, part_ml, block_table, table_stride,
                                                       seq_pos0, S, H, KV, hd, ps, window, nsplit, scale, stream);
 }
-extern "C" long MS_CAT(ms_decode_attention_noalloc_max_floats_nd, MS_ATTN_ND)() { return (long)NOALLOC_SCRATCH_FLOATS; }
+// The most floats of scratch a step may need.  The call also looks up the scratch's address on the current device
+// (the set-up that the entry point would otherwise do at its first call there): a caller that is about to capture
+// a stream calls this first, on each device it uses, and the entry point itself then makes nothing but launches.
+extern "C" long MS_CAT(ms_decode_attention_noalloc_max_floats_nd, MS_ATTN_ND)() {
+    (void)scratch_of_current_device();
+    return (long)NOALLOC_SCRATCH_FLOATS;
+}
 
 // The same from the partial sums of the q/k/v projection: adds them and the bias, rotates q and k
 // by the row's position, writes k and v into the row's page, and attends; a second launch merges

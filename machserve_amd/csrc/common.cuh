@@ -32,6 +32,15 @@ typedef _Float16 elem_t;
 #else
 typedef float elem_t;
 #endif
+// Half precision has five bits of exponent: a value of the 32-bit stream times a norm's weight, not yet divided by
+// the row's root mean square, may lie outside its range (or among its subnormals), which bfloat16, with float's
+// exponent, and float itself do not mind.  The forms that round such a value (the norm folded into the product
+// that reads it) are not taken in the half-precision build: there the norm runs first and rounds after the division.
+#if defined(MS_ELEM_F16)
+constexpr bool kRoundsBeforeTheNormIsSafe = false;
+#else
+constexpr bool kRoundsBeforeTheNormIsSafe = true;
+#endif
 #ifdef MS_ELEM_HALF
 constexpr bool kHalf = true;  // two-byte elements
 typedef elem_t half8_t __attribute__((ext_vector_type(8)));
@@ -165,6 +174,7 @@ template <int NT> __device__ __forceinline__ float block_sum(float v, float* scr
 // Entry points return 0 on success; otherwise ms_last_error() describes the refusal.
 void set_error(const char* fmt, ...);
 int check_launch(const char* what);
+int compute_units();  // of the current device, asked once
 
 #define MS_REQUIRE(cond, ...)            \
     do {                                 \
@@ -175,5 +185,6 @@ int check_launch(const char* what);
     } while (0)
 
 __host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b - 1) / b; }
+__host__ __device__ __forceinline__ long ceil_div(long a, long b) { return (a + b - 1) / b; }
 
 }  // namespace ms

@@ -268,6 +268,12 @@ __global__ __launch_bounds__(256) void rope_kv_write_quads_kernel(RopeArgs a) {
 
 using namespace ms;
 
+// The widest row that the norm and the rotation kernels hold in a block's LDS (floats); a model asks for these
+// when it is put together, so that a wider one is refused then, with the size's name, not at its first step.
+constexpr int MAX_ROW_FLOATS = 15000;
+extern "C" int ms_max_norm_width() { return MAX_ROW_FLOATS; }
+extern "C" int ms_max_rope_row() { return MAX_ROW_FLOATS; }
+
 extern "C" int ms_embed(const int* tokens, const void* table, float* x, int T, int d, float scale, hipStream_t stream) {
     MS_REQUIRE(T > 0 && d > 0, "embed: empty problem T=%d d=%d", T, d);
     hipLaunchKernelGGL(embed_kernel, dim3(T), dim3(256), 0, stream, tokens, (const elem_t*)table, x, d, scale);
@@ -280,7 +286,7 @@ extern "C" int ms_embed(const int* tokens, const void* table, float* x, int T, i
 extern "C" int ms_rmsnorm(float* x, const float* partials, int n_partials, int T, const int* rows, const float* w,
                           void* out, int out_f32, int n, int d, float eps, hipStream_t stream) {
     MS_REQUIRE(n > 0 && d > 0, "rmsnorm: empty problem n=%d d=%d", n, d);
-    MS_REQUIRE(d * sizeof(float) <= 60000, "rmsnorm: width %d exceeds the row buffer", d);
+    MS_REQUIRE(d <= MAX_ROW_FLOATS, "rmsnorm: width %d exceeds the row buffer of %d", d, MAX_ROW_FLOATS);
     MS_REQUIRE(n_partials == 0 || partials, "rmsnorm: %d partial sums without a buffer", n_partials);
     const size_t ps = (size_t)T * d, smem = (size_t)d * sizeof(float);
     const bool f32_out = out_f32 || !kHalf;
@@ -348,7 +354,7 @@ extern "C" int ms_rope_kv_write(const float* qkv, int n_partials, const float* b
                stride, H, KV, hd);
     MS_REQUIRE(!slot_map || (kpool && vpool && ps > 0), "rope: cache write without pools");
     MS_REQUIRE(n_partials >= 1, "rope: %d partial sums", n_partials);
-    MS_REQUIRE(stride * sizeof(float) <= 60000, "rope: a row of %d values exceeds the row buffer", stride);
+    MS_REQUIRE(stride <= MAX_ROW_FLOATS, "rope: a row of %d values exceeds the row buffer of %d", stride, MAX_ROW_FLOATS);
     RopeArgs a{qkv, bias, n_partials, (size_t)T * stride, positions, inv_freq, slot_map, (elem_t*)q_out, (elem_t*)kpool,
                (elem_t*)vpool, stride, H, KV, hd, ps};
     const bool aligned = ((reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(bias) | reinterpret_cast<uintptr_t>(q_out) |

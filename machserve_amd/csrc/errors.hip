@@ -28,12 +28,29 @@ int check_launch(const char* what) {
     return 0;
 }
 
+// Compute units of the current device, asked once (256 if the device will not say).  The products' planners fill
+// the chip by this count: two 128x128 blocks a CU, sixteen waves a CU.
+int compute_units() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1)
+            n = 256;
+        (void)hipGetLastError();
+        cus = n;
+    }
+    return cus;
+}
+
 }  // namespace ms
 
 extern "C" const char* ms_last_error() { return ms::g_error; }
 
 // Kernels launched by this library so far (every launch goes through check_launch).
 extern "C" long ms_launch_count() { return ms::g_launches; }
+
+// Compute units of the current device, as the planners count them.
+extern "C" int ms_compute_units() { return ms::compute_units(); }
 
 // Bytes of an element of this build: 2 (bfloat16 or half precision) or 4.
 extern "C" int ms_elem_bytes() { return (int)sizeof(ms::elem_t); }

@@ -404,22 +404,25 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
     // The largest tile that still gives every CU of the chip a block or two, with K steps of 64 (half
     // the barriers of steps of 32).  Measured on M = 512..8192 of the 0.5B shapes; larger wave tiles
     // (256x128) lose: their accumulators no longer fit the registers of two blocks a CU.
+    // two 128x128 blocks a CU are a round of the chip (512 on 256 CUs); a tile is taken when its blocks fill
+    // six tenths of a round
+    const long round_blocks = 2L * compute_units(), enough = round_blocks * 300 / 512;
     if (M > 64) {
         const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128), b12864 = (long)ceil_div(M, 128) * ceil_div(N, 64);
-        // The chip holds 512 such blocks at a time and a round that is nearly empty takes as long as a full one:
+        // The chip holds a round of such blocks at a time and a round that is nearly empty takes as long as a full one:
         // the time is rounds times the tile's width.  Where tiles a quarter wider save more in rounds than they
         // cost, they are taken (0.5B gate/up product at 2,048 rows: 1,216 tiles of 128x128 are two rounds and three
         // eighths, 976 of 128x160 two rounds less a twentieth: 55 -> 45 us).  Tiles of 128x96 save rounds by the
         // same count but lose more in themselves (8,192 rows: 16.3 against 15.7 ms for the whole prompt).
-        if (ns == 1 && ep.k_per_split >= 128 && b128 >= 300) {
-            const long rounds128 = (b128 + 511) / 512, rounds160 = ((long)ceil_div(M, 128) * ceil_div(N, 160) + 511) / 512;
+        if (ns == 1 && ep.k_per_split >= 128 && b128 >= enough) {
+            const long rounds128 = ceil_div(b128, round_blocks), rounds160 = ceil_div((long)ceil_div(M, 128) * ceil_div(N, 160), round_blocks);
             if (rounds160 * 160 < rounds128 * 128) MS_GEMM(128, 160, 4, 1, 64);
         }
-        if (b128 * ns >= 300) {
+        if (b128 * ns >= enough) {
             if (ep.k_per_split >= 128) MS_GEMM(128, 128, 2, 2, 64);
             MS_GEMM(128, 128, 2, 2, 32);
         }
-        if (b12864 * ns >= 300) {
+        if (b12864 * ns >= enough) {
             if (ep.k_per_split >= 128) MS_GEMM(128, 64, 2, 2, 64);
             MS_GEMM(128, 64, 2, 2, 32);
         }
@@ -427,7 +430,7 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
     // At most two blocks a CU, each a chain of K steps: four LDS buffers keep three steps in flight (0.5B
     // gate/up product at 64 rows, 152 blocks of 14 steps: 10.5 -> 7.8 us; 1.5B: 23.7 -> 21.1; with more
     // blocks than that the blocks hide each other's loads and the two-buffer kernel is as fast).
-    if ((long)ceil_div(M, 64) * ceil_div(N, 64) * ns <= 512 && whole_steps && ep.k_per_split >= 256) MS_GEMM_DEEP(64, 64, 2, 2, 64, 4);
+    if ((long)ceil_div(M, 64) * ceil_div(N, 64) * ns <= round_blocks && whole_steps && ep.k_per_split >= 256) MS_GEMM_DEEP(64, 64, 2, 2, 64, 4);
     MS_GEMM(64, 64, 2, 2, 64);
 #else
     MS_GEMM(64, 64, 2, 2, 32);
@@ -447,7 +450,8 @@ static constexpr int g_force_splits = 0;
 static int plan_tiled_splits(int M, int N, int K) {
 #ifdef MS_ELEM_HALF
     const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
-    if (b128 >= 300 && g_force_splits == 0) return 1;
+    const long round_blocks = 2L * compute_units();  // two 128x128 blocks a CU
+    if (b128 >= round_blocks * 300 / 512 && g_force_splits == 0) return 1;
     // More than six slices cost more in the consumer's sums than they gain here (with very few tiles - a
     // portion of a few hundred rows - slices of 256 still pay).  With few rows the partial sums are small
     // and the weight is all the traffic: a long K is then cut up to 16 times (7B down projection at 64
@@ -461,15 +465,15 @@ static int plan_tiled_splits(int M, int N, int K) {
     // rows 5.1 us in 6 slices, 5.5 in 8)
     const int shortest = b128 <= 16 && M <= 128 ? (K >= 1536 ? 256 : 128) : (b128 <= 32 ? 256 : 512);
     const int limit = max(1, min(K / shortest, most));
-    // The chip holds 512 of the 128x128 blocks at a time (two a CU), and a last round that is nearly
+    // The chip holds two of the 128x128 blocks a CU at a time (512 on 256 CUs), and a last round that is nearly
     // empty takes as long as a full one: the fewest slices that fill their rounds to 70 %, else the
     // count that fills them best (1.5B down projection at 2,048 rows, 192 tiles: 3 slices make a
     // full round and an eighth, 118 us; 2 slices one round three quarters full, 97 us).
     int want = 1;
     double best = 0.0;
     for (int sl = 1; sl <= limit; ++sl) {
-        const long blocks = b128 * sl, rounds = (blocks + 511) / 512;
-        const double filled = (double)blocks / (double)(rounds * 512);
+        const long blocks = b128 * sl, rounds = ceil_div(blocks, round_blocks);
+        const double filled = (double)blocks / (double)(rounds * round_blocks);
         if (filled > best + 1e-9) {
             best = filled;
             want = sl;
@@ -517,7 +521,7 @@ extern "C" int ms_linear_swiglu(const void* a, const void* w, void* out, int M, 
 extern "C" int ms_swiglu_scaled_takes(int M, int I, int K) {
 #ifdef MS_ELEM_HALF
     (void)I;
-    return M >= 1 && M <= 64 && K % 64 == 0 && K >= 256;
+    return kRoundsBeforeTheNormIsSafe && M >= 1 && M <= 64 && K % 64 == 0 && K >= 256;
 #else
     (void)M; (void)I; (void)K;
     return 0;

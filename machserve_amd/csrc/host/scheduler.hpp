@@ -78,23 +78,26 @@ public:
     StepPlan schedule() {
         StepPlan plan;
         const int G = cache_.num_groups(), ps = cache_.page_size();
+        // There are never more decoding requests than the budget holds: a request starts (and a prompt ends) only in
+        // a step that had budget left for it beside every decoding request, so the sum never grows beyond it.  Checked
+        // before anything is preempted, so that a refusal leaves the queues and the pages as they were.
+        {
+            int decoders = 0;
+            for (long id : running_) decoders += reqs_.at(id).decoding();
+            if (decoders > budget_)
+                throw SchedulerError(cat(decoders, " requests decode under a budget of ", budget_, " tokens a step"));
+        }
         while (true) {
             plan.items.clear();
             int budget = budget_;
-            // 1. decoded tokens, oldest request first; they must all fit, or the youngest goes.  There are never
-            //    more decoding requests than the budget holds: a request starts (and a prompt ends) only in a step
-            //    that had budget left for it beside every decoding request, so the sum never grows beyond it.
+            // 1. decoded tokens, oldest request first; they must all fit, or the youngest goes
             std::vector<int> need(G, 0);
-            int decoders = 0;
             for (long id : running_) {
                 const Req& r = reqs_.at(id);
                 if (!r.decoding()) continue;
-                ++decoders;
                 auto n = cache_.pages_needed(r.slot, 1);
                 for (int g = 0; g < G; ++g) need[g] += n[g];
             }
-            if (decoders > budget)
-                throw SchedulerError(cat(decoders, " requests decode under a budget of ", budget, " tokens a step"));
             bool short_of = false;
             for (int g = 0; g < G; ++g) short_of |= cache_.group_available(g) < need[g];
             if (short_of) {

@@ -9,6 +9,9 @@
 // message (ms_last_error).  It calls no hipMalloc, hipFree or allocating library routine.  Every GPU the
 // library runs on holds its own array until the process ends; all calls on one GPU share it, so calls
 // that overlap on one GPU race: the caller orders them (one stream, or events between streams).
+// ms_decode_attention_noalloc_max_floats_nd<N>() also does the entry point's set-up for the current device (it
+// looks up the array's device address, which the entry point would otherwise do at its first call there): call
+// it once per device before a stream capture, and the entry point makes nothing but kernel launches.
 //
 // One library per head-size tile: <N> is the tile in units of 16 (1, 2, 3, 4, 6, 8, 12, 16); a head size
 // runs in the next larger tile.  Operands as in ms_decode_attention_nd<N>: q [S, H * hd], key pool

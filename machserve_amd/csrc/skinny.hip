@@ -488,7 +488,7 @@ static SkinnyPlan plan_skinny(int M, int N, int K, bool allow_partials, bool pai
     const int NT = skinny_nt(M, N, pairs);
     const int col_waves = ceil_div(N, 16 * NT);
     const int slices = ceil_div(K, KSTEP);  // slices of 128 along K: one wave iteration each
-    int want = max(1, min(ceil_div(4096, col_waves), slices));  // waves wanted along K
+    int want = max(1, min(ceil_div(16 * compute_units(), col_waves), slices));  // waves wanted along K: sixteen a CU in all
     if (g_force_ksi > 0) want = min(g_force_ksi, slices);
     SkinnyPlan p;
     if (want == 1) {
@@ -549,7 +549,7 @@ static int plan_skinny_norm(int M, int N, int K, int n_partials) {
     if (M > 16 || n_partials > 6 || K % 8) return 0;
     const int col_waves = ceil_div(N, 32);
     const int slices = ceil_div(K, KSTEP);
-    const int want = max(1, min(ceil_div(4096, col_waves), slices));
+    const int want = max(1, min(ceil_div(16 * compute_units(), col_waves), slices));
     if (want == 1) return 0;
     return want > 4 ? 8 : (want > 2 ? 4 : 2);
 }
@@ -615,10 +615,10 @@ extern "C" int ms_linear_swiglu_skinny(const void* a, const void* w, void* out, 
 // which multiplies 64-row tiles of padding and ends in a long epilogue; the walk over K there is bound by
 // its own instructions, not by memory.)
 extern "C" int ms_swiglu_scaled_skinny_takes(int M, int I, int K) {
-    if (!kHalf || M < 1 || M > 16 || K % 8) return 0;
+    if (!kHalf || !kRoundsBeforeTheNormIsSafe || M < 1 || M > 16 || K % 8) return 0;
     const int n = 2 * ceil_div(I, 16) * 16;
     const SkinnyPlan p = plan_skinny(M, n, K, false, true);
-    return ceil_div(n, 32 * p.wn) * p.wn * p.ksi <= 4096;  // sixteen waves a CU
+    return ceil_div(n, 32 * p.wn) * p.wn * p.ksi <= 16 * compute_units();  // sixteen waves a CU
 }
 
 // ms_linear_swiglu_skinny for rows that came in multiplied by a norm's weight only: both products of a row are
@@ -637,6 +637,7 @@ extern "C" int ms_linear_swiglu_scaled_skinny(const void* a, const float* row_ss
 // to read (measured: with nothing pending it saves a microsecond or two over the norm's own launch;
 // with one pending sum it breaks even at four rows; with five it costs twice as much).
 extern "C" int ms_skinny_norm_takes(int M, int N, int K, int n_partials) {
+    if (!kRoundsBeforeTheNormIsSafe) return 0;  // the kernel rounds x * norm_w before it knows the row's root mean square
     if (n_partials > 1 || (n_partials == 1 && M > 4)) return 0;
     return plan_skinny_norm(M, N, K, n_partials) > 0;
 }
@@ -669,6 +670,7 @@ extern "C" int ms_linear_residual_skinny(const void* a, const void* w, float* x,
 // Column waves of ms_linear_residual_prenorm_skinny for this shape (the first size of its ss_part), or 0 if the
 // shape is not taken: more than 32 rows, or a K that is cut over several blocks.
 extern "C" int ms_skinny_prenorm_parts(int M, int N, int K) {
+    if (!kRoundsBeforeTheNormIsSafe) return 0;  // hn = x * norm_w is rounded before the division
     if (M < 1 || M > 32 || K % 8) return 0;
     const SkinnyPlan p = plan_skinny(M, N, K, true);
     return p.ksb == 1 ? ceil_div(N, 16 * skinny_nt(M, N)) : 0;

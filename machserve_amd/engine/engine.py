@@ -39,7 +39,8 @@ class Engine:
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None, capacity: int = 64,
                  max_batch_tokens: int = 512, chunk_size: Optional[int] = None) -> "Engine":
         loaded = load_model(model_dir, dtype=dtype, device=device, page_size=page_size, num_pages=num_pages,
-                            max_tokens=max_tokens, max_requests=capacity)
+                            max_tokens=max_tokens, max_requests=capacity,
+                            portion=min(chunk_size or max_batch_tokens, max_batch_tokens))
         return cls(loaded, max_batch_tokens, chunk_size, capacity)
 
     def add(self, prompt: Sequence[int], max_new: int, params: Optional[SamplingParams] = None,

@@ -7,7 +7,7 @@ from typing import Optional
 
 import torch
 
-from ..cache import CacheManager, DeviceCache
+from ..cache import CacheManager, DeviceCache, pages_by_need
 from ..config import load_config
 from ..kernels import get_ops
 from ..parts import DecoderModel, Runtime
@@ -38,11 +38,13 @@ class LoadedModel:
 
 
 def load_model(model_dir: Optional[str] = None, *, dtype="bfloat16", device: str = "cuda:0", page_size: int = 64,
-               num_pages: Optional[int] = None, max_tokens: Optional[int] = None, max_requests: int = 64,
-               config=None, tensors=None, ops=None, use_graphs: bool = True) -> LoadedModel:
+               num_pages=None, max_tokens: Optional[int] = None, max_requests: int = 64,
+               config=None, tensors=None, ops=None, use_graphs: bool = True, portion: Optional[int] = None) -> LoadedModel:
     """``model_dir`` holds config.json and model.safetensors; alternatively pass a typed
-    ``config`` and a dict of ``tensors``.  The cache pool has ``num_pages`` pages per group,
-    or enough for ``max_tokens`` tokens."""
+    ``config`` and a dict of ``tensors``.  Every group's pool has ``num_pages`` pages (a dict
+    gives each group its own number), or enough for ``max_tokens`` tokens; with ``portion``
+    (the most tokens of one request that a step will bring) a group of layers that see a window
+    gets only what ``max_requests`` requests can hold of it at a time."""
     dt = parse_dtype(dtype)
     if config is None:
         config = load_config(model_dir)
@@ -55,7 +57,8 @@ def load_model(model_dir: Optional[str] = None, *, dtype="bfloat16", device: str
     if num_pages is None:
         if max_tokens is None:
             max_tokens = 4096
-        num_pages = max(1, -(-max_tokens // page_size))
+        num_pages = (pages_by_need(max_tokens, max_requests, portion, page_size) if portion
+                     else max(1, -(-max_tokens // page_size)))
     cache = CacheManager(model.cache_requests(), page_size, num_pages, max_requests)
     device_cache = DeviceCache(cache, dt, rt.device)
     model.bind_cache(device_cache)

@@ -93,7 +93,7 @@ class StepFunction:
         # costs as much as a few dozen launched steps, so a shape must earn it).  Only for models
         # whose parts read nothing but device memory from the context.
         self.use_graphs = (use_graphs and rt.device.type == "cuda"
-                           and all(getattr(b.mixer, "graph_safe", False) for b in getattr(model, "blocks", [])))
+                           and all(getattr(b, "graph_safe", False) for b in getattr(model, "blocks", [])))
         self._graphs: "OrderedDict[tuple, _DecodeGraph]" = OrderedDict()
         self._graph_pool = None  # the memory pool that all captures share
         self._seen: Dict[tuple, int] = {}
@@ -102,8 +102,8 @@ class StepFunction:
 
     # ------------------------------------------------------------------ context
     def _check_entries(self, entries: Sequence[StepEntry]):
-        """Validates the entries; returns their slots, token counts, flattened tokens and wanted rows.
-        ``self._explicit`` is left as the entries' own positions, flattened ``[rows * axes]``, or empty if none has any."""
+        """Validates the entries before anything is taken or run; returns their slots, token counts, flattened tokens,
+        wanted rows, and the entries' own positions flattened ``[rows * axes]`` (empty if no entry brings any)."""
         if not entries:
             raise StepError("a step needs at least one entry")
         cache, vocab, limit = self.cache, self.model.vocab, self.model.spec.max_positions
@@ -113,8 +113,18 @@ class StepFunction:
         explicit = [] if any(e.positions is not None for e in entries) else None
         for e in entries:
             n = len(e.tokens)
-            if explicit is not None:
+            if n == 0:
+                raise StepError(f"slot {e.slot}: an entry needs at least one token")
+            if e.slot in seen:
+                raise StepError(f"slot {e.slot} appears twice in one step")
+            seen.add(e.slot)
+            try:
                 base = cache.length(e.slot)
+            except CacheError as err:  # not a request's slot
+                raise StepError(str(err)) from err
+            if base + n > limit:
+                raise StepError(f"slot {e.slot}: position {base + n - 1} is beyond the model's {limit} positions")
+            if explicit is not None:
                 rows = e.positions if e.positions is not None else [[base + j] * axes for j in range(n)]
                 if len(rows) != n or any(len(r) != axes for r in rows):
                     raise StepError(f"slot {e.slot}: positions must be {n} rows of {axes} numbers")
@@ -122,13 +132,6 @@ class StepFunction:
                     if min(r) < 0 or max(r) >= limit:
                         raise StepError(f"slot {e.slot}: position {list(r)} is outside the model's {limit} positions")
                     explicit.extend(int(v) for v in r)
-            if n == 0:
-                raise StepError(f"slot {e.slot}: an entry needs at least one token")
-            if e.slot in seen:
-                raise StepError(f"slot {e.slot} appears twice in one step")
-            seen.add(e.slot)
-            if cache.length(e.slot) + n > limit:
-                raise StepError(f"slot {e.slot}: position {cache.length(e.slot) + n - 1} is beyond the model's {limit} positions")
             toks = [int(t) for t in e.tokens]
             if min(toks) < 0 or max(toks) >= vocab:
                 bad = next(t for t in toks if not 0 <= t < vocab)
@@ -140,8 +143,20 @@ class StepFunction:
             slots.append(e.slot)
             counts.append(n)
             tokens.extend(toks)
-        self._explicit = explicit or []
-        return slots, counts, tokens, want
+        return slots, counts, tokens, want, explicit or []
+
+    def _take_pages(self, entries: Sequence[StepEntry]) -> None:
+        """The pages the entries' tokens need, in every group: all of them or, with ``OutOfPages``, none."""
+        cache = self.cache
+        reserved: Dict[str, int] = {}
+        for e in entries:
+            for k, v in cache.pages_needed(e.slot, len(e.tokens)).items():
+                reserved[k] = reserved.get(k, 0) + v
+        for k, v in reserved.items():
+            if cache.free_pages(k) < v:
+                raise OutOfPages(f"group {k}: the step needs {v} new pages, {cache.free_pages(k)} are free")
+        for e in entries:
+            cache.extend(e.slot, len(e.tokens))
 
     def _context_from(self, dev: torch.Tensor, offsets, widths: Dict[str, int], host=None, sequential: bool = True) -> StepContext:
         """A step context over the device copy of a buffer laid out by ``CacheManager.build_step``."""
@@ -159,17 +174,17 @@ class StepFunction:
             ctx.attention_work[g] = sec(f"work/{g}").view(-1, 2)
         return ctx
 
-    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
-        slots, counts, tokens, want = self._check_entries(entries)
+    def build_context(self, entries: Sequence[StepEntry], checked=None) -> StepContext:
+        slots, counts, tokens, want, explicit = checked or self._check_entries(entries)
         try:
             host, offsets, widths = self.cache.build_step(slots, counts, tokens, want, self.heads_per_kv, self.rows_per_block,
-                                                          1, 0, self.position_axes, self._explicit)
+                                                          1, 0, self.position_axes, explicit)
         except CacheError as e:
             raise StepError(str(e)) from e
         dev = torch.from_numpy(host).to(self.rt.device)  # one buffer, one copy
         lists = {k: host[offsets[k][0]:offsets[k][0] + offsets[k][1]].tolist()
                  for k in ("tokens", "positions", "seq_q_start", "seq_q_len", "seq_pos0", "seq_slot", "want_rows")}
-        return self._context_from(dev, offsets, widths, lists, sequential=not self._explicit)
+        return self._context_from(dev, offsets, widths, lists, sequential=not explicit)
 
     # ------------------------------------------------------------------ captured decode steps
     @staticmethod
@@ -186,14 +201,14 @@ class StepFunction:
             return b
         return -(-n // 16) * 16
 
-    def _decode_shape(self, entries: Sequence[StepEntry], sampled: bool):
+    def _decode_shape(self, checked, sampled: bool):
         """The buffer of a decode step (every row's logits are computed), its graph's key, and the
         number of rows added.  The step is filled up to a bucket's size, so that a few graphs serve every
         batch size while requests end one by one, with rows that belong to no request: token 0 at position 0
         of the cache manager's scratch slot and scratch page, so that they change no key, value or state that
         a request owns (a mixer with state of fixed size may be captured too); their logits are dropped.  A
         decode step's time hardly depends on a few rows more."""
-        slots, counts, tokens, _ = self._check_entries(entries)
+        slots, counts, tokens = checked[:3]
         pad = self._decode_bucket(len(slots)) - len(slots)
         try:
             built = self.cache.build_step(slots, counts, tokens, list(range(len(slots) + pad)), self.heads_per_kv,
@@ -219,7 +234,7 @@ class StepFunction:
         # for given tokens per request, wanted rows and table widths the buffer's layout is always the same
         return (tuple(counts), n_want, tuple(sorted(widths.items())), sampled)
 
-    def _run_graph(self, key: tuple, built, sampling=None, after: Optional["LaunchedDecode"] = None):
+    def _run_graph(self, key: tuple, built, sampling=None, after: Optional["LaunchedDecode"] = None, fill_rows: int = 0):
         host, offsets, widths = built
         extra: Dict[str, np.ndarray] = {}
         if sampling is not None:
@@ -287,6 +302,10 @@ class StepFunction:
             self._graphs[key] = dg
             while len(self._graphs) > 1 and (len(self._graphs) > self.MAX_GRAPHS or self.graph_bytes() > self.MAX_GRAPH_BYTES):
                 self._graphs.popitem(last=False)
+        if fill_rows and self.cache.device is not None:
+            # rows that fill the step up advance the scratch slot's state of fixed size, step after step: it starts
+            # from zero each time, so that it stays finite whatever the mixer does with it
+            self.cache.device.zero_state(self.cache.scratch_slot)
         dg.graph.replay()
         return (dg.sampled if sampling is not None else dg.logits), dg
 
@@ -315,21 +334,15 @@ class StepFunction:
         if after is not None and after.slots != slots:
             raise StepError("a step fed from the device must hold the requests of the step before, in the same order")
         cache = self.cache
-        reserved: Dict[str, int] = {}
-        for e in entries:
-            for k, v in cache.pages_needed(e.slot, 1).items():
-                reserved[k] = reserved.get(k, 0) + v
-        for k, v in reserved.items():
-            if cache.free_pages(k) < v:
-                raise OutOfPages(f"group {k}: the step needs {v} new pages, {cache.free_pages(k)} are free")
-        for e in entries:
-            cache.extend(e.slot, 1)
-        built, key, pad = self._decode_shape(entries, True)
+        checked = self._check_entries(entries)
+        self._take_pages(entries)
+        built, key, pad = self._decode_shape(checked, True)
         if not self._ready(key, self.DECODE_CAPTURE_AFTER):
             return None  # the pages stay with the requests; the caller runs the step as it is
-        # the added rows sample as the first row does (same logits, same state): the same token
-        filled = [list(v) + [v[0]] * pad for v in (temperatures, top_ks, top_ps, states)]
-        sampled, graph = self._run_graph(key, built, tuple(filled), after)
+        # the rows that fill the step up are rows of the scratch slot: they sample greedily (their token is some
+        # token of the vocabulary, which is all that the next step's embedding needs of it) and are dropped
+        filled = [list(v) + [fill] * pad for v, fill in ((temperatures, 0.0), (top_ks, 0), (top_ps, 1.0), (states, 0))]
+        sampled, graph = self._run_graph(key, built, tuple(filled), after, fill_rows=pad)
         for e in entries:
             cache.commit(e.slot, 1)
         # the samples go to a pinned buffer of their own (the graph's is overwritten by its next replay)
@@ -347,7 +360,7 @@ class StepFunction:
     def collect(self, launched: "LaunchedDecode"):
         """``(tokens, logprobs)`` of a launched step as host lists; waits for them."""
         launched.done.synchronize()
-        n = len(launched.slots)  # rows beyond are copies of the first
+        n = len(launched.slots)  # rows beyond belong to no request
         return launched.result[0, :n].tolist(), launched.result[1, :n].view(torch.float32).tolist()
 
     # ------------------------------------------------------------------ the step
@@ -358,21 +371,13 @@ class StepFunction:
         model, and advances the requests' lengths.  With ``borrow_logits`` the result may be a
         buffer that the next step overwrites (the engine samples from it at once)."""
         cache = self.cache
-        reserved: Dict[str, int] = {}
-        for e in entries:
-            need = cache.pages_needed(e.slot, len(e.tokens))
-            for k, v in need.items():
-                reserved[k] = reserved.get(k, 0) + v
-        for k, v in reserved.items():
-            if cache.free_pages(k) < v:
-                raise OutOfPages(f"group {k}: the step needs {v} new pages, {cache.free_pages(k)} are free")
-        for e in entries:
-            cache.extend(e.slot, len(e.tokens))
+        checked = self._check_entries(entries)  # a step that is refused has taken nothing
+        self._take_pages(entries)
         graphs = self.use_graphs and all(e.positions is None for e in entries)  # a captured step takes positions from the cache
         if graphs and all(len(e.tokens) == 1 for e in entries) and len({e.slot for e in entries}) == len(entries):
-            built, key, pad = self._decode_shape(entries, False)
+            built, key, pad = self._decode_shape(checked, False)
             if self._ready(key, self.DECODE_CAPTURE_AFTER):
-                logits, _ = self._run_graph(key, built)
+                logits, _ = self._run_graph(key, built, fill_rows=pad)
             else:
                 host, offsets, widths = built
                 logits = self.model.forward(self._context_from(torch.from_numpy(host).to(self.rt.device), offsets, widths))
@@ -387,7 +392,7 @@ class StepFunction:
             elif not borrow_logits:
                 logits = logits.clone()  # the graph's own buffer is overwritten by its next replay
         elif graphs:
-            slots, counts, tokens, want = self._check_entries(entries)
+            slots, counts, tokens, want, _ = checked
             # block tables as wide as the next power of two of pages: a prompt that grows by a
             # portion a step keeps its shape for many steps
             pages = max(-(-(cache.length(sl) + n) // cache.page_size) for sl, n in zip(slots, counts))
@@ -408,7 +413,7 @@ class StepFunction:
                 host, offsets, widths = built
                 logits = self.model.forward(self._context_from(torch.from_numpy(host).to(self.rt.device), offsets, widths))
         else:
-            logits = self.model.forward(self.build_context(entries))
+            logits = self.model.forward(self.build_context(entries, checked))
         for e in entries:
             cache.commit(e.slot, len(e.tokens))
         return logits

@@ -98,12 +98,19 @@ class HipOps:
         if shape and t.shape != shape:
             raise KernelError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
 
-    def require_sizes(self, what: str, reductions=(), head_dim: Optional[int] = None) -> None:
+    def require_sizes(self, what: str, reductions=(), head_dim: Optional[int] = None, norm_width: Optional[int] = None,
+                      rotated_row: Optional[int] = None) -> None:
         """Refuses, when a model is put together, sizes that the kernels do not take: a product sums over a
-        multiple of 8 elements, a head has a multiple of 16 up to the largest attention tile."""
+        multiple of 8 elements, a head has a multiple of 16 up to the largest attention tile, a normalised row
+        and a row of q, k and v that is rotated and written to the cache fit a block's row buffer."""
         for name, k in reductions:
             if k <= 0 or k % 8:
                 raise KernelError(f"{what}: {name} = {k} must be a positive multiple of 8 (the products sum over it in 16-byte chunks)")
+        if norm_width is not None and not 0 < norm_width <= self._core.ms_max_norm_width():
+            raise KernelError(f"{what}: width {norm_width} is outside what the norm kernel takes (1 to {self._core.ms_max_norm_width()})")
+        if rotated_row is not None and not 0 < rotated_row <= self._core.ms_max_rope_row():
+            raise KernelError(f"{what}: (heads + 2 x key/value heads) x head size = {rotated_row} is outside what the rotation "
+                              f"kernel takes (1 to {self._core.ms_max_rope_row()})")
         if head_dim is not None:
             try:
                 build.attention_tile_for(head_dim)

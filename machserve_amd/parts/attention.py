@@ -25,8 +25,10 @@ class Attention(Mixer):
         if s.heads % s.kv_heads:
             raise ValueError(f"attention: {s.heads} heads are not a multiple of {s.kv_heads} key/value heads")
         self.nq, self.nkv = s.heads * s.head_dim, s.kv_heads * s.head_dim
-        require_kernel_sizes(rt, "attention", [("hidden size", s.hidden), ("heads x head size", self.nq)], s.head_dim)
-        self.scale = float(s.head_dim) ** -0.5
+        require_kernel_sizes(rt, "attention", [("hidden size", s.hidden), ("heads x head size", self.nq)], s.head_dim,
+                             rotated_row=self.nq + (2 * self.nkv if s.kv_source is None else 0))
+        scale = getattr(s, "scale", None)
+        self.scale = float(s.head_dim) ** -0.5 if scale is None else float(scale)
         self.position = POSITION_ENCODINGS.build(s.position, rt) if s.position is not None else None
         self.writes_cache = s.kv_source is None
         self.group = None

@@ -165,12 +165,14 @@ class PendingNorm:
         return self.stream.ops.linear_swiglu(self.tensor(), w_gate_up, intermediate)
 
 
-def require_kernel_sizes(rt: "Runtime", what: str, reductions=(), head_dim: Optional[int] = None) -> None:
+def require_kernel_sizes(rt: "Runtime", what: str, reductions=(), head_dim: Optional[int] = None,
+                         norm_width: Optional[int] = None, rotated_row: Optional[int] = None) -> None:
     """Lets the kernels refuse sizes they do not take while the model is built, with the size's name
-    (``reductions``: pairs of name and size that products sum over), rather than at the first step."""
+    (``reductions``: pairs of name and size that products sum over; ``norm_width``: the width of a row that is
+    normalised; ``rotated_row``: the width of a row of q, k and v), rather than at the first step."""
     check = getattr(rt.ops, "require_sizes", None)
     if check is not None:
-        check(what, reductions, head_dim)
+        check(what, reductions, head_dim, norm_width, rotated_row)
 
 
 class Part:
@@ -246,14 +248,59 @@ class FeedForward(Part):
 
 
 class Block:
-    """An arrangement of a mixer, a feed-forward and their norms around the stream."""
+    """An arrangement of parts around the stream.  A block is built from its layer's spec and the runtime and
+    **builds its own parts** from the fields of that spec, which belong to it: the model around it asks only for what
+    is below, so an arrangement with other parts (a norm after each branch, one norm for parallel branches, no
+    feed-forward, two mixers side by side) is a registered class and a spec with the fields it reads, with ``block``
+    naming its kind.
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm):
-        self.mixer, self.feed_forward = mixer, feed_forward
-        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+    The defaults serve a block with at most one mixer in ``self.mixer``; a block with several overrides
+    :meth:`mixers`, and :meth:`cache_request` / :meth:`bind_cache` deal the requests and bindings out in order."""
 
-    def parts(self):
-        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+    mixer: Optional[Mixer] = None
+
+    def __init__(self, spec, rt: Runtime):
+        self.spec, self.rt = spec, rt
+
+    def parts(self) -> List[Part]:
+        """Every part of the block that declares tensors (sub-parts of parts excepted: they list their own)."""
+        raise NotImplementedError
+
+    def mixers(self) -> List[Mixer]:
+        return [self.mixer] if self.mixer is not None else []
+
+    def cache_request(self):
+        """What the block's mixers ask of the cache manager: one mixer's request as it is, several mixers' requests
+        as one flat list (:meth:`bind_cache` deals the bindings back out)."""
+        ms = self.mixers()
+        if len(ms) <= 1:
+            return ms[0].cache_request() if ms else None
+        out = []
+        for m in ms:
+            r = m.cache_request()
+            out.extend(r if isinstance(r, (list, tuple)) else [r])
+        return out
+
+    def bind_cache(self, binding) -> None:
+        ms = self.mixers()
+        if len(ms) == 1:
+            ms[0].bind_cache(binding)
+            return
+        at = 0
+        for m in ms:
+            r = m.cache_request()
+            if isinstance(r, (list, tuple)):
+                m.bind_cache(binding[at:at + len(r)])
+                at += len(r)
+            else:
+                if binding[at] is not None:
+                    m.bind_cache(binding[at])
+                at += 1
+
+    @property
+    def graph_safe(self) -> bool:
+        """Whether every mixer reads nothing but device memory from the step (its steps may then be captured)."""
+        return all(getattr(m, "graph_safe", False) for m in self.mixers())
 
     def forward(self, stream: ResidualStream, ctx: StepContext) -> None:
         raise NotImplementedError

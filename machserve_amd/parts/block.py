@@ -3,11 +3,23 @@
 from __future__ import annotations
 
 from .base import Block
-from .registry import register_block
+from .registry import FEED_FORWARDS, MIXERS, NORMS, register_block
 
 
 @register_block("prenorm")
 class PreNormBlock(Block):
+    """Reads ``mixer``, ``feed_forward``, ``mixer_norm`` and ``feed_forward_norm`` of its layer's spec."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.mixer = MIXERS.build(spec.mixer, rt)
+        self.feed_forward = FEED_FORWARDS.build(spec.feed_forward, rt)
+        self.mixer_norm = NORMS.build(spec.mixer_norm, rt)
+        self.feed_forward_norm = NORMS.build(spec.feed_forward_norm, rt)
+
+    def parts(self):
+        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+
     def forward(self, stream, ctx):
         self.mixer.forward(self._input(self.mixer_norm, self.mixer, stream), stream, ctx)
         self.feed_forward.forward(self._input(self.feed_forward_norm, self.feed_forward, stream), stream, ctx)

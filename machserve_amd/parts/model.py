@@ -11,7 +11,7 @@ import torch
 
 from ..config.specs import ModelSpec
 from .base import Block, Part, ResidualStream, Runtime, StepContext, TensorDecl, require_kernel_sizes
-from .registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, register_embedding, register_head
+from .registry import BLOCKS, EMBEDDINGS, HEADS, NORMS, register_embedding, register_head
 
 
 @register_embedding("embedding")
@@ -68,10 +68,8 @@ class DecoderModel:
         require_kernel_sizes(rt, "output head", [("width", spec.embedding.width)])
         self.embedding = EMBEDDINGS.build(spec.embedding, rt)
         self.blocks: List[Block] = []
-        for layer in spec.layers:
-            block_cls = BLOCKS.get(layer.block)
-            self.blocks.append(block_cls(MIXERS.build(layer.mixer, rt), FEED_FORWARDS.build(layer.feed_forward, rt),
-                                         NORMS.build(layer.mixer_norm, rt), NORMS.build(layer.feed_forward_norm, rt)))
+        for layer in spec.layers:  # a block builds its own parts from the fields of its layer's spec
+            self.blocks.append(BLOCKS.get(layer.block)(layer, rt))
         self.order = list(spec.order)
         self.final_norm = NORMS.build(spec.final_norm, rt)
         self.head = HEADS.build(spec.head, rt, self.embedding)
@@ -104,7 +102,7 @@ class DecoderModel:
 
         out = []
         for p, i in enumerate(self.order):
-            req = self.blocks[i].mixer.cache_request()
+            req = self.blocks[i].cache_request()
             out.append([placed(r, p, i) for r in req] if isinstance(req, (list, tuple)) else placed(req, p, i))
         return out
 
@@ -112,17 +110,17 @@ class DecoderModel:
         self._bindings = [device_cache.binding(p) for p in range(len(self.order))]
         for p, i in enumerate(self.order):  # a layer that runs once keeps its binding for good
             if self._bindings[p] is not None:
-                self.blocks[i].mixer.bind_cache(self._bindings[p])
+                self.blocks[i].bind_cache(self._bindings[p])
         self._rebind = len(set(self.order)) != len(self.order)
 
     def attention_rows_per_token(self) -> List[int]:
-        return sorted({g for g in (b.mixer.attention_rows_per_token() for b in self.blocks) if g})
+        return sorted({g for b in self.blocks for m in b.mixers() for g in [m.attention_rows_per_token()] if g})
 
     def attention_rows_per_block(self) -> Optional[int]:
         """The unit of the attention work lists, which every mixer's kernel must share (the lists are made
         once per step); None if no mixer wants them."""
-        units = {(u, type(b.mixer).__name__, getattr(b.mixer.spec, "head_dim", None))
-                 for b in self.blocks for u in [b.mixer.attention_rows_per_block()] if u}
+        units = {(u, type(m).__name__, getattr(m.spec, "head_dim", None))
+                 for b in self.blocks for m in b.mixers() for u in [m.attention_rows_per_block()] if u}
         if len({u for u, _, _ in units}) > 1:
             raise ValueError("the mixers' attention kernels take blocks of different numbers of rows: "
                              + ", ".join(f"{name} (head size {hd}): {u}" for u, name, hd in sorted(units)))
@@ -143,7 +141,7 @@ class DecoderModel:
         stream = ResidualStream(self.embedding.forward(ctx.tokens), self.rt.ops)
         for p, i in enumerate(self.order):
             if self._rebind and self._bindings[p] is not None:
-                self.blocks[i].mixer.bind_cache(self._bindings[p])
+                self.blocks[i].bind_cache(self._bindings[p])
             self.blocks[i].forward(stream, ctx)
         if ctx.want_rows.numel() == 0:
             return None

@@ -3,12 +3,16 @@
 reads it: the norm's factor is one number a row, so a product's kernel can apply it to its finished sums."""
 from __future__ import annotations
 
-from .base import Norm, PendingNorm, TensorDecl
+from .base import Norm, PendingNorm, TensorDecl, require_kernel_sizes
 from .registry import register_norm
 
 
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        require_kernel_sizes(rt, "rmsnorm", norm_width=spec.width)
+
     def tensor_decls(self):
         return [TensorDecl("weight", (self.spec.width,), "vector")]
 

@@ -215,6 +215,42 @@ def test_decoders_never_outnumber_the_budget_and_nobody_starves():
     assert steps <= 4 * 13 // 2 + 4   # 52 tokens through a budget of two, a few half-empty steps at the seams
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_more_slots_than_budget_under_random_arrivals_and_preemptions(seed):
+    """More requests may run than a step holds tokens, pages are short and requests arrive at random: in every
+    plan the decoding requests fit the budget (the core refuses a plan that would break this before it has
+    preempted anybody), every step runs something, and all requests finish."""
+    rng = random.Random(100 + seed)
+    budget = rng.choice([2, 3, 5])
+    s = _scheduler(pages=rng.randint(5, 9), page_size=16, max_batch_tokens=budget, chunk_size=rng.choice([None, 2]), slots=8)
+    want, queue = {}, [(rng.randint(1, 40), rng.randint(1, 30), rng.randrange(0, 60)) for _ in range(14)]
+    queue.sort(key=lambda q: q[2])
+    steps = preempted = 0
+    while queue or s.has_work():
+        while queue and (queue[0][2] <= steps or not s.has_work()):
+            n, m, _ = queue.pop(0)
+            want[s.add([rng.randrange(50) for _ in range(n)], m)] = m
+        p = s.schedule()
+        assert p.items and p.n_tokens <= budget
+        assert sum(r.decoding for r in s.running) <= budget
+        preempted += len(p.preempted)
+        _run_plan(s, p, token=rng.randrange(50))
+        s.cache.check()
+        steps += 1
+        assert steps < 5000
+    assert {i: len(r.generated) for i, r in s.finished.items()} == want
+    _PREEMPTED.append(preempted)
+
+
+_PREEMPTED = []
+
+
+def test_the_random_arrivals_above_did_preempt():
+    if not _PREEMPTED:
+        pytest.skip("the test above did not run in this process")
+    assert sum(_PREEMPTED) > 0
+
+
 def test_a_window_group_is_sized_by_its_window_not_by_the_request():
     """A long request on a model whose layers all see a window needs pages for window + portion keys
     only: it is admitted with a pool far smaller than its length, and runs to the end."""
@@ -262,10 +298,77 @@ def test_random_load_always_finishes(seed):
     assert {i: len(r.generated) for i, r in s.finished.items()} == want
 
 
+def test_pages_by_need_give_a_window_group_what_its_requests_can_hold_and_the_bytes_follow(tmp_path):
+    """A model whose later layers see a window: with the rule, the window group's pool holds what its requests can
+    hold of it at a time, not the whole pool once more; a dict names each group's pages; the device cache's byte
+    count is pages + 1 (the scratch page) times the layers' page bytes; and the engine still equals the plain model."""
+    from machserve_amd.cache import CacheError, CacheManager, pages_by_need
+    from machserve_amd.engine import Engine, load_model
+    from machserve_amd.parts import PagedKVRequest
+    reqs = [PagedKVRequest(2, 16), PagedKVRequest(2, 16, 40), PagedKVRequest(2, 16, 40)]
+    m = CacheManager(reqs, 16, pages_by_need(max_tokens=4096, max_requests=3, portion=24, page_size=16), 3)
+    # all keys: 4096 / 16; window 40 + portion 24 - 1 = 63 keys touch at most 4 + 1 pages a request
+    assert {n: g.pool.num_pages for n, g in m.groups.items()} == {"full": 256, "window40": 3 * 5}
+    m = CacheManager(reqs, 16, {"full": 7, "window40": 3}, 3)
+    assert {n: g.pool.num_pages for n, g in m.groups.items()} == {"full": 7, "window40": 3}
+    with pytest.raises(CacheError, match="window40"):
+        CacheManager(reqs, 16, {"full": 7}, 3)
+    with pytest.raises(CacheError, match="nobody"):
+        CacheManager(reqs, 16, {"full": 7, "window40": 3, "nobody": 1}, 3)
+    d = make_model_dir(tmp_path, "C")     # configuration C has layers that see a window
+    w, sizes = read_for_plain(d)
+    lm = load_model(d, dtype="float32", device="cpu", page_size=16, max_tokens=320, max_requests=2, portion=16, ops=EmulatedOps())
+    windows = {g.spec.window for g in lm.cache.groups.values()}
+    assert None in windows and len(windows) == 2, "configuration C must have both kinds of layers"
+    want_bytes = 0
+    for g in lm.cache.groups.values():
+        pages = 320 // 16 if g.spec.window is None else min(20, 2 * (-(-(g.spec.window + 15) // 16) + 1))
+        assert g.pool.num_pages == pages
+        want_bytes += len(g.spec.layers) * (pages + 1) * 2 * g.spec.kv_heads * 16 * g.spec.head_dim * 4
+    assert lm.device_cache.bytes() == want_bytes
+    assert lm.device_cache.bytes() < sum(len(g.spec.layers) for g in lm.cache.groups.values()) * 21 * 2 * 16 * 4 * max(
+        g.spec.kv_heads * g.spec.head_dim for g in lm.cache.groups.values())
+    eng = Engine(lm, max_batch_tokens=16, max_running=2)
+    prompts = [random_prompt(n, sizes["vocab"], 70 + n) for n in (90, 33)]
+    got = eng.generate(prompts, max_new=8)
+    for p, g in zip(prompts, got):
+        assert g == P.greedy_generate(w, sizes, p, 8)
+
+
+def test_a_refused_step_takes_no_pages(tmp_path):
+    """A step with a bad token, a slot twice, a place beyond its tokens, or a slot that no request holds is refused
+    before anything is taken: the tables, the free pages and the lengths are what they were."""
+    from machserve_amd.engine import StepEntry, StepError, load_model
+    d = make_model_dir(tmp_path, "A")
+    lm = load_model(d, dtype="float32", device="cpu", page_size=16, num_pages=6, max_requests=3, ops=EmulatedOps())
+    a, b = lm.cache.admit(), lm.cache.admit()
+    lm.step([StepEntry(a, [1, 2, 3], [2]), StepEntry(b, [4] * 17, [])])
+    free, lengths, tables = lm.cache.free_pages(), dict(lm.cache.lengths), [lm.cache.table("full", s) for s in (a, b)]
+    bad = [
+        [StepEntry(a, [5] * 20, []), StepEntry(b, [512], [0])],               # a token outside the vocabulary, after a good entry
+        [StepEntry(a, [5] * 20, []), StepEntry(a, [1], [0])],                  # a slot twice
+        [StepEntry(a, [5] * 20, [20])],                                        # a wanted place beyond the tokens
+        [StepEntry(a, [5] * 20, []), StepEntry(2, [1], [0])],                  # a slot nobody holds
+        [StepEntry(a, [5] * 20, []), StepEntry(b, [], [])],                    # an empty entry
+        [StepEntry(a, [5] * 300, [])],                                         # beyond the model's positions
+    ]
+    for entries in bad:
+        with pytest.raises(StepError):
+            lm.step(entries)
+        lm.cache.check()
+        assert lm.cache.free_pages() == free and dict(lm.cache.lengths) == lengths
+        assert [lm.cache.table("full", s) for s in (a, b)] == tables
+    # and the step function still works
+    out = lm.step([StepEntry(a, [5] * 20, [19])])
+    assert out.shape == (1, 512) and lm.cache.length(a) == 23
+
+
 # ---------------------------------------------------------------------------- engine on the CPU stand-ins
 
-@pytest.mark.parametrize("which,pages,budget", [("A", 8, 512), ("A", 5, 12), ("B", 6, 24), ("C", 16, 32)])
-def test_engine_generations_equal_plain_greedy(tmp_path, which, pages, budget):
+@pytest.mark.parametrize("which,pages,budget,runs_out", [("A", 8, 512, False), ("A", 5, 12, False), ("A", 3, 64, True),
+                                                          ("B", 6, 24, False), ("B", 3, 64, True), ("C", 16, 32, False),
+                                                          ("C", 3, 32, True)])
+def test_engine_generations_equal_plain_greedy(tmp_path, which, pages, budget, runs_out):
     """The reference's central test (crates/mach-model/tests/continuous.rs:80-97, 216-247,
     393-427): what the engine generates equals single-request greedy generation, token for
     token, also when prompts are cut, requests wait for a slot, and pages run out."""
@@ -275,14 +378,18 @@ def test_engine_generations_equal_plain_greedy(tmp_path, which, pages, budget):
     ps = {"A": 16, "B": 32, "C": 16}[which]
     lm = load_model(d, dtype="float32", device="cpu", page_size=ps, num_pages=pages, max_requests=3, ops=EmulatedOps())
     eng = Engine(lm, max_batch_tokens=budget)
-    prompts = [random_prompt(n, sizes["vocab"], 40 + n) for n in (5, 17, 33, 9)]
-    got = eng.generate(prompts, max_new=8)
-    for p, g in zip(prompts, got):
-        assert g == P.greedy_generate(w, sizes, p, 8)
+    # when pages are to run out: three prompts that fill a page each, so that their decoded tokens need a second one
+    # at about the same time, from a pool of three
+    lengths = (ps - 1, ps - 2, ps, 9) if runs_out else (5, 17, 33, 9)
+    prompts = [random_prompt(n, sizes["vocab"], 40 + n) for n in lengths]
+    ids = [eng.add(p, 8) for p in prompts]
+    done = eng.run()
+    for p, i in zip(prompts, ids):
+        assert done[i].generated == P.greedy_generate(w, sizes, p, 8)
     lm.cache.check()
     assert all(g.pool.available() == g.pool.num_pages for g in lm.cache.groups.values())
-    if pages <= 6:
-        assert any(r.preemptions for r in eng.scheduler.finished.values()) or True
+    preemptions = sum(done[i].preemptions for i in ids)
+    assert (preemptions > 0) == runs_out, f"{preemptions} preemptions with {pages} pages"
 
 
 def test_engine_sampling_is_deterministic_and_survives_preemption(tmp_path):

@@ -94,6 +94,20 @@ def test_sizes_the_kernels_do_not_take_are_refused_when_the_model_is_built(tmp_p
         load_model(d, dtype="bfloat16", device=DEV, page_size=16, num_pages=4)
 
 
+def test_rows_too_wide_for_the_norm_and_the_rotation_are_refused_when_the_part_is_built():
+    """The norm and the rotation kernels hold a row in a block's LDS: a wider one is refused when the part is built,
+    with the size, not at the first step."""
+    from machserve_amd.config import AttentionSpec, NormSpec, RotarySpec
+    from machserve_amd.parts import MIXERS, NORMS
+    rt = _runtime(torch.bfloat16)
+    most = rt.ops._core.ms_max_norm_width()
+    NORMS.build(NormSpec("rmsnorm", most, 1e-6), rt)
+    with pytest.raises(Exception, match=f"width {most + 8}"):
+        NORMS.build(NormSpec("rmsnorm", most + 8, 1e-6), rt)
+    with pytest.raises(Exception, match=r"head size = 15360"):
+        MIXERS.build(AttentionSpec("attention", 1024, 100, 10, 128, RotarySpec("rotary", 128, 1e4)), rt)
+
+
 def test_eos_stops_generation(dirs):
     import machserve_amd
     w, sizes = read_for_plain(dirs["A"])
@@ -149,6 +163,19 @@ def test_random_arrivals_under_page_pressure_equal_the_plain_model(dirs, which, 
         assert len(done[rid].generated) == max_new
         assert_greedy(w, sizes, prompt, done[rid].generated, dtype, f"request {rid} ({len(prompt)} tokens, {max_new} new)")
     print(f"seed {seed}: {step} steps, {sum(done[r].preemptions for r in ids)} preemptions")
+    _PREEMPTIONS[(which, dtype, seed)] = sum(done[r].preemptions for r in ids)
+
+
+_PREEMPTIONS = {}
+
+
+def test_the_random_arrivals_did_run_out_of_pages():
+    """The seeds above are there for what happens when pages run out: over all of them (at least those that ran in
+    this process before this test) some request must have been preempted, and in both element types."""
+    if not _PREEMPTIONS:
+        pytest.skip("the random-arrival tests did not run in this process")
+    for dtype in {k[1] for k in _PREEMPTIONS}:
+        assert sum(n for k, n in _PREEMPTIONS.items() if k[1] == dtype) > 0, f"no preemption in any {dtype} run: {_PREEMPTIONS}"
 
 
 def test_captured_steps_are_dropped_and_captured_again(dirs):
@@ -526,17 +553,17 @@ def test_block_arrangement_alone(dtype):
     sizes: x += mixer(norm(x)); x += feed_forward(norm(x))
     (crates/mach-model/src/batched.rs:3180-3200).  A portion and single tokens against the plain parts."""
     from machserve_amd.cache import CacheManager, DeviceCache
-    from machserve_amd.config import AttentionSpec, GatedMlpSpec, NormSpec, RotarySpec
+    from machserve_amd.config import AttentionSpec, GatedMlpSpec, LayerSpec, NormSpec, RotarySpec
     from machserve_amd.engine.step import StepEntry, StepFunction
-    from machserve_amd.parts import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, ResidualStream
+    from machserve_amd.parts import BLOCKS, ResidualStream
     rt = _runtime(dtype)
     H, KV, hd, d, I, T, eps = 3, 1, 48, 112, 136, 40, 1e-5
     names = {k: k for k in ("q.weight", "k.weight", "v.weight", "o.weight", "q.bias", "k.bias", "v.bias")}
-    mixer = MIXERS.build(AttentionSpec("attention", d, H, KV, hd, RotarySpec("rotary", hd, 5e4), tensors=names), rt)
-    ff = FEED_FORWARDS.build(GatedMlpSpec("gated_mlp", d, I), rt)
-    n1, n2 = NORMS.build(NormSpec("rmsnorm", d, eps), rt), NORMS.build(NormSpec("rmsnorm", d, eps), rt)
-    block = BLOCKS.get("prenorm")(mixer, ff, n1, n2)
-    assert block.parts() == [n1, mixer, n2, ff]
+    layer = LayerSpec("prenorm", AttentionSpec("attention", d, H, KV, hd, RotarySpec("rotary", hd, 5e4), tensors=names),
+                      GatedMlpSpec("gated_mlp", d, I), NormSpec("rmsnorm", d, eps), NormSpec("rmsnorm", d, eps))
+    block = BLOCKS.get(layer.block)(layer, rt)   # the arrangement builds its own parts from the layer's spec
+    n1, mixer, n2, ff = block.parts()
+    assert (mixer, ff, n1, n2) == (block.mixer, block.feed_forward, block.mixer_norm, block.feed_forward_norm)
     g = torch.Generator().manual_seed(11)
     r = lambda *s: torch.randn(*s, generator=g) * 0.1
     t = {"q.weight": r(H * hd, d), "k.weight": r(KV * hd, d), "v.weight": r(KV * hd, d), "o.weight": r(d, H * hd),
@@ -545,9 +572,9 @@ def test_block_arrangement_alone(dtype):
     t = {k: (v.to(dtype) if v is not None and v.dim() == 2 else v) for k, v in t.items()}
     dev = {k: (v.to(DEV) if v is not None else None) for k, v in t.items()}
     mixer.load(dev), ff.load(dev), n1.load({"weight": dev["n1"]}), n2.load({"weight": dev["n2"]})
-    cache = CacheManager([mixer.cache_request()], 16, 4, 1)
+    cache = CacheManager([block.cache_request()], 16, 4, 1)
     dc = DeviceCache(cache, dtype, rt.device)
-    mixer.bind_cache(dc.binding(0))
+    block.bind_cache(dc.binding(0))
 
     class OneLayer:
         vocab = 100

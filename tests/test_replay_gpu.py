@@ -175,7 +175,7 @@ def test_mixed_with_page_reuse(models, which, dtype):
     state = {}  # request -> [slot, fed]
     waiting = list(range(len(seqs)))
     portion = [9, 2, 17, 5]
-    step, reused = 0, set()
+    step, used = 0, []
     first_pages = None
     while waiting or state:
         while waiting and len(state) < live_cap:
@@ -205,7 +205,7 @@ def test_mixed_with_page_reuse(models, which, dtype):
             got[r].append(logits[k:k + n])
             k += n
             state[r][1] += n
-            reused.update(lm.cache.table(next(iter(lm.cache.groups)), state[r][0]))
+            used.append((r, frozenset(p for p in lm.cache.table(next(iter(lm.cache.groups)), state[r][0]) if p >= 0)))
             if state[r][1] == len(seqs[r]):
                 lm.cache.release(state.pop(r)[0])
         step += 1
@@ -213,6 +213,11 @@ def test_mixed_with_page_reuse(models, which, dtype):
     assert all(g.pool.available() == g.pool.num_pages for g in lm.cache.groups.values())
     total_pages = sum(-(-len(s) // ps) for s in seqs)
     assert total_pages > pages, "the trace must need more pages than the pool has"
+    owners = {}
+    for r, held in used:
+        for p in held:
+            owners.setdefault(p, set()).add(r)
+    assert max(len(o) for o in owners.values()) >= 2, "some page must have served two requests, one after the other"
     for r in range(len(seqs)):
         check(torch.cat(got[r]), refs[r], dtype, f"{which} request {r} mixed")
 

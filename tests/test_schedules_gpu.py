@@ -1,0 +1,175 @@
+"""Schedules at the far ends of what the engine runs: dozens of requests decoding side by side (the buckets of 48 and
+64 rows, every product in the tiled kernel, the norm that adds many pending planes, split keys, sampling of all
+rows inside the captured step), one request tens of thousands of positions long, and temperature sampling end to
+end; every logit and every token against the plain model
+(crates/mach-model/tests/continuous.rs:80-97, 393-427: the engine's tokens equal one request's alone)."""
+import pytest
+import torch
+
+from gpu_util import DEV
+from plain import qwen2_plain as P
+from tiny_configs import CONFIGS, TINY_A, make_model_dir, random_prompt, read_for_plain
+
+pytestmark = pytest.mark.gpu
+
+
+def _stored(w, dtype):
+    return w if dtype == torch.float32 else {k: v.to(dtype).float() if v.dim() == 2 else v for k, v in w.items()}
+
+
+def _bound(dtype, scale):
+    return 2e-5 + 2e-5 * scale if dtype == torch.float32 else 3e-2 * scale
+
+
+def _many_decoders(lm, w, sizes, dtype, n, lengths, steps, vocab, captured):
+    """``n`` requests with prompts of ``lengths`` (in turn) are fed, a few prompts a step; then all decode side by side
+    for ``steps`` steps with given tokens, and once more with the sampler inside the step.  Every logit of the
+    prompts' ends and of the decoded positions against the plain model."""
+    from machserve_amd.engine import StepEntry
+    if captured:
+        lm.step.DECODE_CAPTURE_AFTER = 0   # capture at once: the test has only a few steps
+    seqs = [random_prompt(lengths[i % len(lengths)] + steps + 1, vocab, 500 + i) for i in range(n)]
+    fed = [lengths[i % len(lengths)] for i in range(n)]
+    ww = _stored(w, dtype)
+    refs = [P.forward(ww, sizes, s) for s in seqs]
+    slots = [lm.cache.admit() for _ in range(n)]
+    worst = 0.0
+
+    def compare(logits, who):
+        nonlocal worst
+        got = logits.float().cpu()
+        for row, r in enumerate(who):
+            ref = refs[r][fed[r] - 1]
+            err = (got[row] - ref).abs().max().item()
+            assert err <= _bound(dtype, ref.abs().max().item()), f"request {r} at position {fed[r] - 1}: error {err:.3e}"
+            worst = max(worst, err)
+
+    for first in range(0, n, 8):   # prompts, eight requests a step
+        who = list(range(first, min(first + 8, n)))
+        compare(lm.step([StepEntry(slots[r], seqs[r][:fed[r]], [fed[r] - 1]) for r in who]), who)
+    everyone = list(range(n))
+    for _ in range(steps):
+        entries = [StepEntry(slots[r], [seqs[r][fed[r]]], [0]) for r in everyone]
+        for r in everyone:
+            fed[r] += 1
+        compare(lm.step(entries), everyone)
+    if captured:
+        assert lm.step.use_graphs and any(len(k[0]) >= n and set(k[0]) == {1} for k in lm.step._graphs), \
+            "the decode steps must have run from a captured graph"
+        # one more step with the sampler inside the captured step: greedy rows and rows at a temperature
+        temps = [0.0 if r % 2 == 0 else 0.7 for r in everyone]
+        states = [1000 + r for r in everyone]
+        entries = [StepEntry(slots[r], [seqs[r][fed[r]]], [0]) for r in everyone]
+        for r in everyone:
+            fed[r] += 1
+        out = lm.step.decode_and_sample(entries, temps, [0] * n, [1.0] * n, states)
+        assert out is not None, "a decode step of plain sampling takes the captured path"
+        tokens, _ = out
+        for r in everyone:
+            ref = refs[r][fed[r] - 1]
+            if dtype == torch.float32 and temps[r] > 0:
+                # The draw is the first token whose cumulated probability exceeds u * total (crates/mach-model/src/
+                # sampling.rs:1259-1270).  Over a flat row of 150,000 tokens the 32-bit sums of the kernel's segments and of
+                # a walk in index order differ in rounding by more than one token's share, so the token is held to the
+                # target in mass: the target lies within 1e-4 of the total of the token's own interval.  (Token for token
+                # equality is held at the small vocabularies, where a token's share is far above the rounding.)
+                u, _ = P.next_uniform(states[r])
+                p = torch.exp((ref.double() - ref.double().max()) / temps[r])
+                cum, total = torch.cumsum(p, 0), p.sum().item()
+                tok = tokens[r]
+                assert cum[tok].item() > u * total - 1e-4 * total and (cum[tok] - p[tok]).item() <= u * total + 1e-4 * total, \
+                    f"request {r}: token {tok} covers {((cum[tok] - p[tok]) / total).item():.6f}..{(cum[tok] / total).item():.6f}, u = {u:.6f}"
+                if vocab <= 4096:
+                    want, _ = P.sample(ref.numpy(), temps[r], 0, 1.0, states[r])
+                    assert tok == want, f"request {r}: sampled {tok}, the plain draw is {want}"
+            elif temps[r] == 0:
+                assert ref[tokens[r]] >= ref.max() - _bound(dtype, ref.abs().max().item()), f"request {r}: greedy token {tokens[r]}"
+    else:
+        assert not lm.step._graphs
+    for s in slots:
+        lm.cache.release(s)
+    lm.cache.check()
+    return worst
+
+
+@pytest.mark.parametrize("captured", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n", [40, 64])
+def test_dozens_of_requests_decode_side_by_side_tiny(tmp_path, n, dtype, captured):
+    from machserve_amd.engine import load_model
+    d = make_model_dir(tmp_path, "B")
+    w, sizes = read_for_plain(d)
+    lm = load_model(d, dtype=dtype, device=DEV, page_size=16, num_pages=n * 4 + 8, max_requests=n, use_graphs=captured)
+    _many_decoders(lm, w, sizes, dtype, n, (1, 7, 15, 16, 17, 30, 33, 40), 6, sizes["vocab"], captured)
+
+
+@pytest.mark.parametrize("captured", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_dozens_of_requests_decode_side_by_side_at_real_layer_sizes(dtype, captured):
+    """The layer sizes of Qwen2.5-0.5B with two layers: the path that the benchmark's 64-request point runs on."""
+    from machserve_amd.config import config_from_dict
+    from machserve_amd.engine import load_model
+    from machserve_amd.weights import random_tensor_dict
+    raw = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 2, "max_position_embeddings": 4096,
+           "rms_norm_eps": 1e-6, "rope_theta": 1000000.0, "hidden_act": "silu", "hidden_size": 896, "num_attention_heads": 14,
+           "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936, "tie_word_embeddings": True}
+    cfg = config_from_dict(raw)
+    tensors = random_tensor_dict(cfg, 3)
+    n = 64 if captured else 40
+    lm = load_model(config=cfg, tensors=tensors, dtype=dtype, device=DEV, page_size=64, num_pages=n + 4, max_requests=n,
+                    use_graphs=captured)
+    _many_decoders(lm, tensors, P.sizes_from_config(raw), dtype, n, (1, 2, 3, 5, 8), 6, cfg.vocab_size, captured)
+
+
+@pytest.mark.timeout(400)   # the plain model walks 20,000 rows of four heads one by one
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_twenty_thousand_positions(tmp_path, dtype):
+    """One request of 20,480 prompt tokens in portions of 4,096 and then eight decoded tokens: block tables 320
+    pages wide, dozens of key splits, rotation angles of tens of thousands of radians.  Logits at the portions'
+    ends and middles and at every decoded position."""
+    from machserve_amd.engine import StepEntry, load_model
+    from machserve_amd.weights import write_random_model
+    raw = dict(TINY_A, max_position_embeddings=32768, rope_theta=1000000.0)
+    d = write_random_model(raw, 4, str(tmp_path / "long"))
+    w, sizes = read_for_plain(d)
+    toks = random_prompt(20488, 512, 6)
+    ref = P.forward(_stored(w, dtype), sizes, toks)
+    lm = load_model(d, dtype=dtype, device=DEV, page_size=64, num_pages=324)
+    slot = lm.cache.admit()
+    got, where, i = [], [], 0
+    for c in (4096,) * 5:
+        want = [0, c // 2, c - 1]
+        got.append(lm.step([StepEntry(slot, toks[i:i + c], want)]))
+        where += [i + k for k in want]
+        i += c
+    for j in range(20480, 20488):
+        got.append(lm.step([StepEntry(slot, [toks[j]], [0])]))
+        where.append(j)
+    got = torch.cat(got).float().cpu()
+    scale = ref.abs().max().item()
+    # 32-bit: the same bound as at 5,000 positions (sums over thousands of keys in another order)
+    allowed = 1e-4 + 1e-4 * scale if dtype == torch.float32 else 3e-2 * scale
+    err = (got - ref[where]).abs().max().item()
+    assert err <= allowed, f"max error {err:.3e}, allowed {allowed:.3e}"
+    if dtype == torch.float32:
+        assert torch.equal(got.argmax(-1), ref[where].argmax(-1))
+
+
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_temperature_sampling_through_the_entry_point_equals_the_plain_draws(tmp_path, which):
+    """``generate`` with a temperature and top-p in 32-bit: every request's tokens are the CPU mirror's draws
+    (crates/mach-model/src/sampling.rs:1169-1274) on the plain model's logits, seed by seed."""
+    import machserve_amd
+    d = make_model_dir(tmp_path, which)
+    w, sizes = read_for_plain(d)
+    prompts = [random_prompt(n, sizes["vocab"], 300 + n) for n in (4, 21, 35)]
+    got = machserve_amd.generate(d, prompts, max_new=6, dtype="float32", temperature=0.8, top_p=0.9, seed=41, page_size=16,
+                                 capacity=3, max_batch_tokens=32)
+    for i, (p, g) in enumerate(zip(prompts, got)):
+        seq, state = list(p), 41 + i
+        for n, tok in enumerate(g):
+            want, state = P.sample(P.forward(w, sizes, seq)[-1].numpy(), 0.8, 0, 0.9, state)
+            assert tok == want, f"request {i}, token {n}: the engine drew {tok}, the plain model's draw is {want}"
+            seq.append(tok)
+    greedy = machserve_amd.generate(d, prompts, max_new=6, dtype="float32", page_size=16)
+    assert greedy != got, "the test must tell a draw from the most likely token"

@@ -14,8 +14,9 @@ from plain import qwen2_plain as P
 
 from machserve_amd.config import (AttentionSpec, EmbeddingSpec, GatedMlpSpec, HeadSpec, LayerSpec, ModelSpec, NormSpec,
                                   RotarySpec, register_architecture)
-from machserve_amd.parts import (FeedForward, Head, Mixer, PagedKVRequest, PositionEncoding, StateRequest, TensorDecl,
-                                 register_feed_forward, register_head, register_mixer, register_position_encoding)
+from machserve_amd.parts import (FEED_FORWARDS, MIXERS, NORMS, Block, FeedForward, Head, Mixer, PagedKVRequest, PositionEncoding,
+                                 ResidualStream, StateRequest, TensorDecl, register_block, register_feed_forward, register_head,
+                                 register_mixer, register_position_encoding)
 
 WIDTH, HEADS, KV, HD, INTER, VOCAB = 48, 3, 1, 16, 80, 90
 EXPERTS, EXPERT_INTER = 3, 24
@@ -467,6 +468,150 @@ def test_a_mixer_with_state_is_captured_filled_up_and_launched_ahead():
     lm = _generate_graph_toy("cuda:0", None, 60)
     assert lm.step.use_graphs and len(lm.step._graphs) >= 1
     assert any(k[0] == (1, 1, 1, 1) for k in lm.step._graphs), "a step of three requests is captured as one of four rows"
+
+
+# ---------------------------------------------------------------------------- toy arrangements of a block
+
+@dataclass(frozen=True)
+class SandwichSpec:
+    """A layer whose two branches are normalised before *and after*: four norms, and a softmax scale of its own."""
+    block: str
+    mixer: object
+    feed_forward: object
+    norms: tuple   # before the mixer, after it, before the feed-forward, after it
+
+
+@register_block("toy_sandwich")
+class Sandwich(Block):
+    """x += norm(mixer(norm(x))); x += norm(feed_forward(norm(x))): the arrangement builds its four norms and its two
+    branches from the fields of its own spec; each branch adds into a stream of its own that starts at zero."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.mixer = MIXERS.build(spec.mixer, rt)
+        self.feed_forward = FEED_FORWARDS.build(spec.feed_forward, rt)
+        self.norms = [NORMS.build(n, rt) for n in spec.norms]
+
+    def parts(self):
+        return self.norms + [self.mixer, self.feed_forward]
+
+    def forward(self, stream, ctx):
+        for before, branch_part, after in ((self.norms[0], self.mixer, self.norms[1]),
+                                           (self.norms[2], self.feed_forward, self.norms[3])):
+            branch = ResidualStream(torch.zeros_like(stream.value()), stream.ops)
+            branch_part.forward(before.forward(stream), branch, ctx)
+            stream.add(after.forward(branch).float())
+
+
+@dataclass(frozen=True)
+class MixerOnlySpec:
+    block: str
+    mixer: object
+    norm: object
+
+
+@register_block("toy_mixer_only")
+class MixerOnly(Block):
+    """x += mixer(norm(x)) and nothing else: a layer without a feed-forward."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.mixer, self.norm = MIXERS.build(spec.mixer, rt), NORMS.build(spec.norm, rt)
+
+    def parts(self):
+        return [self.norm, self.mixer]
+
+    def forward(self, stream, ctx):
+        self.mixer.forward(self.norm.forward(stream), stream, ctx)
+
+
+SANDWICH_SCALE = 0.11   # not HD ** -0.5 = 0.25
+
+
+@dataclass
+class SandwichToyConfig:
+    @classmethod
+    def from_dict(cls, raw):
+        return cls()
+
+    def to_spec(self):
+        norm = lambda name: NormSpec("rmsnorm", WIDTH, 1e-5, {"weight": name})
+        names = lambda i: {k: f"l{i}.att.{k}" for k in ("q.weight", "k.weight", "v.weight", "o.weight", "q.bias", "k.bias", "v.bias")}
+        att0 = AttentionSpec("attention", WIDTH, HEADS, KV, HD, RotarySpec("rotary", HD, 1e4), tensors=names(0), scale=SANDWICH_SCALE)
+        ff0 = GatedMlpSpec("gated_mlp", WIDTH, INTER, "silu", {k: f"l0.ff.{k}" for k in ("gate.weight", "up.weight", "down.weight")})
+        layers = (SandwichSpec("toy_sandwich", att0, ff0, (norm("l0.n1"), norm("l0.n2"), norm("l1.n1"), norm("l1.n2"))),
+                  MixerOnlySpec("toy_mixer_only", AttentionSpec("attention", WIDTH, HEADS, KV, HD, RotarySpec("rotary", HD, 1e4),
+                                                                tensors=names(2)), norm("l2.n1")))
+        return ModelSpec("SandwichToyForCausalLM", EmbeddingSpec(VOCAB, WIDTH, {"weight": "emb"}), layers, order=(0, 1, 0),
+                         final_norm=norm("nf"), head=HeadSpec(VOCAB, WIDTH, True), max_positions=512)
+
+
+register_architecture("SandwichToyForCausalLM", SandwichToyConfig)
+
+
+def plain_sandwich_toy(t, toks, scale0=SANDWICH_SCALE):
+    T = len(toks)
+    pos = torch.arange(T)
+    x = t["emb"][torch.tensor(toks)]
+
+    def att(i, xn, scale):
+        q = P.rope(P.linear(xn, t[f"l{i}.att.q.weight"], t[f"l{i}.att.q.bias"]).view(T, HEADS, HD), pos, 1e4)
+        k = P.rope(P.linear(xn, t[f"l{i}.att.k.weight"], t[f"l{i}.att.k.bias"]).view(T, KV, HD), pos, 1e4)
+        v = P.linear(xn, t[f"l{i}.att.v.weight"]).view(T, KV, HD)
+        # the plain attention scales by HD ** -0.5: another scale is a factor on the queries
+        o = P.attention(q * (scale / HD ** -0.5), k, v)
+        return P.linear(o.reshape(T, -1), t[f"l{i}.att.o.weight"])
+
+    for i in (0, 1, 0):
+        if i == 0:
+            x = x + P.rms_norm(att(0, P.rms_norm(x, t["l0.n1"], 1e-5), scale0), t["l0.n2"], 1e-5)
+            y = P.swiglu(P.rms_norm(x, t["l1.n1"], 1e-5), t["l0.ff.gate.weight"], t["l0.ff.up.weight"], t["l0.ff.down.weight"])
+            x = x + P.rms_norm(y, t["l1.n2"], 1e-5)
+        else:
+            x = x + att(2, P.rms_norm(x, t["l2.n1"], 1e-5), HD ** -0.5)
+    return P.linear(P.rms_norm(x, t["nf"], 1e-5), t["emb"])
+
+
+def _check_sandwich(device, ops):
+    """Blocks that build parts of their own (four norms; no feed-forward), and an attention whose scale the spec gives:
+    a request in portions beside one token by token, against the plain parts."""
+    from machserve_amd.config import config_from_dict
+    from machserve_amd.engine import StepEntry, load_model
+    t = {k: v for k, v in toy_tensors().items() if k.startswith(("emb", "nf", "l0.", "l1.n", "l2.n1", "l2.att"))}
+    lm = load_model(config=config_from_dict({"architectures": ["SandwichToyForCausalLM"]}), tensors=t, dtype=torch.float32,
+                    device=device, page_size=16, num_pages=12, max_requests=2, ops=ops)
+    assert [type(b).__name__ for b in lm.model.blocks] == ["Sandwich", "MixerOnly"]
+    assert len(lm.model.blocks[0].parts()) == 6 and lm.model.blocks[0].mixer.scale == SANDWICH_SCALE
+    gen = torch.Generator().manual_seed(5)
+    seqs = [torch.randint(0, VOCAB, (n,), generator=gen).tolist() for n in (37, 9)]
+    refs = [plain_sandwich_toy(t, s) for s in seqs]
+    slots = [lm.cache.admit() for _ in seqs]
+    cuts = [[20, 2, 6, 9], [1, 1, 1, 6]]
+    got, fed = [[], []], [0, 0]
+    for step in range(4):
+        entries = [StepEntry(slots[r], seqs[r][fed[r]:fed[r] + cuts[r][step]], list(range(cuts[r][step]))) for r in range(2)]
+        logits = lm.step(entries)
+        k = 0
+        for r in range(2):
+            n = cuts[r][step]
+            got[r].append(logits[k:k + n].float().cpu())
+            k += n
+            fed[r] += n
+    for r in range(2):
+        out = torch.cat(got[r])
+        assert (out - refs[r]).abs().max() <= 2e-4 * (1 + refs[r].abs().max()), f"request {r}"
+    # the test can tell the scale: with the usual one the plain model is far from this
+    usual = plain_sandwich_toy(t, seqs[0], HD ** -0.5)
+    assert (usual - refs[0]).abs().max() > 50 * 2e-4 * (1 + refs[0].abs().max())
+
+
+def test_blocks_that_build_their_own_parts_on_the_cpu_stand_ins():
+    _check_sandwich("cpu", EmulatedOps())
+
+
+@pytest.mark.gpu
+def test_blocks_that_build_their_own_parts_on_the_gpu():
+    _check_sandwich("cuda:0", None)
 
 
 def test_toy_model_on_the_cpu_stand_ins():
