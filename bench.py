@@ -248,7 +248,8 @@ def main() -> int:
     ap.add_argument("--page-size", type=int, default=64)
     ap.add_argument("--no-points", action="store_true", help="skip the further points and the prefill")
     ap.add_argument("--no-kernels", action="store_true", help="skip the break-down by kind of kernel (a second run under rocprofv3)")
-    ap.add_argument("--more-shapes", action="store_true", help="add decode and prefill points of the 1.5B and 7B layer sizes")
+    ap.add_argument("--more-shapes", action="store_true", help="further decode and prefill points of the 1.5B and 7B layer sizes")
+    ap.add_argument("--fewer-points", action="store_true", help="skip the points in other precisions, of other layer sizes and of the first token")
     ap.add_argument("--sync-steps", action="store_true", help="wait for each decode step's tokens before the next is launched")
     ap.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for profiles)")
     ap.add_argument("--prefill-tokens", type=int, default=None, help="tokens of the prefill (default: the context)")
@@ -266,13 +267,14 @@ def main() -> int:
     from machserve_amd.sampling import SamplingParams
     from machserve_amd.weights import random_tensor_dict
 
-    dt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[args.dtype]
-    page = args.page_size
+    DT = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}
+    dt = DT[args.dtype]
     gen = torch.Generator().manual_seed(1)
     models = {}
 
-    def model_of(shape):
-        if shape not in models:
+    def model_of(shape, dtn=None):
+        dtn = dtn or args.dtype
+        if (shape, dtn) not in models:
             raw = dict(SHAPES[shape][1])
             full = raw["num_hidden_layers"]
             if args.layers and shape == args.shape:
@@ -280,8 +282,8 @@ def main() -> int:
             cfg = config_from_dict(raw)
             models.clear()  # one model's weights at a time
             torch.cuda.empty_cache()
-            models[shape] = (cfg, random_tensor_dict(cfg, 0, dt, device="cuda:0"), full)
-        return models[shape]
+            models[(shape, dtn)] = (cfg, random_tensor_dict(cfg, 0, DT[dtn], device="cuda:0"), full)
+        return models[(shape, dtn)]
 
     def prompts(cfg, n, length):
         return [torch.randint(0, cfg.vocab_size, (length,), generator=gen).tolist() for _ in range(n)]
@@ -289,18 +291,20 @@ def main() -> int:
     recording = [False]
     recorders = []
 
-    def make_engine(shape, batch, budget, ctx, windows=1):
-        cfg, tensors, _ = model_of(shape)
+    def make_engine(shape, batch, budget, ctx, windows=1, dtn=None, page=None):
+        cfg, tensors, _ = model_of(shape, dtn)
+        page = page or args.page_size
         per_req = -(-(ctx + args.warmup + windows * args.steps + 2 * batch + 96) // page)
-        lm = load_model(config=cfg, tensors=tensors, dtype=dt, page_size=page, num_pages=batch * per_req + 4, max_requests=batch)
+        lm = load_model(config=cfg, tensors=tensors, dtype=DT[dtn or args.dtype], page_size=page, num_pages=batch * per_req + 4,
+                        max_requests=batch)
         if args.record_calls and not recorders:
             recorders.append(Recorder(lm.rt.ops, cfg.vocab_size, lambda: recording[0]))
         return Engine(lm, max_batch_tokens=budget, max_running=batch)
 
-    def decode_run(shape, batch, ctx, windows=3):
+    def decode_run(shape, batch, ctx, windows=3, dtn=None, page=None):
         """(tokens a second, milliseconds a step) of the median of ``windows`` timed runs of ``--steps`` decode steps."""
-        cfg = model_of(shape)[0]
-        eng = make_engine(shape, batch, 4096, ctx, windows)
+        cfg = model_of(shape, dtn)[0]
+        eng = make_engine(shape, batch, 4096, ctx, windows, dtn, page)
         for p in prompts(cfg, batch, ctx):
             eng.add(p, args.warmup + windows * args.steps + 2 * batch + 88, SamplingParams())  # early ones decode while later ones prefill
         while any(not r.decoding for r in eng.scheduler.running) or eng.scheduler.waiting:
@@ -333,16 +337,16 @@ def main() -> int:
         dt_s = statistics.median(times)
         return batch * args.steps / dt_s, dt_s / args.steps * 1e3
 
-    def prefill_run(shape, tokens):
-        cfg = model_of(shape)[0]
-        eng = make_engine(shape, 1, tokens, tokens)
+    def prefill_run(shape, tokens, dtn=None):
+        cfg = model_of(shape, dtn)[0]
+        eng = make_engine(shape, 1, tokens, tokens, 1, dtn)
         times = []
-        for rep in range(4):
+        # a step of a size that keeps coming is captured after a few sightings and then replayed, as in serving: the first
+        # ones are launched kernel by kernel, one captures, the last three are timed
+        for rep in range(eng.loaded.step.FILLED_CAPTURE_AFTER + 4):
             eng.add(prompts(cfg, 1, tokens)[0], 1, SamplingParams())
             torch.cuda.synchronize()
-            recording[0] = bool(args.record_calls) and rep == 3
-            if recording[0] and recorders:
-                del recorders[0].calls[:]
+            recording[0] = bool(args.record_calls)  # the capture issues the step's operations once: they are listed then
             t0 = time.perf_counter()
             em, done = eng.step()
             torch.cuda.synchronize()
@@ -351,22 +355,47 @@ def main() -> int:
             assert len(em) == 1 and len(done) == 1
         del eng
         torch.cuda.empty_cache()
-        return min(times[1:])
+        return min(times[-3:])
 
-    def decode_bytes(cfg, batch, ctx, windows):
-        nums = model_numbers(cfg, dt.itemsize)
+    def decode_bytes(cfg, batch, ctx, windows, dtn=None):
+        nums = model_numbers(cfg, DT[dtn or args.dtype].itemsize)
         mean_ctx = ctx + args.warmup + windows * args.steps / 2
         return nums["weight_bytes"] + batch * mean_ctx * nums["kv_bytes_per_token"]
 
-    def decode_point(shape, batch, ctx):
-        tok_s, ms = decode_run(shape, batch, ctx)
-        rate = decode_bytes(model_of(shape)[0], batch, ctx, 3) / (ms * 1e-3) / 1e9
+    def decode_point(shape, batch, ctx, dtn=None, page=None):
+        tok_s, ms = decode_run(shape, batch, ctx, 3, dtn, page)
+        rate = decode_bytes(model_of(shape, dtn)[0], batch, ctx, 3, dtn) / (ms * 1e-3) / 1e9
         return tok_s, {"ms": round(ms, 4), "GBs": round(rate, 1), "frac": round(rate / PEAK_HBM_GBS, 4)}
 
-    def prefill_point(shape, tokens):
-        t = prefill_run(shape, tokens)
-        fl = prefill_flops(model_of(shape)[0], tokens)
-        return tokens / t, {"ms": round(t * 1e3, 3), "TFLOPs": round(fl / t / 1e12, 1), "frac": round(fl / t / PEAK_FLOPS[args.dtype], 4)}
+    def prefill_point(shape, tokens, dtn=None):
+        t = prefill_run(shape, tokens, dtn)
+        fl = prefill_flops(model_of(shape, dtn)[0], tokens)
+        return tokens / t, {"ms": round(t * 1e3, 3), "TFLOPs": round(fl / t / 1e12, 1),
+                            "frac": round(fl / t / PEAK_FLOPS[dtn or args.dtype], 4)}
+
+    def first_token_points(shape, lengths):
+        """Time to the first token of one prompt, from ``add`` to its sampled token on the host, for prompts of
+        lengths that the engine has not seen: the steps of the sizes that prompts are filled up to (every 64
+        tokens up to 512) were captured before, by ``Engine.warm_up``, with other tokens."""
+        cfg = model_of(shape)[0]
+        eng = make_engine(shape, 2, 1024, 1024)
+        eng.warm_up(range(64, 513, 64))
+        out = {}
+        for n in lengths:
+            times = []
+            for rep in range(3):   # other tokens each time; the first is the cold one of this length
+                eng.add(prompts(cfg, 1, n)[0], 1, SamplingParams())
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                em, done = eng.step()
+                times.append(time.perf_counter() - t0)
+                assert len(em) == 1 and len(done) == 1
+            fl = prefill_flops(cfg, n)
+            out[n] = (n / times[0], {"ms": round(times[0] * 1e3, 3), "ms_again": round(min(times[1:]) * 1e3, 3),
+                                     "TFLOPs": round(fl / times[0] / 1e12, 1), "frac": round(fl / times[0] / PEAK_FLOPS[args.dtype], 4)})
+        del eng
+        torch.cuda.empty_cache()
+        return out
 
     shape_name = SHAPES[args.shape][0]
     cfg, _, full_layers = model_of(args.shape)
@@ -374,14 +403,20 @@ def main() -> int:
     prefill_tokens = args.prefill_tokens or ctx
 
     def save_calls(kind):
-        """The traced run's list of one step's operations: the last graph's worth for decoding, the last step's for prefill."""
+        """The traced run's list of one step's operations: the last time the model's operations were issued (launched, or
+        recorded into a graph), and the sampling after it (inside the graph for decoding, after the step for a prompt)."""
         calls = recorders[0].calls if recorders else []
+        starts = [i for i, c in enumerate(calls) if c[0] == "embedding"]
         if kind == "decode":  # the capture ran the step's operations once under recording: the last such run
             ends = [i for i, c in enumerate(calls) if c[0] == "sampling"]
-            starts = [i for i, c in enumerate(calls) if c[0] == "embedding"]
             if ends and starts:
                 first = max(s for s in starts if s < ends[-1])
                 calls = calls[first:ends[-1] + 1]
+        elif starts:
+            first = last = starts[-1]
+            while last < len(calls) and calls[last][0] != "sampling":
+                last += 1
+            calls = calls[first:last + 1]  # with the one sampling call that follows the step (later steps, replayed, list only theirs)
         with open(args.record_calls, "w") as f:
             json.dump(calls, f)
 
@@ -409,7 +444,7 @@ def main() -> int:
             "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
             "tied_head": bool(cfg.tie_word_embeddings), "rope_theta": cfg.rope_theta, "rms_eps": cfg.rms_norm_eps,
-            "page_size": page, "prefill_tokens": prefill_tokens, "sampling": "greedy",
+            "page_size": args.page_size, "prefill_tokens": prefill_tokens, "sampling": "greedy",
             "stepping": "one at a time" if args.sync_steps else "launched one step ahead",
         },
         "timed": "median of three windows of `steps` steps",
@@ -435,16 +470,29 @@ def main() -> int:
         if args.dtype == "bf16" and cfg.num_hidden_layers == full_layers and args.shape == "0.5b" and ctx == 2048:
             out["vs_reference"] = {"decode_b64_ctx2048": round(points["decode_b64"] / REF_DECODE_B64_CTX2048, 2),
                                    "prefill_2048": round(p_tok_s / REF_PREFILL_2048, 2)}
-        if args.more_shapes:
-            for shape, runs in (("1.5b", (("decode_b8", 8, 512), ("decode_b64", 64, 2048))), ("7b", (("decode_b1", 1, 2048), ("decode_b64", 64, 2048)))):
-                if shape == args.shape:
-                    continue
-                for name, batch, c in runs:
-                    v, detail[f"{shape}_{name}_ctx{c}"] = decode_point(shape, batch, c)
+        if args.shape == "0.5b" and args.dtype == "bf16" and cfg.num_hidden_layers == full_layers and not args.fewer_points:
+            # the first token of a prompt of a length not seen before (the reference quotes 512 tokens, docs/roadmap.md:260-261)
+            for n, (v, d) in first_token_points(args.shape, (128, 500, 512)).items():
+                points[f"first_token_{n}"], detail[f"first_token_{n}"] = round(v, 1), d
+            # the same configuration in the reference's own fast precision and in true 32-bit
+            for dtn in ("f16", "f32"):
+                v, detail[f"{dtn}_decode_b8"] = decode_point(args.shape, args.batch, ctx, dtn)
+                points[f"{dtn}_decode_b8"] = round(v, 1)
+                v, detail[f"{dtn}_prefill_2048"] = prefill_point(args.shape, 2048, dtn)
+                points[f"{dtn}_prefill_2048"] = round(v, 1)
+            # the two larger configurations of the same architecture: 1.5B, eight requests of 512 tokens decoding with pages
+            # of 16 tokens; 7B, 64 requests at 2,048-token contexts and one 2,048-token prompt
+            runs = {"1.5b": [("decode_b8", 8, 512, 16)], "7b": [("decode_b64", 64, 2048, None)]}
+            if args.more_shapes:
+                runs["1.5b"].append(("decode_b64", 64, 2048, None))
+                runs["7b"].insert(0, ("decode_b1", 1, 2048, None))
+            for shape, rs in runs.items():
+                for name, batch, c, pg in rs:
+                    v, detail[f"{shape}_{name}_ctx{c}"] = decode_point(shape, batch, c, None, pg)
                     points[f"{shape}_{name}_ctx{c}"] = round(v, 1)
-                v, detail[f"{shape}_prefill_2048"] = prefill_point(shape, 2048)
-                points[f"{shape}_prefill_2048"] = round(v, 1)
-            model_of(args.shape)
+                if shape == "7b" or args.more_shapes:
+                    v, detail[f"{shape}_prefill_2048"] = prefill_point(shape, 2048)
+                    points[f"{shape}_prefill_2048"] = round(v, 1)
         out["points"], out["points_detail"] = points, detail
     models.clear()
     torch.cuda.empty_cache()

@@ -234,11 +234,13 @@ class CacheManager:
         self.core.check()
 
     def build_step(self, slots, counts, tokens, want_rows, heads_per_kv, rows_per_block: int, table_multiple: int = 1,
-                   pad_rows: int = 0, axes: int = 1, explicit_positions=()):
+                   pad_rows: int = 0, axes: int = 1, explicit_positions=(), fill=None):
         """The step's int32 buffer as ``(numpy array, {section: (start, size)}, {group: table width})``;
-        see ``CacheCore::build_step`` for the sections, the rows that fill a step up and the positions."""
+        see ``CacheCore::build_step`` for the sections, the rows that fill a step up and the positions.
+        ``fill = (rows, requests, wanted rows)`` fills the step up to that size with rows of the scratch slot."""
+        rows, seqs, want = fill or (0, 0, 0)
         return self.core.build_step(slots, counts, tokens, want_rows, list(heads_per_kv), rows_per_block, table_multiple,
-                                    pad_rows, axes, list(explicit_positions))
+                                    pad_rows, axes, list(explicit_positions), rows, seqs, want)
 
     @property
     def scratch_slot(self) -> int:

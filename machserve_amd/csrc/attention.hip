@@ -128,6 +128,7 @@ __global__ __launch_bounds__(256 * KG, attention_waves_per_simd<KG>()) void page
     if (a.pair_span > 0 && turn >= a.pair_span)
         item = turn < 2 * a.pair_span ? a.n_work - 1 - (turn - a.pair_span) : turn - a.pair_span;
     const int s = a.work[item * 2], r0 = a.work[item * 2 + 1];
+    if (s < 0) return;  // an item that only fills the list up to a size that many steps share (the same for the whole block)
     const int g = a.H / a.KV;
     const int q_start = a.seq_q_start[s], q_len = a.seq_q_len[s], pos0 = a.seq_pos0[s];
     const int R = q_len * g;

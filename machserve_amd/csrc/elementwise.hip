@@ -359,12 +359,17 @@ extern "C" int ms_rope_kv_write(const float* qkv, int n_partials, const float* b
                (elem_t*)vpool, stride, H, KV, hd, ps};
     const bool aligned = ((reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(bias) | reinterpret_cast<uintptr_t>(q_out) |
                            reinterpret_cast<uintptr_t>(kpool)) & 15) == 0;
-    if (hd % 8 == 0 && stride % 4 == 0 && a.partial_stride % 4 == 0 && aligned && n_partials <= 4) {
+    // (up to eight partial sums: a portion of 65 to 128 rows cuts the projection's K seven times)
+    if (hd % 8 == 0 && stride % 4 == 0 && a.partial_stride % 4 == 0 && aligned && n_partials <= 8) {
         switch (n_partials) {
             case 1: hipLaunchKernelGGL(rope_kv_write_quads_kernel<1>, dim3(T), dim3(256), 0, stream, a); break;
             case 2: hipLaunchKernelGGL(rope_kv_write_quads_kernel<2>, dim3(T), dim3(256), 0, stream, a); break;
             case 3: hipLaunchKernelGGL(rope_kv_write_quads_kernel<3>, dim3(T), dim3(256), 0, stream, a); break;
-            default: hipLaunchKernelGGL(rope_kv_write_quads_kernel<4>, dim3(T), dim3(256), 0, stream, a); break;
+            case 4: hipLaunchKernelGGL(rope_kv_write_quads_kernel<4>, dim3(T), dim3(256), 0, stream, a); break;
+            case 5: hipLaunchKernelGGL(rope_kv_write_quads_kernel<5>, dim3(T), dim3(256), 0, stream, a); break;
+            case 6: hipLaunchKernelGGL(rope_kv_write_quads_kernel<6>, dim3(T), dim3(256), 0, stream, a); break;
+            case 7: hipLaunchKernelGGL(rope_kv_write_quads_kernel<7>, dim3(T), dim3(256), 0, stream, a); break;
+            default: hipLaunchKernelGGL(rope_kv_write_quads_kernel<8>, dim3(T), dim3(256), 0, stream, a); break;
         }
         return check_launch("rope_kv_write");
     }

@@ -252,17 +252,42 @@ public:
     // is the scratch page; their rows run like any other and leave no trace in what requests own.  "positions" is
     // [T, axes]: on every axis a row's index in its request's cache, unless `explicit_positions` ([T, axes]
     // flattened, rows of the entries only) gives the caller's own (where a row sits in the cache never follows them).
+    //
+    // `fill_rows`, `fill_seqs`, `fill_want` > 0 fill a step of any mix up to a size that many steps share (one
+    // captured graph then serves them all): requests of the scratch slot are appended until there are `fill_seqs`
+    // requests and `fill_rows` rows, the last of them taking what rows are left (token 0 at positions 0, 1, ...,
+    // all of its pages being the scratch page, so rows a page apart write the same place: nobody reads it); the
+    // wanted rows are filled up to `fill_want` with the step's last row; and every work list is filled up, with
+    // items of request -1 that the attention kernel skips, to the most items that any step of this size can have,
+    // fill_rows * g / rows_per_block + fill_seqs.  Needs fill_rows - rows >= fill_seqs - entries >= 1, or both zero (a step
+    // that has the size already: only its wanted rows and work lists are filled up).
     py::tuple build_step(const std::vector<int>& slots_in, const std::vector<int>& counts_in, const std::vector<int>& tokens_in,
-                         const std::vector<int>& want_rows, const std::vector<int>& heads_per_kv, int rows_per_block,
-                         int table_multiple, int pad_rows, int axes, const std::vector<int>& explicit_positions) const {
+                         const std::vector<int>& want_in, const std::vector<int>& heads_per_kv, int rows_per_block,
+                         int table_multiple, int pad_rows, int axes, const std::vector<int>& explicit_positions,
+                         int fill_rows, int fill_seqs, int fill_want) const {
         const int S_real = (int)slots_in.size();
         if (S_real == 0 || counts_in.size() != slots_in.size()) throw CacheError("a step needs at least one entry");
         if (pad_rows < 0) throw CacheError("pad_rows must not be negative");
-        std::vector<int> slots(slots_in), counts(counts_in), tokens(tokens_in);
+        std::vector<int> slots(slots_in), counts(counts_in), tokens(tokens_in), want_rows(want_in);
         slots.insert(slots.end(), pad_rows, scratch_slot());
         counts.insert(counts.end(), pad_rows, 1);
         tokens.insert(tokens.end(), pad_rows, 0);
-        const int S = S_real + pad_rows;
+        const int T_real = (int)tokens_in.size();
+        if (fill_rows > 0) {
+            if (pad_rows) throw CacheError("a step is filled up with single rows or to a size, not both");
+            const int more_seqs = fill_seqs - S_real, more_rows = fill_rows - T_real;
+            if (more_seqs < 0 || more_rows < more_seqs || (more_seqs == 0 && more_rows > 0))
+                throw CacheError(cat("a step of ", S_real, " requests and ", T_real, " rows cannot be filled up to ", fill_seqs, " and ", fill_rows));
+            if ((int)want_rows.size() > fill_want) throw CacheError(cat(want_rows.size(), " wanted rows exceed ", fill_want));
+            if (more_seqs > 0) {
+                slots.insert(slots.end(), more_seqs, scratch_slot());
+                counts.insert(counts.end(), more_seqs - 1, 1);
+                counts.push_back(more_rows - (more_seqs - 1));
+                tokens.insert(tokens.end(), more_rows, 0);
+            }
+            want_rows.insert(want_rows.end(), fill_want - want_rows.size(), fill_rows - 1);
+        }
+        const int S = (int)slots.size();
         std::vector<int> q_start(S), pos0(S);
         int T = 0;
         for (int i = 0; i < S; ++i) {
@@ -275,8 +300,8 @@ public:
         std::vector<std::pair<std::string, std::vector<int32_t>>> sections;
         auto add = [&](const std::string& name, std::vector<int32_t> v) { sections.emplace_back(name, std::move(v)); };
         if (axes < 1) throw CacheError(cat("positions have ", axes, " axes"));
-        if (!explicit_positions.empty() && explicit_positions.size() != (size_t)(T - pad_rows) * axes)
-            throw CacheError(cat("positions given for ", explicit_positions.size(), " numbers, the step has ", T - pad_rows, " rows of ", axes));
+        if (!explicit_positions.empty() && explicit_positions.size() != (size_t)T_real * axes)
+            throw CacheError(cat("positions given for ", explicit_positions.size(), " numbers, the step has ", T_real, " rows of ", axes));
         std::vector<int32_t> positions((size_t)T * axes);
         for (int i = 0; i < S; ++i)
             for (int j = 0; j < counts[i]; ++j)
@@ -294,11 +319,12 @@ public:
             const Group& g = groups_[gi];
             int width = 1;
             for (int i = 0; i < S_real; ++i) width = std::max(width, (int)g.tables.at(slots[i]).size());
+            for (int i = S_real; i < S; ++i) width = std::max(width, (counts[i] + page_size_ - 1) / page_size_);
             if (table_multiple > 1) width = (width + table_multiple - 1) / table_multiple * table_multiple;
             std::vector<int32_t> table((size_t)S * width, -1), slot_map(T);
-            for (int i = S_real; i < S; ++i) {
-                table[(size_t)i * width] = scratch_page((int)gi);
-                slot_map[q_start[i]] = scratch_page((int)gi) * page_size_;
+            for (int i = S_real; i < S; ++i) {  // rows that belong to nobody: every page is the scratch page
+                for (int p = 0; p * page_size_ < counts[i]; ++p) table[(size_t)i * width + p] = scratch_page((int)gi);
+                for (int j = 0; j < counts[i]; ++j) slot_map[q_start[i] + j] = scratch_page((int)gi) * page_size_ + j % page_size_;
             }
             for (int i = 0; i < S_real; ++i) {
                 const auto& t = g.tables.at(slots[i]);
@@ -329,6 +355,13 @@ public:
             for (const Item& it : items) {
                 work.push_back(it.seq);
                 work.push_back(it.r0);
+            }
+            if (fill_rows > 0) {  // as many items as any step of this size can have; the kernel skips request -1
+                const size_t most = (size_t)(fill_rows * hk + rows_per_block - 1) / rows_per_block + fill_seqs;
+                while (work.size() < 2 * most) {
+                    work.push_back(-1);
+                    work.push_back(0);
+                }
             }
             add("work/" + std::to_string(hk), std::move(work));
         }

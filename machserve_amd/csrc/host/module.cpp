@@ -60,7 +60,8 @@ PYBIND11_MODULE(ms_host, m) {
         .def("check", &CacheCore::check)
         .def("build_step", &CacheCore::build_step, py::arg("slots"), py::arg("counts"), py::arg("tokens"), py::arg("want_rows"),
              py::arg("heads_per_kv"), py::arg("rows_per_block"), py::arg("table_multiple") = 1, py::arg("pad_rows") = 0, py::arg("axes") = 1,
-             py::arg("explicit_positions") = std::vector<int>());
+             py::arg("explicit_positions") = std::vector<int>(), py::arg("fill_rows") = 0, py::arg("fill_seqs") = 0,
+             py::arg("fill_want") = 0);
 
     py::register_exception<SchedulerError>(m, "SchedulerError", PyExc_ValueError);
     py::class_<PlanItem>(m, "PlanItem")

@@ -43,6 +43,31 @@ class Engine:
                             portion=min(chunk_size or max_batch_tokens, max_batch_tokens))
         return cls(loaded, max_batch_tokens, chunk_size, capacity)
 
+    def warm_up(self, prompt_lengths: Sequence[int]) -> int:
+        """Captures, before any request has come, the steps that prompts of these lengths run as (each alone in its
+        step), so that the first prompt of such a size is replayed and not launched kernel by kernel: a step is
+        filled up to a size that many steps share, so a few lengths (say every 64 up to the token budget) cover every
+        prompt in between.  For each length two steps are captured: a prompt of exactly that many tokens, and one a
+        token shorter, which is filled up to it (and stands for every prompt that is).  Each capture runs a prompt
+        of token 0 in a request of its own, which is then released.  Returns how many steps were captured; 0 where
+        steps are not captured at all."""
+        from ..cache import OutOfPages
+        lm = self.loaded
+        if not lm.step.use_graphs or self.scheduler.has_work():
+            return 0
+        before = len(lm.step._graphs)
+        for n in sorted({m for length in prompt_lengths for m in (int(length) - 1, int(length))}):
+            if not 1 <= n <= min(self.scheduler.max_batch_tokens, lm.model.spec.max_positions) or lm.cache.slots.available() < 1:
+                continue
+            slot = lm.cache.admit()
+            try:
+                lm.step([StepEntry(slot, [0] * n, [n - 1])], borrow_logits=True, capture_now=True)
+            except OutOfPages:
+                pass
+            finally:
+                lm.cache.release(slot)
+        return len(lm.step._graphs) - before
+
     def add(self, prompt: Sequence[int], max_new: int, params: Optional[SamplingParams] = None,
             eos: Optional[int] = None, stop_seqs: Sequence[Sequence[int]] = ()) -> int:
         vocab = self.loaded.model.vocab

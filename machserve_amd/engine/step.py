@@ -73,12 +73,15 @@ class StepFunction:
     # captured step needs only while it runs comes from one pool that all captures share, since they run one
     # after another on one stream.  This reserve is device memory beside the weights and the page pools.
     MAX_GRAPH_BYTES = 2 << 30
-    CAPTURE_MAX_ROWS = 320  # a larger step keeps the device busy longer than the host needs to launch it (and replays slower)
+    # A larger step keeps the device busy about as long as the host needs to launch it (2,048 rows of the 0.5B sizes:
+    # 4.06 ms launched, 3.95 ms replayed).
+    CAPTURE_MAX_ROWS = 2048
     # A capture costs 7 ms; a replayed step is 0.9 ms shorter than a launched one with a few requests, 0.3 to
     # 0.4 ms with 64 requests or a few hundred rows.  While requests end one by one most shapes last a few
     # steps, so a shape is captured only when it has come this often before: at worst that doubles what the
     # better choice would have cost.
-    CAPTURE_AFTER = 16        # a step other than plain decoding
+    CAPTURE_AFTER = 16        # a step other than plain decoding, in its own shape
+    FILLED_CAPTURE_AFTER = 4  # ... filled up to a size that many steps share: such a size keeps coming
     DECODE_CAPTURE_AFTER = 8  # a decode step
 
     def __init__(self, model, cache: CacheManager, rt, attention_rows_per_block: int = 64, use_graphs: bool = True):
@@ -230,6 +233,38 @@ class StepFunction:
         return False
 
     @staticmethod
+    def _row_bucket(n: int) -> int:
+        """Rows of the captured step that takes a step of ``n`` rows which is not plain decoding: multiples of 16 up
+        to 64 rows, of 64 up to 512, of 256 beyond (a step's time grows slowly with its rows while they are few:
+        1.25 ms at 16 rows of the 0.5B sizes, 1.35 at 64, 1.47 at 128, 1.52 at 256, 2.0 at 512)."""
+        if n <= 64:
+            return -(-n // 16) * 16
+        return -(-n // 64) * 64 if n <= 512 else -(-n // 256) * 256
+
+    def _fill_shape(self, n_seqs: int, n_rows: int, n_want: int):
+        """``(rows, requests, wanted rows)`` that a step of any mix is filled up to, or None if it runs in its own
+        shape: the requests to the next power of two that leaves room for one more (the rows that fill the step up
+        need a request to belong to), the rows to their bucket, the wanted rows to a power of two; a step whose rows are
+        a bucket's already keeps its requests.  Beyond 512 rows a
+        step is filled by at most 64 rows: more would cost more than the launches that a replay saves."""
+        if self._row_bucket(n_rows) == n_rows:
+            seqs, rows = n_seqs, n_rows  # the step has a shared size already (a portion of the token budget, say)
+        else:
+            seqs = 2
+            while seqs < n_seqs + 1:
+                seqs *= 2
+            rows = self._row_bucket(n_rows + seqs - n_seqs)
+        if rows > self.CAPTURE_MAX_ROWS or (n_rows > 512 and rows - n_rows > 64):
+            return None
+        want = 0
+        if n_want:
+            want = 1
+            while want < n_want:
+                want *= 2
+            want = max(n_want, min(want, rows))
+        return rows, seqs, want
+
+    @staticmethod
     def _graph_key(counts, n_want: int, widths, sampled: bool) -> tuple:
         # for given tokens per request, wanted rows and table widths the buffer's layout is always the same
         return (tuple(counts), n_want, tuple(sorted(widths.items())), sampled)
@@ -364,12 +399,14 @@ class StepFunction:
         return launched.result[0, :n].tolist(), launched.result[1, :n].view(torch.float32).tolist()
 
     # ------------------------------------------------------------------ the step
-    def __call__(self, entries: Sequence[StepEntry], borrow_logits: bool = False) -> Optional[torch.Tensor]:
+    def __call__(self, entries: Sequence[StepEntry], borrow_logits: bool = False, capture_now: bool = False) -> Optional[torch.Tensor]:
         """Float32 logits ``[number of wanted places, vocab]`` in the order of the entries and
         of their ``want`` lists (None if nothing is wanted).  Takes the pages the new tokens
         need (raises ``OutOfPages`` before anything ran if they are not there), runs the
         model, and advances the requests' lengths.  With ``borrow_logits`` the result may be a
-        buffer that the next step overwrites (the engine samples from it at once)."""
+        buffer that the next step overwrites (the engine samples from it at once); with
+        ``capture_now`` a step that may run from a captured graph is captured at once, not
+        when its shape has come a few times."""
         cache = self.cache
         checked = self._check_entries(entries)  # a step that is refused has taken nothing
         self._take_pages(entries)
@@ -399,19 +436,32 @@ class StepFunction:
             width = self.TABLE_BUCKET
             while width < pages:
                 width *= 2
+            # filled up to a size that many steps share (rows, requests, wanted rows), so that one captured graph
+            # serves every step of that size; a step that would have to be filled too far runs in its own shape
+            fill = self._fill_shape(len(slots), len(tokens), len(want))
             try:
                 built = cache.build_step(slots, counts, tokens, want, self.heads_per_kv, self.rows_per_block, width, 0,
-                                         self.position_axes)
+                                         self.position_axes, (), fill)
             except CacheError as e:
                 raise StepError(str(e)) from e
-            key = self._graph_key(counts, len(want), built[2], False)
-            if len(tokens) <= self.CAPTURE_MAX_ROWS and self._ready(key, self.CAPTURE_AFTER):
-                logits, _ = self._run_graph(key, built)
-                if logits is not None and not borrow_logits:
-                    logits = logits.clone()
+            if fill is not None:
+                key = ("filled",) + fill + tuple(sorted(built[2].items()))
+                after = 0 if capture_now else self.FILLED_CAPTURE_AFTER
+            else:
+                key = self._graph_key(counts, len(want), built[2], False)
+                after = 0 if capture_now else self.CAPTURE_AFTER
+            if (fill is not None or len(tokens) <= self.CAPTURE_MAX_ROWS) and self._ready(key, after):
+                logits, _ = self._run_graph(key, built, fill_rows=0 if fill is None else fill[0] - len(tokens))
+                if logits is not None:
+                    if fill is not None:
+                        logits = logits[:len(want)] if want else None  # rows beyond belong to nobody
+                    if logits is not None and not borrow_logits:
+                        logits = logits.clone()
             else:  # most shapes never come again: they run as they are
                 host, offsets, widths = built
                 logits = self.model.forward(self._context_from(torch.from_numpy(host).to(self.rt.device), offsets, widths))
+                if fill is not None and logits is not None:
+                    logits = logits[:len(want)] if want else None
         else:
             logits = self.model.forward(self.build_context(entries, checked))
         for e in entries:

@@ -123,6 +123,8 @@ class EmulatedOps:
         out = torch.zeros(T, H * hd)
         done = set()
         for s, r0 in work.tolist():
+            if s < 0:   # an item that only fills the list up
+                continue
             qs, ql, p0 = int(seq_q_start[s]), int(seq_q_len[s]), int(seq_pos0[s])
             for r in range(r0, min(r0 + 64, ql * g)):
                 tok, j = divmod(r, g)

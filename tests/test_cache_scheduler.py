@@ -335,6 +335,53 @@ def test_pages_by_need_give_a_window_group_what_its_requests_can_hold_and_the_by
         assert g == P.greedy_generate(w, sizes, p, 8)
 
 
+@pytest.mark.parametrize("which", ["A", "C"])
+def test_a_step_filled_up_to_a_shared_size_gives_the_same_logits(tmp_path, which):
+    """Steps of any mix are filled up to a size that many steps share (rows, requests, wanted rows, work items) so
+    that one captured graph serves them all: the rows that fill a step up belong to nobody, write to the scratch page
+    and the scratch slot, and change no logit of a request.  Here on the CPU stand-ins, through the same buffer."""
+    from machserve_amd.engine import StepEntry, load_model
+    d = make_model_dir(tmp_path, which)
+    w, sizes = read_for_plain(d)
+    lm = load_model(d, dtype="float32", device="cpu", page_size=16, num_pages=24, max_requests=4, ops=EmulatedOps())
+    sf = lm.step
+    assert sf._fill_shape(1, 100, 1) == (128, 2, 1) and sf._fill_shape(3, 17, 3) == (32, 4, 4) and sf._fill_shape(4, 60, 0) == (64, 8, 0) and sf._fill_shape(4, 64, 0) == (64, 4, 0)
+    assert sf._fill_shape(1, 600, 1) is None and sf._fill_shape(1, 1000, 1) == (1024, 2, 1) and sf._fill_shape(1, 2048, 1) == (2048, 1, 1) and sf._fill_shape(2, 5000, 1) is None
+    seqs = [random_prompt(n, sizes["vocab"], 20 + n) for n in (50, 23, 9)]
+    refs = [P.forward(w, sizes, s) for s in seqs]
+    slots = [lm.cache.admit() for _ in seqs]
+    fed = [0, 0, 0]
+    for cuts in ([30, 23, 0], [19, 0, 8], [1, 0, 1], [0, 0, 0]):
+        if not any(cuts):   # a step that has a shared size already: sixteen rows of one request
+            lm.cache.release(slots[1])
+            slots[1], fed[1], seqs[1] = lm.cache.admit(), 0, random_prompt(16, sizes["vocab"], 99)
+            refs[1] = P.forward(w, sizes, seqs[1])
+            cuts = [0, 16, 0]
+        entries = [StepEntry(slots[r], seqs[r][fed[r]:fed[r] + n], [0, n - 1] if n > 1 else [0]) for r, n in enumerate(cuts) if n]
+        who = [r for r, n in enumerate(cuts) if n]
+        checked = sf._check_entries(entries)
+        sf._take_pages(entries)
+        sl, counts, tokens, want, _ = checked
+        fill = sf._fill_shape(len(sl), len(tokens), len(want))
+        host, offsets, widths = lm.cache.build_step(sl, counts, tokens, want, sf.heads_per_kv, sf.rows_per_block, 8, 0, 1, (), fill)
+        assert offsets["tokens"][1] == fill[0] and offsets["seq_slot"][1] == fill[1] and offsets["want_rows"][1] == fill[2]
+        for g in sf.heads_per_kv:   # as many work items as any step of this size can have
+            assert offsets[f"work/{g}"][1] == 2 * (-(-fill[0] * g // sf.rows_per_block) + fill[1])
+        logits = lm.model.forward(sf._context_from(torch.from_numpy(host), offsets, widths))[:len(want)]
+        k = 0
+        for r, e in zip(who, entries):
+            for place in e.want:
+                ref = refs[r][fed[r] + place]
+                assert (logits[k] - ref).abs().max() <= 2e-5 * (1 + ref.abs().max())
+                k += 1
+            lm.cache.commit(e.slot, len(e.tokens))
+            fed[r] += len(e.tokens)
+        lm.cache.check()
+    for s_ in slots:
+        lm.cache.release(s_)
+    assert all(g.pool.available() == g.pool.num_pages for g in lm.cache.groups.values())
+
+
 def test_a_refused_step_takes_no_pages(tmp_path):
     """A step with a bad token, a slot twice, a place beyond its tokens, or a slot that no request holds is refused
     before anything is taken: the tables, the free pages and the lengths are what they were."""

@@ -294,6 +294,17 @@ def test_rope_kv_write(dtype, H, KV, hd, ps, theta):
     assert_close(q2, q_ref2, dtype, "q from partial sums")
     assert_close(kd, kp2, dtype, "key pages from partial sums")
     assert_close(vd, vp2, dtype, "value pages from partial sums")
+    # seven and eleven partial sums (a portion of about a hundred rows cuts the projection's K seven times)
+    for n in (7, 11):
+        g = torch.Generator().manual_seed(16 + n)
+        cut = torch.randn((n - 1, *qkv.shape), generator=g)
+        parts = torch.cat([cut, (qkv - cut.sum(0)).unsqueeze(0)])
+        kd.zero_(), vd.zero_()
+        qn = ops.rope_kv_write(parts.to(DEV), bias.to(DEV), pos.to(DEV), inv.to(DEV), perm.to(DEV), kd, vd, H, KV, hd, ps)
+        assert_close(qn, emu.rope_kv_write(parts.sum(0) + bias, None, pos, inv, perm, kp2.zero_(), vp2.zero_(), H, KV, hd, ps), dtype,
+                     f"q from {n} partial sums")
+        assert_close(kd, kp2, dtype, f"key pages from {n} partial sums")
+        assert_close(vd, vp2, dtype, f"value pages from {n} partial sums")
 
 
 def _dead_pages_removed(table, seqs, ps, window):

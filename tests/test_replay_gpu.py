@@ -238,7 +238,7 @@ def test_a_step_shape_that_recurs_is_replayed_from_its_graph(models, which, dtyp
 
     def run(use_graphs):
         lm = engine(models, which, dtype, 24)
-        lm.step.CAPTURE_AFTER = lm.step.DECODE_CAPTURE_AFTER = 3
+        lm.step.CAPTURE_AFTER = lm.step.FILLED_CAPTURE_AFTER = lm.step.DECODE_CAPTURE_AFTER = 3
         if not use_graphs:
             lm.step.use_graphs = False
         replays = [0]

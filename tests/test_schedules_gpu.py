@@ -173,3 +173,74 @@ def test_temperature_sampling_through_the_entry_point_equals_the_plain_draws(tmp
             seq.append(tok)
     greedy = machserve_amd.generate(d, prompts, max_new=6, dtype="float32", page_size=16)
     assert greedy != got, "the test must tell a draw from the most likely token"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_steps_of_any_mix_run_from_graphs_of_shared_sizes(tmp_path, which, dtype):
+    """Prompts of many lengths, alone and beside requests that decode, each step filled up to a size that many steps
+    share and run from the captured graph of that size: fewer graphs than steps, and every logit the plain model's.
+    The rows that fill a step up belong to nobody; the cache is consistent afterwards."""
+    from machserve_amd.engine import StepEntry, load_model
+    d = make_model_dir(tmp_path, which)
+    w, sizes = read_for_plain(d)
+    ww = _stored(w, dtype)
+    lm = load_model(d, dtype=dtype, device=DEV, page_size=16, num_pages=40, max_requests=4)
+    lm.step.FILLED_CAPTURE_AFTER = 0   # every step that can be filled up runs from a graph, captured at its first coming
+    limit = CONFIGS[which]["max_position_embeddings"]
+    lengths = [n for n in (3, 17, 18, 30, 33, 47, 64, 65, 100, 127, 130, 200) if n + 12 <= limit]
+    seqs = [random_prompt(n + 12, sizes["vocab"], 900 + n) for n in lengths]
+    refs = [P.forward(ww, sizes, s) for s in seqs]
+    steps = 0
+
+    def compare(logits, rows):
+        got = logits.float().cpu()
+        assert got.shape[0] == len(rows)
+        for k, (r, pos) in enumerate(rows):
+            ref = refs[r][pos]
+            err = (got[k] - ref).abs().max().item()
+            assert err <= _bound(dtype, ref.abs().max().item()), f"request {r} ({lengths[r]} tokens) at position {pos}: error {err:.3e}"
+
+    decoding = {}   # request -> [slot, fed]
+    for r, n in enumerate(lengths):
+        # the new prompt, whole, beside one token of each request that decodes (at most two of them)
+        slot = lm.cache.admit()
+        entries, rows = [StepEntry(slot, seqs[r][:n], [0, n - 1])], [(r, 0), (r, n - 1)]
+        for q, (s_, fed) in decoding.items():
+            entries.append(StepEntry(s_, [seqs[q][fed]], [0]))
+            rows.append((q, fed))
+            decoding[q][1] += 1
+        compare(lm.step(entries), rows)
+        steps += 1
+        decoding[r] = [slot, n]
+        for q in [q for q, (s_, fed) in decoding.items() if fed >= lengths[q] + 10 or len(decoding) > 2][:1]:
+            lm.cache.release(decoding.pop(q)[0])
+        lm.cache.check()
+    filled = [k for k in lm.step._graphs if k[0] == "filled"]
+    assert filled and len(filled) < steps, f"{len(filled)} graphs of shared sizes for {steps} steps"
+    for s_, _ in decoding.values():
+        lm.cache.release(s_)
+    assert all(g.pool.available() == g.pool.num_pages for g in lm.cache.groups.values())
+
+
+def test_warm_up_captures_the_sizes_that_prompts_will_come_in(tmp_path):
+    """After ``Engine.warm_up`` the first prompt of a length is replayed from a graph captured before any request came,
+    and the tokens are the plain model's."""
+    from machserve_amd.engine import Engine
+    d = make_model_dir(tmp_path, "B")
+    w, sizes = read_for_plain(d)
+    eng = Engine.from_dir(d, dtype="float32", page_size=16, num_pages=40, capacity=2, max_batch_tokens=256)
+    n = eng.warm_up([16, 32, 48, 64, 128, 192, 256])
+    assert n >= 12 and not eng.loaded.cache.live_requests()
+    known = set(eng.loaded.step._graphs)
+    replayed = []
+    inner = eng.loaded.step._run_graph
+
+    def counted(key, *a, **kw):
+        replayed.append(key in known)
+        return inner(key, *a, **kw)
+    eng.loaded.step._run_graph = counted
+    for length in (100, 37, 150, 64):
+        prompt = random_prompt(length, sizes["vocab"], 40 + length)
+        assert eng.generate([prompt], max_new=3) == [P.greedy_generate(w, sizes, prompt, 3)]
+    assert replayed and replayed[0] and sum(replayed) >= 4, "the prompts' steps must have run from the graphs of the warm-up"
