@@ -48,7 +48,15 @@ constexpr int KPAD = 4, VPAD = 4;
 constexpr int NT = BKV / 16;             // 16-key score tiles per key tile
 constexpr int NTP = (NT + 1) / 2;        // pairs of score tiles = K steps of the PV product
 constexpr int K_LD = HDT + KPAD, V_LD = BKV + VPAD;
+// Flat rows of a work item.  The kernel of 32-row tiles (two-byte elements, head size 64) takes 128 a block; the
+// general kernel takes 64, and where a library has both, two of its blocks share an item.
+#if defined(MS_ELEM_HALF) && MS_ATTN_ND == 4
+#define MS_HAS_ROWS32 1
+constexpr int ROWS_PER_BLOCK = 128;
+#else
 constexpr int ROWS_PER_BLOCK = 64;
+#endif
+constexpr int SUB_BLOCKS = ROWS_PER_BLOCK / 64;  // blocks of the general kernel per work item
 constexpr float NEG_BIG = -1e30f;
 #ifdef MS_ELEM_HALF
 constexpr int MAX_KEY_GROUPS = ND <= 4 ? 4 : 2;  // groups of four waves that may share a block's keys
@@ -123,15 +131,17 @@ __global__ __launch_bounds__(256 * KG, attention_waves_per_simd<KG>()) void page
     // with its context, and blocks go to the CUs in turn: with two blocks a CU, block b shares its
     // CU with block b + (number of CUs).  So the list's heaviest `pair_span` items come first, then
     // its lightest ones, lightest first (each beside one of the heaviest), then the middle.
-    const int kvh = blockIdx.x % a.KV, turn = blockIdx.x / a.KV;
+    // (a work item of ROWS_PER_BLOCK rows is SUB_BLOCKS blocks of 64 rows here, side by side)
+    const int kvh = blockIdx.x % a.KV, sub = (blockIdx.x / a.KV) % SUB_BLOCKS, turn = blockIdx.x / (a.KV * SUB_BLOCKS);
     int item = turn;
     if (a.pair_span > 0 && turn >= a.pair_span)
         item = turn < 2 * a.pair_span ? a.n_work - 1 - (turn - a.pair_span) : turn - a.pair_span;
-    const int s = a.work[item * 2], r0 = a.work[item * 2 + 1];
+    const int s = a.work[item * 2], r0 = a.work[item * 2 + 1] + 64 * sub;
     if (s < 0) return;  // an item that only fills the list up to a size that many steps share (the same for the whole block)
     const int g = a.H / a.KV;
     const int q_start = a.seq_q_start[s], q_len = a.seq_q_len[s], pos0 = a.seq_pos0[s];
     const int R = q_len * g;
+    if (r0 >= R) return;  // the item's rows end in the block beside this one (the same for the whole block)
     const int hd = a.hd, ps = a.ps;
     const int* table = a.block_table + (size_t)s * a.table_stride;
 
@@ -145,7 +155,7 @@ __global__ __launch_bounds__(256 * KG, attention_waves_per_simd<KG>()) void page
 
     // keys any row of the block may see, and of those the rounds of tiles that are this split's
     constexpr int ROUND = KG * BKV;  // keys per round of the block
-    const int last_row = min(r0 + ROWS_PER_BLOCK, R) - 1;
+    const int last_row = min(r0 + 64, R) - 1;
     int kv_hi = pos0 + last_row / g + 1;
     int kv_lo = 0;
     if (a.window > 0) kv_lo = max(0, pos0 + r0 / g - a.window + 1);
@@ -491,6 +501,351 @@ __global__ __launch_bounds__(256 * KG, attention_waves_per_simd<KG>()) void page
     }
 }
 
+
+// ---------------------------------------------------------------------------------------
+// The same attention in tiles of 32 query rows by 32 keys (`mfma_f32_32x32x16`), for the two-byte element
+// types and a head size of 64.  The counters of the kernel above say that it spends fifteen vector instructions
+// on every matrix instruction, and its blocks of 64 rows read the keys and values of a long prompt so often
+// (a block of 64 flat rows is nine tokens of seven heads) that the traffic from the L2 comes within sight of that
+// path's ceiling.  Here a block is 128 flat rows, four waves of 32 rows under each of four key groups (sixteen waves,
+// a whole CU), so a tile that was brought into LDS feeds twice the rows; a lane holds sixteen keys of one query row
+// (one step across lanes instead of two) and a fragment read from LDS feeds twice the arithmetic; the
+// accumulator is rescaled only when a row's maximum has risen by more than a factor of 2^8 (a probability then
+// reaches 256 at most, which neither the 32-bit sums nor the rounded probabilities mind); tiles go from memory
+// straight into one of four LDS stages, three rounds before they are multiplied (no staging registers, no
+// stores); and the block's share of the block table is copied into LDS once, so that no round waits for a page
+// number.  Key tiles start at absolute multiples of 32, tile t belongs to group t mod 4, and every decision is a
+// row's own, so a row's result depends neither on the step's cut nor on the rows beside it.
+//
+// Operands (K = 16): A is 32 rows x 16, lane l holds row l % 32, elements (l / 32) * 8 .. + 8; B likewise by
+// column; the result has column l % 32 and, in register v, row 8 * (v / 4) + 4 * (l / 32) + v % 4.  With
+// S^T = K Q^T a lane's registers 8c .. 8c + 7 are therefore rows 16c + {0..3, 8..11} + 4 * (l / 32) of the key
+// tile: if row R of the tile holds key R with bits 2 and 3 exchanged, they are the eight consecutive keys
+// 16c + 8 * (l / 32) .., which is a B fragment of P^T as it stands and one 16-byte read of V^T.
+//
+// A tile that is loaded straight into LDS cannot be zeroed on its way: keys that are not there (beyond the
+// rows' positions, in pages given back behind a window, in tiles past the block's range) read the start of the
+// pool instead, and are masked in the scores; the pools hold finite values everywhere, so a value that meets a
+// zero probability adds nothing.
+#ifdef MS_HAS_ROWS32
+namespace r32 {
+constexpr int KG = 4, RW = 4, TK = 32;  // key groups, waves of rows, keys of a group's tile
+constexpr int GT = RW * 64;             // threads of a key group
+constexpr int ROUND = KG * TK;          // keys of a round of the block
+constexpr int NS = 4;                   // LDS stages: a tile is asked for NS - 1 rounds before it is multiplied
+constexpr int NC = HDT / 16;            // steps of the score product
+constexpr int NDT = HDT / 32;           // 32-row tiles of the output's head dimension
+// LDS rows are unpadded; 16-byte chunk q of row r sits at q ^ f(r), with f such that the rows a fragment read takes
+// in one pass (0..7 with 16..23, 8..15 with 24..31) fall on different banks.
+constexpr int K_BYTES = TK * HDT * 2, V_BYTES = HDT * TK * 2;
+constexpr int STAGE = K_BYTES + V_BYTES;
+constexpr int PER_LANE = 16 * NDT + 2;  // what a group hands over per lane: the output, the reference, the sum
+constexpr int MERGE_BYTES = (KG - 1) * RW * 64 * PER_LANE * 4;
+constexpr int SMEM = NS * KG * STAGE > MERGE_BYTES ? NS * KG * STAGE : MERGE_BYTES;
+constexpr int MAX_TABLE = 2048;  // pages of a block's share of the block table (in LDS)
+constexpr float RISE = 8.0f;     // a row's reference maximum follows its maximum when that has risen by more (in powers of two)
+static_assert(ROWS_PER_BLOCK == RW * 32, "a work item is what one block of this kernel takes");
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ void mma_32x32x16(f32x16& acc, const Frag& a, const Frag& b) {
+#if defined(MS_ELEM_BF16)
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, acc, 0, 0, 0);
+#else
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.v, b.v, acc, 0, 0, 0);
+#endif
+}
+// The largest of three, as one instruction (from `fmaxf` the compiler makes two for every operand it cannot prove to be
+// no signalling NaN; scores are sums of products of finite values, or -inf where masked).
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ int swap_bits_2_3(int r) { return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1); }
+__device__ __forceinline__ int k_swizzle(int r) { return ((r >> 1) & 3) | (((r >> 4) & 1) << 2); }  // rows of 8 chunks
+__device__ __forceinline__ int v_swizzle(int d) { return ((d >> 2) & 1) | (((d >> 4) & 1) << 1); }  // rows of 4 chunks
+}  // namespace r32
+
+__global__ __launch_bounds__(r32::KG * r32::GT, 4) void paged_attention_rows32_kernel(AttnArgs a) {
+    using namespace r32;
+    static_assert(HDT == 64 && TK == 32 && RW == 4, "the swizzles and the tiles' split over a group's waves are written for this shape");
+    static_assert(SMEM + MAX_TABLE * 4 + 1024 <= 160 * 1024, "the tiles of a block exceed the LDS of a CU");
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[SMEM];
+    __shared__ int tab[MAX_TABLE];
+    __shared__ unsigned kofs[KG][NS][2], vofs[KG][NS][2];  // [group][round % NS][16-key group of the tile]
+
+    const int kg = threadIdx.x >> 8, tg = threadIdx.x & 255, lane = tg & 63, rw = tg >> 6;
+    const int n32 = lane & 31, h = lane >> 5;
+    auto stage = [&](int b) { return smem + (KG * b + kg) * STAGE; };
+    const int kvh = blockIdx.x % a.KV, item = blockIdx.x / a.KV;
+    const int s = a.work[item * 2], r0 = a.work[item * 2 + 1];
+    if (s < 0) return;  // an item that only fills the list up (the same for the whole block)
+    const int g = a.H / a.KV;
+    const int q_start = a.seq_q_start[s], q_len = a.seq_q_len[s], pos0 = a.seq_pos0[s];
+    const int R = q_len * g;
+    constexpr int hd = HDT;
+    const int ps = a.ps;
+    const int* table = a.block_table + (size_t)s * a.table_stride;
+
+    // this lane's query row (both halves of the wave hold the same 32 rows)
+    const int row = r0 + rw * 32 + n32;
+    const bool valid = row < R;
+    const int tok = valid ? row / g : 0;
+    const int head = kvh * g + (valid ? row % g : 0);
+    const int pos = pos0 + tok;
+    const bool wave_active = r0 + rw * 32 < R;
+
+    const int last_row = min(r0 + ROWS_PER_BLOCK, R) - 1;
+    int kv_hi = pos0 + last_row / g + 1;
+    int kv_lo = 0;
+    if (a.window > 0) kv_lo = max(0, pos0 + r0 / g - a.window + 1);
+    const int lo_key = a.window > 0 ? pos - a.window + 1 : 0;
+    const int sp = blockIdx.y;
+    if (a.nsplit > 1) {
+        const int first = (kv_lo / ROUND) * ROUND;
+        const int per = ceil_div(ceil_div(kv_hi - first, ROUND), a.nsplit) * ROUND;
+        kv_lo = max(kv_lo, first + sp * per);
+        kv_hi = min(kv_hi, first + (sp + 1) * per);
+    }
+    // a row's partial result of this split: d = 32 dt + 8 (v / 4) + 4 h + v % 4 in register v of tile dt
+    auto write_partial = [&](const f32x16* o, float m, float l) {
+        const size_t base = (((size_t)(q_start + tok)) * a.H + head) * a.nsplit + sp;
+        float* po = a.part_o + base * hd;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                const int d0 = 32 * dt + 8 * qd + 4 * h;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) po[d0 + i] = o[dt][4 * qd + i];
+            }
+        if (h == 0) { a.part_ml[base * 2] = m * a.scale; a.part_ml[base * 2 + 1] = l; }
+    };
+    if (kv_lo >= kv_hi) {  // nothing for this split (the same for every thread of the block)
+        if (a.nsplit > 1 && kg == 0 && valid) {
+            f32x16 zero[NDT];
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) zero[dt][i] = 0.f;
+            write_partial(zero, NEG_BIG, 0.f);
+        }
+        return;
+    }
+    // the pages of the block's keys, once: those of [kt_first, kv_hi), at most MAX_TABLE of them (the launcher sees to it)
+    const int kt_first = (kv_lo / ROUND) * ROUND;
+    const int page_first = kt_first / ps, n_tab = min(ceil_div(kv_hi, ps), a.table_stride) - page_first;
+    for (int i = threadIdx.x; i < n_tab; i += KG * GT) tab[i] = table[page_first + i];
+
+    Frag qf[NC];
+    {
+        const elem_t* qrow = a.q + ((size_t)(q_start + tok) * a.H + head) * hd;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) qf[c] = valid ? frag_load(qrow + c * 16 + h * 8) : frag_zero();
+    }
+    f32x16 acc[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
+    // m_ref: the maximum that the exponentials refer to (a row's own running maximum, followed lazily)
+    float m_ref = NEG_BIG, l_run = 0.f;
+    const float sl = a.scale * 1.4426950408889634f;
+
+    // A group's four waves bring the group's tile, a quarter of K and a quarter of V^T each: a wave's load lands at the
+    // wave's LDS base + 16 * lane, so the chunk that belongs at place p = 64 * wave + lane of the K tile (row p / 8,
+    // chunk p % 8 ^ swizzle) is the one this lane asks for; likewise the V^T tile (row p / 4).  Which 16-key group of
+    // the tile a chunk lies in picks the page offset, which the group's first two threads leave in LDS a round before.
+    const int p_own = 64 * rw + lane;
+    const int Rk = p_own >> 3, kq = (p_own & 7) ^ k_swizzle(Rk), kl = swap_bits_2_3(Rk);  // row Rk of the tile holds key kl
+    const elem_t* k_src = a.kpool + (kl & 15) * hd + kq * 8;
+    const int k_grp = kl >> 4;
+    const int dv = p_own >> 2, vq = (p_own & 3) ^ v_swizzle(dv);  // keys 8 vq .. + 8 of row dv of V^T
+    const elem_t* v_src = a.vpool + (size_t)dv * ps + (vq & 1) * 8;
+    const int v_grp = vq >> 1;
+    // Offsets of the group's tile of the next round to be looked up, by the group's first two threads (one 16-key group of
+    // the tile each), stepped from round to round rather than divided out.  Keys that are not there (past the
+    // block's range, in a page given back) get offset 0: the first rows of the pool, finite and masked.
+    int key_next = kt_first + kg * TK + (tg & 1) * 16, lp_next = key_next / ps, off_next = key_next - lp_next * ps;
+    const int round_pages = ROUND / ps, round_rem = ROUND % ps;
+    auto fill_offsets = [&](int r) {
+        if (tg < 2) {
+            const bool there = key_next < kv_hi && lp_next < a.table_stride;
+            const int page = there ? tab[min(lp_next - page_first, n_tab - 1)] : -1;
+            const size_t pk = (size_t)max(page, 0) * a.KV + kvh;
+            kofs[kg][r % NS][tg] = page >= 0 ? (unsigned)(((pk * ps + off_next) * hd) >> 4) : 0u;
+            vofs[kg][r % NS][tg] = page >= 0 ? (unsigned)((pk * hd * ps + off_next) >> 4) : 0u;
+            key_next += ROUND;
+            lp_next += round_pages;
+            off_next += round_rem;
+            if (off_next >= ps) {
+                off_next -= ps;
+                ++lp_next;
+            }
+        }
+    };
+    // the group's tile of round r straight into stage r % NS (in assembly: of a load that it knows to write LDS the
+    // compiler would make every later LDS read wait; the waits are written by hand at the rounds' ends)
+    const uint32_t lds_own = __builtin_amdgcn_readfirstlane(
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char*)(smem + kg * STAGE + 1024 * rw));
+    auto load_direct = [&](int r) {
+        const int b = r % NS;
+        const elem_t* gk = k_src + ((size_t)kofs[kg][b][k_grp] << 4);
+        const elem_t* gv = v_src + ((size_t)vofs[kg][b][v_grp] << 4);
+        const uint32_t kb = lds_own + b * (KG * STAGE), vb = kb + K_BYTES;
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gk), "s"(kb) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gv), "s"(vb) : "memory", "m0");
+    };
+    // End of a round: this wave's loads of all but the last `behind` rounds have landed and its LDS accesses are
+    // done; then everybody's.  (A wave's loads complete in order, two a round.)
+    auto round_end = [&](bool full) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (full) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * (NS - 2)) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // rows of this wave: the first and the last position decide which tiles need no mask at all
+    const int pos_first = pos0 + (r0 + rw * 32) / g;
+    const int pos_last = pos0 + min(r0 + rw * 32 + 31, max(R - 1, 0)) / g;
+    const int lo_last = a.window > 0 ? pos_last - a.window + 1 : 0;
+    // where this lane reads its fragments in a stage: row n32 of the K tile, row 32 dt + n32 of V^T, chunk 2c + h
+    const int k_row = n32 * (HDT * 2), k_sw = k_swizzle(n32), v_row = K_BYTES + n32 * (TK * 2), v_sw = v_swizzle(n32);
+
+    // Round r: group kg has the tile of absolute index (kt_first / 32) + r * KG + kg.  Its page offsets are written a
+    // round before its loads go out, its loads NS - 1 rounds before it is multiplied, and one barrier a round
+    // separates the steps.
+    const int n_rounds = ceil_div(kv_hi - kt_first, ROUND);
+    // the queries and the table are here before the first tile is asked for, so that no later wait of the compiler's
+    // for them takes the tiles' loads with it
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int c = 0; c < NC; ++c) asm volatile("" : "+v"(qf[c].v));
+    __syncthreads();  // the table is in LDS
+    for (int r = 0; r < NS - 1; ++r) fill_offsets(r);
+    __syncthreads();
+    for (int r = 0; r < NS - 1; ++r)
+        if (r < n_rounds) load_direct(r);
+    fill_offsets(NS - 1);
+    round_end(n_rounds >= NS - 1);
+    for (int r = 0; r < n_rounds; ++r) {
+        const int kt0 = kt_first + r * ROUND + kg * TK;
+        const unsigned char* st = stage(r % NS);
+        const bool more = r + NS - 1 < n_rounds;
+        if (more) load_direct(r + NS - 1);  // into the stage that round r - 1 has left
+        const bool busy = wave_active && kt0 < kv_hi;
+        if (busy) {
+            // S^T = K Q^T: register v of this lane is key kt0 + 16 (v / 8) + 8 h + v % 8 for query row n32
+            f32x16 sc;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sc[i] = 0.f;
+            auto k_frag = [&](int c) { return frag_load(reinterpret_cast<const elem_t*>(st + k_row + (((2 * c + h) ^ k_sw) << 4))); };
+            Frag kf[2] = {k_frag(0), k_frag(1)};  // two fragments in flight
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                mma_32x32x16(sc, kf[c & 1], qf[c]);
+                if (c + 2 < NC) kf[c & 1] = k_frag(c + 2);
+            }
+            // the values of the first sixteen keys, which the step after next multiplies by: asked for before the exponentials
+            auto v_frag = [&](int c, int dt) {
+                return frag_load(reinterpret_cast<const elem_t*>(st + v_row + dt * (32 * TK * 2) + (((2 * c + h) ^ v_sw) << 4)));
+            };
+            Frag vf[NDT];
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) vf[dt] = v_frag(0, dt);
+            const bool whole = kt0 + TK - 1 <= pos_first && kt0 >= lo_last;
+            if (!whole) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int key = kt0 + 16 * (i / 8) + 8 * h + (i % 8);
+                    const bool ok = valid && key <= pos && key >= lo_key;
+                    sc[i] = ok ? sc[i] : -INFINITY;
+                }
+            }
+            float tmax = max3(max3(max3(sc[0], sc[1], sc[2]), max3(sc[3], sc[4], sc[5]), max3(sc[6], sc[7], sc[8])),
+                              max3(max3(sc[9], sc[10], sc[11]), sc[12], sc[13]), max3(sc[14], sc[15], sc[15]));
+            tmax = max3(tmax, __shfl_xor(tmax, 32, WAVE), tmax);
+            // a row's reference follows its maximum only when that has risen far; for every other row the factor is
+            // exactly one and nothing changes
+            const bool rise = (tmax - m_ref) * sl > RISE;
+            if (__any(rise)) {
+                const float m_new = rise ? tmax : m_ref;
+                const float alpha = exp2_f((m_ref - m_new) * sl);
+                l_run *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc[dt][i] *= alpha;
+                m_ref = m_new;
+            }
+            const float mb = m_ref * sl;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sc[i] = exp2_f(fmaf(sc[i], sl, -mb));
+            float t8[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) t8[i] = sc[i] + sc[i + 8];
+            float psum = ((t8[0] + t8[1]) + (t8[2] + t8[3])) + ((t8[4] + t8[5]) + (t8[6] + t8[7]));
+            psum += __shfl_xor(psum, 32, WAVE);
+            l_run += psum;
+            // O^T += V^T P^T: registers 8c .. 8c + 7 are the probabilities of keys 16c + 8h .. + 8, a B fragment as they stand
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                Frag pf;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) pf.v[i] = from_f32<elem_t>(sc[8 * c + i]);
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt) {
+                    mma_32x32x16(acc[dt], vf[dt], pf);
+                    if (c == 0) vf[dt] = v_frag(1, dt);
+                }
+            }
+        }
+        if (r + NS < n_rounds) fill_offsets(r + NS);  // read when that round's loads go out, at the top of the next round
+        round_end(more);
+    }
+
+    // groups 1.. hand (output, reference, sum) to group 0 through LDS, which adds them in group order
+    float* mg = reinterpret_cast<float*>(smem);
+    if (kg > 0) {
+        float* mine = mg + ((size_t)(kg - 1) * RW + rw) * 64 * PER_LANE;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) mine[(dt * 16 + i) * 64 + lane] = acc[dt][i];
+        mine[(16 * NDT) * 64 + lane] = m_ref;
+        mine[(16 * NDT + 1) * 64 + lane] = l_run;
+    }
+    __syncthreads();
+    if (kg > 0) return;
+    for (int o = 0; o < KG - 1; ++o) {
+        const float* other = mg + ((size_t)o * RW + rw) * 64 * PER_LANE;
+        const float m_o = other[(16 * NDT) * 64 + lane], l_o = other[(16 * NDT + 1) * 64 + lane];
+        const float m_new = fmaxf(m_ref, m_o);
+        const float c0 = exp2_f((m_ref - m_new) * sl), c1 = exp2_f((m_o - m_new) * sl);
+        l_run = l_run * c0 + l_o * c1;
+        m_ref = m_new;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[dt][i] = acc[dt][i] * c0 + other[(dt * 16 + i) * 64 + lane] * c1;
+    }
+    if (valid && a.nsplit > 1) {
+        write_partial(acc, m_ref, l_run);
+    } else if (valid) {
+        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+        elem_t* orow = a.out + ((size_t)(q_start + tok) * a.H + head) * hd;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                const int d0 = 32 * dt + 8 * qd + 4 * h;
+                half4_t o4 = {from_f32<elem_t>(acc[dt][4 * qd] * inv), from_f32<elem_t>(acc[dt][4 * qd + 1] * inv),
+                              from_f32<elem_t>(acc[dt][4 * qd + 2] * inv), from_f32<elem_t>(acc[dt][4 * qd + 3] * inv)};
+                *reinterpret_cast<half4_t*>(orow + d0) = o4;
+            }
+    }
+}
+#endif  // MS_HAS_ROWS32
 
 // ---------------------------------------------------------------------------------------
 // Decode attention: every request of the step has one row.  The g query heads of one KV
@@ -1016,10 +1371,10 @@ extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
     } else if (span < 4 * BKV) {
         groups = 1;
     }
-    MS_REQUIRE((long)n_work * KV < 2147483647L, "attention: %d blocks of rows times %d key/value heads", n_work, KV);
-    const dim3 grid((unsigned)(n_work * KV), (unsigned)nsplit);
+    MS_REQUIRE((long)n_work * KV * SUB_BLOCKS < 2147483647L, "attention: %d blocks of rows times %d key/value heads", n_work, KV);
+    const dim3 grid((unsigned)(n_work * KV * SUB_BLOCKS), (unsigned)nsplit);
     // how many blocks of each variant a CU holds, and how many CUs there are: asked once
-    static int cus = 0, resident[3] = {0, 0, 0};
+    static int cus = 0, resident[4] = {0, 0, 0, 0};
     if (cus == 0) {
         int dev = 0, n = 0;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1)
@@ -1032,7 +1387,26 @@ extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
         (void)hipGetLastError();
         cus = n;
     }
-    auto span_for = [&](int variant) { return resident[variant] == 2 ? (cus / KV > 0 ? cus / KV : 1) : 0; };
+    auto span_for = [&](int variant) { return resident[variant] == 2 ? (cus / (KV * SUB_BLOCKS) > 0 ? cus / (KV * SUB_BLOCKS) : 1) : 0; };
+#ifdef MS_HAS_ROWS32
+    {
+        // tiles of 32 rows by 32 keys under four key groups, a block a CU (the list's order, longest contexts first, is
+        // the order the blocks start in): where the block tables allow contexts of 2,048 keys and more (measured on
+        // one prompt of the 0.5B head shape: 512 tokens 13.9 against 11.9 us, 2,048 32.2 against 34.4, 4,096 60 against 83,
+        // 8,192 194 against 252), the head size is the tile's, and a block's share of the block table fits its
+        // place in LDS (asked for by name with max_key_groups = 32)
+        const long pages_of_span = window > 0 ? ((long)window + 2 * ROWS_PER_BLOCK + r32::ROUND) / ps + 2 : (long)table_stride;
+        if (hd == HDT && pages_of_span <= r32::MAX_TABLE && (max_key_groups == 32 || (max_key_groups == 0 && span >= 2048))) {
+            a.pair_span = 0;
+            const dim3 grid32((unsigned)(n_work * KV), (unsigned)nsplit);
+            hipLaunchKernelGGL(paged_attention_rows32_kernel, grid32, dim3(r32::KG * r32::GT), 0, stream, a);
+            int rc32 = check_launch("paged_attention (32-row tiles)");
+            if (rc32 || nsplit == 1) return rc32;
+            hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)((size_t)T * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit);
+            return check_launch("attention_merge");
+        }
+    }
+#endif
     if (groups >= 4 && MAX_KEY_GROUPS >= 4) {
         // sixteen waves leave each 128 registers, which only the small bfloat16 tiles fit into
         a.pair_span = span_for(2);

@@ -22,7 +22,7 @@ CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "csrc")
 CSRC = os.path.normpath(CSRC)
 ARCH = "gfx950"
 FLAGS = ["-O3", f"--offload-arch={ARCH}", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
-         "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+         "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-inline-asm"]
 ELEM_DEFINE = {"bf16": "MS_ELEM_BF16", "f16": "MS_ELEM_F16", "f32": "MS_ELEM_F32"}
 CORE_SOURCES = ["errors.hip", "gemm.hip", "skinny.hip", "elementwise.hip", "sampling.hip"]
 ATTENTION_TILES = (1, 2, 3, 4, 6, 8, 12, 16)  # head-size tiles in units of 16

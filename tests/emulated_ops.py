@@ -113,8 +113,10 @@ class EmulatedOps:
                 vpool[page[t], :, :, off[t]] = v[t]
         return q
 
+    rows_per_block = 64  # flat rows of a work item; a test that hands over a GPU library's work list sets that library's
+
     def attention_rows_per_block(self, hd):
-        return 64
+        return self.rows_per_block
 
     def paged_attention(self, q, kpool, vpool, block_table, seq_q_start, seq_q_len, seq_pos0, work, H, KV, hd,
                         page_size, window, scale):
@@ -126,7 +128,7 @@ class EmulatedOps:
             if s < 0:   # an item that only fills the list up
                 continue
             qs, ql, p0 = int(seq_q_start[s]), int(seq_q_len[s]), int(seq_pos0[s])
-            for r in range(r0, min(r0 + 64, ql * g)):
+            for r in range(r0, min(r0 + self.rows_per_block, ql * g)):
                 tok, j = divmod(r, g)
                 pos = p0 + tok
                 lo = 0 if not window else max(0, pos - window + 1)

@@ -335,7 +335,7 @@ def _attention_case(dtype, H, KV, hd, ps, window, seqs, seed, peak=False, groups
         for p in range(-(-(c + n) // ps)):
             table[i, p] = order.pop()
         q_start.append(T), q_len.append(n), pos0.append(c)
-        work += [(i, r0) for r0 in range(0, n * g, 64)]
+        work += [(i, r0) for r0 in range(0, n * g, ops.attention_rows_per_block(hd))]
         T += n
     q = rnd((T, H * hd), dtype, seed + 3)
     if peak:
@@ -352,6 +352,7 @@ def _attention_case(dtype, H, KV, hd, ps, window, seqs, seed, peak=False, groups
     args = (i32(q_start), i32(q_len), i32(pos0), i32(work).view(-1, 2))
     if groups or splits:
         emu = EmulatedOps(torch.float32)  # the reference unrounded: the tolerance allows the output's one rounding
+    emu.rows_per_block = ops.attention_rows_per_block(hd)
     ref = emu.paged_attention(q, kp, vp, table, *args, H, KV, hd, ps, window, hd ** -0.5)
     if dead_pages:
         table = _dead_pages_removed(table, seqs, ps, window)
@@ -380,6 +381,24 @@ def test_attention_key_groups(dtype, groups, H, KV, hd, ps, window):
     seqs = [(0, 1), (0, 300), (517, 1), (700, 37), (3, 2), (1023, 1), (64 * groups, 1), (64 * groups - 1, 2)]
     got, ref = _attention_case(dtype, H, KV, hd, ps, window, seqs, 300 + hd + groups, peak=True, groups=groups)
     assert_close(got, ref, dtype, f"attention with {groups} key groups")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("splits,dead_pages", [(0, False), (3, False), (0, True)])
+@pytest.mark.parametrize("H,KV,hd,ps,window", [(14, 2, 64, 64, None), (6, 2, 64, 16, 100), (20, 1, 64, 128, None), (8, 8, 64, 32, 333),
+                                               (3, 1, 64, 16, 31)])
+def test_attention_in_tiles_of_32_rows(dtype, splits, dead_pages, H, KV, hd, ps, window):
+    """The kernel of 32-row tiles that the two-byte libraries have for a head size of 64 (blocks of 128 flat rows, four
+    key groups, tiles loaded straight into four LDS stages, the block table in LDS, a reference maximum that follows
+    lazily), asked for by name: requests that end inside a tile, inside a round of four tiles and inside a block of
+    rows, contexts of a few thousand keys, a window with the pages behind it given back, the keys cut over blocks, and
+    a far key that must not be missed.  (The 32-bit library has no such kernel and answers with its general one.)"""
+    if dead_pages and window is None:
+        pytest.skip("pages are given back behind a window only")
+    seqs = [(0, 1), (0, 300), (517, 1), (3000, 37), (3, 2), (1023, 1), (128, 1), (127, 2), (31, 2), (95, 130), (2040, 19)]
+    got, ref = _attention_case(dtype, H, KV, hd, ps, window, seqs, 600 + ps + splits, peak=True, groups=32, splits=splits,
+                               dead_pages=dead_pages)
+    assert_close(got, ref, dtype, "attention in tiles of 32 rows")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -538,7 +557,8 @@ def test_attention_long_contexts(dtype, H, KV, hd, ps, window):
     qq = rnd((n, H * hd), dtype, 704)
     qq[n - 1] = q[1]
     i32 = lambda x: torch.tensor(x, dtype=torch.int32)
-    args = (i32([0]), i32([n]), i32([c]), i32([(0, r0) for r0 in range(0, n * g, 64)]).view(-1, 2))
+    emu.rows_per_block = ops.attention_rows_per_block(hd)
+    args = (i32([0]), i32([n]), i32([c]), i32([(0, r0) for r0 in range(0, n * g, emu.rows_per_block)]).view(-1, 2))
     tab = table[1:2].contiguous()
     ref2 = emu.paged_attention(qq, kp, vp, tab, *args, H, KV, hd, ps, window, hd ** -0.5)
     got2 = ops.paged_attention(qq.to(DEV), kp.to(DEV), vp.to(DEV), tab.to(DEV), *[a.to(DEV) for a in args], H, KV, hd, ps,
