@@ -593,7 +593,7 @@ __global__ __launch_bounds__(r32::KG * r32::GT, 4) void paged_attention_rows32_k
     const int tok = valid ? row / g : 0;
     const int head = kvh * g + (valid ? row % g : 0);
     const int pos = pos0 + tok;
-    const bool wave_active = r0 + rw * 32 < R;
+    const bool wave_active = __builtin_amdgcn_readfirstlane((int)(r0 + rw * 32 < R)) != 0;  // the same for the whole wave
 
     const int last_row = min(r0 + ROWS_PER_BLOCK, R) - 1;
     int kv_hi = pos0 + last_row / g + 1;
@@ -633,7 +633,8 @@ __global__ __launch_bounds__(r32::KG * r32::GT, 4) void paged_attention_rows32_k
         return;
     }
     // the pages of the block's keys, once: those of [kt_first, kv_hi), at most MAX_TABLE of them (the launcher sees to it)
-    const int kt_first = (kv_lo / ROUND) * ROUND;
+    kv_hi = __builtin_amdgcn_readfirstlane(kv_hi);
+    const int kt_first = __builtin_amdgcn_readfirstlane((kv_lo / ROUND) * ROUND);
     const int page_first = kt_first / ps, n_tab = min(ceil_div(kv_hi, ps), a.table_stride) - page_first;
     for (int i = threadIdx.x; i < n_tab; i += KG * GT) tab[i] = table[page_first + i];
 
@@ -696,15 +697,6 @@ __global__ __launch_bounds__(r32::KG * r32::GT, 4) void paged_attention_rows32_k
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gk), "s"(kb) : "memory", "m0");
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gv), "s"(vb) : "memory", "m0");
     };
-    // End of a round: this wave's loads of all but the last `behind` rounds have landed and its LDS accesses are
-    // done; then everybody's.  (A wave's loads complete in order, two a round.)
-    auto round_end = [&](bool full) {
-        __builtin_amdgcn_sched_barrier(0);
-        if (full) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * (NS - 2)) : "memory");
-        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-    };
     // rows of this wave: the first and the last position decide which tiles need no mask at all
     const int pos_first = pos0 + (r0 + rw * 32) / g;
     const int pos_last = pos0 + min(r0 + rw * 32 + 31, max(R - 1, 0)) / g;
@@ -715,7 +707,8 @@ __global__ __launch_bounds__(r32::KG * r32::GT, 4) void paged_attention_rows32_k
     // Round r: group kg has the tile of absolute index (kt_first / 32) + r * KG + kg.  Its page offsets are written a
     // round before its loads go out, its loads NS - 1 rounds before it is multiplied, and one barrier a round
     // separates the steps.
-    const int n_rounds = ceil_div(kv_hi - kt_first, ROUND);
+    // (the same for the whole block: kept in scalar registers, so that the rounds' branches are scalar ones)
+    const int n_rounds = __builtin_amdgcn_readfirstlane(ceil_div(kv_hi - kt_first, ROUND));
     // the queries and the table are here before the first tile is asked for, so that no later wait of the compiler's
     // for them takes the tiles' loads with it
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -727,25 +720,41 @@ __global__ __launch_bounds__(r32::KG * r32::GT, 4) void paged_attention_rows32_k
     for (int r = 0; r < NS - 1; ++r)
         if (r < n_rounds) load_direct(r);
     fill_offsets(NS - 1);
-    round_end(n_rounds >= NS - 1);
+    // End of a round: the tiles of all rounds but the youngest one asked for have landed (a wave's loads complete in
+    // order, two a round), and this wave's LDS accesses are done; then everybody's.
+    auto round_end = [&](bool one_behind) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (one_behind) asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    round_end(n_rounds >= NS - 1);  // rounds 0 and 1 are here
+    // S^T = K Q^T of the group's tile of round r: register v of this lane is key kt0 + 16 (v / 8) + 8 h + v % 8 for query
+    // row n32.  The scores of round r + 1 are asked for at the end of round r, behind the products of round r: the
+    // matrix cores work on them while other waves take their exponentials.
+    f32x16 sc;
+    auto scores = [&](int r) {
+        const unsigned char* st = stage(r % NS);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sc[i] = 0.f;
+        auto k_frag = [&](int c) { return frag_load(reinterpret_cast<const elem_t*>(st + k_row + (((2 * c + h) ^ k_sw) << 4))); };
+        Frag kf[2] = {k_frag(0), k_frag(1)};  // two fragments in flight
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            mma_32x32x16(sc, kf[c & 1], qf[c]);
+            if (c + 2 < NC) kf[c & 1] = k_frag(c + 2);
+        }
+    };
+    const int kg_keys = __builtin_amdgcn_readfirstlane(kg * TK);
+    auto busy_in = [&](int r) { return wave_active && kt_first + r * ROUND + kg_keys < kv_hi; };
+    if (busy_in(0)) scores(0);
     for (int r = 0; r < n_rounds; ++r) {
         const int kt0 = kt_first + r * ROUND + kg * TK;
         const unsigned char* st = stage(r % NS);
         const bool more = r + NS - 1 < n_rounds;
         if (more) load_direct(r + NS - 1);  // into the stage that round r - 1 has left
-        const bool busy = wave_active && kt0 < kv_hi;
-        if (busy) {
-            // S^T = K Q^T: register v of this lane is key kt0 + 16 (v / 8) + 8 h + v % 8 for query row n32
-            f32x16 sc;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) sc[i] = 0.f;
-            auto k_frag = [&](int c) { return frag_load(reinterpret_cast<const elem_t*>(st + k_row + (((2 * c + h) ^ k_sw) << 4))); };
-            Frag kf[2] = {k_frag(0), k_frag(1)};  // two fragments in flight
-#pragma unroll
-            for (int c = 0; c < NC; ++c) {
-                mma_32x32x16(sc, kf[c & 1], qf[c]);
-                if (c + 2 < NC) kf[c & 1] = k_frag(c + 2);
-            }
+        if (busy_in(r)) {
             // the values of the first sixteen keys, which the step after next multiplies by: asked for before the exponentials
             auto v_frag = [&](int c, int dt) {
                 return frag_load(reinterpret_cast<const elem_t*>(st + v_row + dt * (32 * TK * 2) + (((2 * c + h) ^ v_sw) << 4)));
@@ -762,14 +771,15 @@ __global__ __launch_bounds__(r32::KG * r32::GT, 4) void paged_attention_rows32_k
                     sc[i] = ok ? sc[i] : -INFINITY;
                 }
             }
-            float tmax = max3(max3(max3(sc[0], sc[1], sc[2]), max3(sc[3], sc[4], sc[5]), max3(sc[6], sc[7], sc[8])),
-                              max3(max3(sc[9], sc[10], sc[11]), sc[12], sc[13]), max3(sc[14], sc[15], sc[15]));
-            tmax = max3(tmax, __shfl_xor(tmax, 32, WAVE), tmax);
-            // a row's reference follows its maximum only when that has risen far; for every other row the factor is
-            // exactly one and nothing changes
-            const bool rise = (tmax - m_ref) * sl > RISE;
-            if (__any(rise)) {
-                const float m_new = rise ? tmax : m_ref;
+            // this lane's half of the row's keys
+            const float tmax = max3(max3(max3(sc[0], sc[1], sc[2]), max3(sc[3], sc[4], sc[5]), max3(sc[6], sc[7], sc[8])),
+                                    max3(max3(sc[9], sc[10], sc[11]), sc[12], sc[13]), max3(sc[14], sc[15], sc[15]));
+            // A row's reference follows its maximum only when that has risen far (the two lanes of a row keep the same
+            // reference: where either's half has risen far they exchange their maxima); for every other row the factor
+            // is exactly one and nothing changes.  After a prompt's first tiles this is rare.
+            if (__any((tmax - m_ref) * sl > RISE)) {
+                const float row_max = max3(tmax, __shfl_xor(tmax, 32, WAVE), tmax);
+                const float m_new = (row_max - m_ref) * sl > RISE ? row_max : m_ref;
                 const float alpha = exp2_f((m_ref - m_new) * sl);
                 l_run *= alpha;
 #pragma unroll
@@ -784,26 +794,27 @@ __global__ __launch_bounds__(r32::KG * r32::GT, 4) void paged_attention_rows32_k
             float t8[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) t8[i] = sc[i] + sc[i + 8];
-            float psum = ((t8[0] + t8[1]) + (t8[2] + t8[3])) + ((t8[4] + t8[5]) + (t8[6] + t8[7]));
-            psum += __shfl_xor(psum, 32, WAVE);
-            l_run += psum;
+            l_run += ((t8[0] + t8[1]) + (t8[2] + t8[3])) + ((t8[4] + t8[5]) + (t8[6] + t8[7]));  // of this lane's half of the keys
             // O^T += V^T P^T: registers 8c .. 8c + 7 are the probabilities of keys 16c + 8h .. + 8, a B fragment as they stand
+            Frag pf[2];
 #pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                Frag pf;
+            for (int c = 0; c < 2; ++c)
 #pragma unroll
-                for (int i = 0; i < 8; ++i) pf.v[i] = from_f32<elem_t>(sc[8 * c + i]);
+                for (int i = 0; i < 8; ++i) pf[c].v[i] = from_f32<elem_t>(sc[8 * c + i]);
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
 #pragma unroll
                 for (int dt = 0; dt < NDT; ++dt) {
-                    mma_32x32x16(acc[dt], vf[dt], pf);
+                    mma_32x32x16(acc[dt], vf[dt], pf[c]);
                     if (c == 0) vf[dt] = v_frag(1, dt);
                 }
-            }
         }
+        if (r + 1 < n_rounds && busy_in(r + 1)) scores(r + 1);
         if (r + NS < n_rounds) fill_offsets(r + NS);  // read when that round's loads go out, at the top of the next round
         round_end(more);
     }
 
+    l_run += __shfl_xor(l_run, 32, WAVE);  // the row's two halves (they were scaled alike all along)
     // groups 1.. hand (output, reference, sum) to group 0 through LDS, which adds them in group order
     float* mg = reinterpret_cast<float*>(smem);
     if (kg > 0) {

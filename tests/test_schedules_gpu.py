@@ -244,3 +244,48 @@ def test_warm_up_captures_the_sizes_that_prompts_will_come_in(tmp_path):
         prompt = random_prompt(length, sizes["vocab"], 40 + length)
         assert eng.generate([prompt], max_new=3) == [P.greedy_generate(w, sizes, prompt, 3)]
     assert replayed and replayed[0] and sum(replayed) >= 4, "the prompts' steps must have run from the graphs of the warm-up"
+
+
+@pytest.mark.timeout(300)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_long_prompts_at_head_size_64(tmp_path, dtype):
+    """A head size of 64 and block tables that allow thousands of keys: in the two-byte libraries the prompt's portions
+    run in the attention kernel of 32-row tiles (blocks of 128 flat rows, four key groups, tiles straight into LDS).
+    A prompt of 3,000 tokens in portions that end inside tiles and blocks, beside a second request that arrives
+    later, then decoded tokens; logits at the portions' first, middle and last rows and at every decoded position."""
+    from machserve_amd.engine import StepEntry, load_model
+    from machserve_amd.weights import write_random_model
+    raw = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_size": 320, "num_hidden_layers": 2,
+           "num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 64, "intermediate_size": 328, "vocab_size": 900,
+           "max_position_embeddings": 8192, "rms_norm_eps": 1e-6, "rope_theta": 1000000.0, "tie_word_embeddings": False,
+           "hidden_act": "silu", "use_sliding_window": False}
+    d = write_random_model(raw, 7, str(tmp_path / "hd64"))
+    w, sizes = read_for_plain(d)
+    ww = _stored(w, dtype)
+    a, b = random_prompt(3008, 900, 11), random_prompt(708, 900, 12)
+    ra, rb = P.forward(ww, sizes, a), P.forward(ww, sizes, b)
+    lm = load_model(d, dtype=dtype, device=DEV, page_size=32, num_pages=130, max_requests=2)
+    assert lm.model.attention_rows_per_block() == (64 if dtype == torch.float32 else 128)
+    sa, sb = lm.cache.admit(), lm.cache.admit()
+    got_a, got_b, where_a, where_b = [], [], [], []
+    ia = ib = 0
+    for ca, cb in ((1100, 0), (900, 0), (611, 333), (389, 367)):
+        entries = [StepEntry(sa, a[ia:ia + ca], [0, ca // 2, ca - 1])]
+        if cb:
+            entries.append(StepEntry(sb, b[ib:ib + cb], [0, cb - 1]))
+        out = lm.step(entries)
+        got_a.append(out[:3]), where_a.extend([ia, ia + ca // 2, ia + ca - 1])
+        if cb:
+            got_b.append(out[3:]), where_b.extend([ib, ib + cb - 1])
+        ia, ib = ia + ca, ib + cb
+    for j in range(8):
+        out = lm.step([StepEntry(sa, [a[ia + j]], [0]), StepEntry(sb, [b[ib]], [0])] if j == 0 else [StepEntry(sa, [a[ia + j]], [0])])
+        got_a.append(out[:1]), where_a.append(ia + j)
+        if j == 0:
+            got_b.append(out[1:]), where_b.append(ib)
+    for got, ref, where in ((torch.cat(got_a), ra, where_a), (torch.cat(got_b), rb, where_b)):
+        got = got.float().cpu()
+        scale = ref.abs().max().item()
+        allowed = {torch.float32: 1e-4 + 1e-4 * scale, torch.bfloat16: 3e-2 * scale, torch.float16: 3e-2 / 8 * scale}[dtype]
+        err = (got - ref[where]).abs().max().item()
+        assert err <= allowed, f"max error {err:.3e}, allowed {allowed:.3e}"
