@@ -18,7 +18,7 @@ from dataclasses import dataclass, asdict
 from typing import Optional
 
 from .specs import (AttentionSpec, ConfigError, EmbeddingSpec, GatedMlpSpec, HeadSpec, LayerSpec, ModelSpec,
-                    NormSpec, RotarySpec)
+                    NormSpec, RotarySpec, YarnSpec)
 
 ARCHITECTURE = "Qwen2ForCausalLM"
 
@@ -59,6 +59,7 @@ class Qwen2Config:
     max_window_layers: int
     attention_bias: bool
     torch_dtype: Optional[str]
+    rope_scaling: Optional[YarnSpec] = None
 
     @classmethod
     def from_dict(cls, raw: dict) -> "Qwen2Config":
@@ -82,8 +83,7 @@ class Qwen2Config:
         act = d.get("hidden_act", "silu")
         if act != "silu":
             raise ConfigError(f"config.json: hidden_act {act!r} is not supported (silu only)")
-        if d.get("rope_scaling") is not None:
-            raise ConfigError(f"config.json: rope_scaling {d['rope_scaling']!r} is not supported")
+        yarn = cls._yarn_of(d.get("rope_scaling"))
         theta = d.get("rope_theta")
         if theta is None and isinstance(d.get("rope_parameters"), dict):
             theta = d["rope_parameters"].get("rope_theta")
@@ -111,8 +111,35 @@ class Qwen2Config:
             use_sliding_window=use_win, sliding_window=window if use_win else None,
             max_window_layers=int(max_win_layers) if max_win_layers is not None else layers,
             attention_bias=bool(d.get("attention_bias", True)),
-            torch_dtype=d.get("torch_dtype"),
+            torch_dtype=d.get("torch_dtype"), rope_scaling=yarn,
         )
+
+    @staticmethod
+    def _yarn_of(rs) -> Optional[YarnSpec]:
+        """``rope_scaling``: absent, or YaRN with the keys and defaults of ``crates/mach-server/src/startup.rs:172-199``
+        (``type`` or ``rope_type`` "yarn", ``factor`` > 1, ``original_max_position_embeddings`` > 0, ``beta_fast`` 32,
+        ``beta_slow`` 1, ``mscale`` 1, ``mscale_all_dim`` 0); any other kind is refused, as the reference refuses it."""
+        if rs is None:
+            return None
+        if not isinstance(rs, dict):
+            raise ConfigError(f"config.json: rope_scaling must be an object, got {rs!r}")
+        kind = rs.get("type", rs.get("rope_type"))
+        if kind in (None, "default"):
+            return None
+        if kind != "yarn":
+            raise ConfigError(f"config.json: rope_scaling of type {kind!r} is not supported (only yarn)")
+
+        def number(key, default):
+            v = rs.get(key, default)
+            if isinstance(v, bool) or not isinstance(v, (int, float)):
+                raise ConfigError(f"config.json: rope_scaling.{key} must be a number, got {v!r}")
+            return float(v)
+        factor, orig = number("factor", 1.0), rs.get("original_max_position_embeddings", 0)
+        if isinstance(orig, bool) or not isinstance(orig, int) or orig <= 0 or factor <= 1.0:
+            raise ConfigError("config.json: rope_scaling of type yarn needs factor > 1 and original_max_position_embeddings > 0 "
+                              f"(got factor={factor}, original_max_position_embeddings={orig!r})")
+        return YarnSpec(factor, orig, number("beta_fast", 32.0), number("beta_slow", 1.0), number("mscale", 1.0),
+                        number("mscale_all_dim", 0.0))
 
     @classmethod
     def from_json_file(cls, path: str) -> "Qwen2Config":
@@ -123,6 +150,11 @@ class Qwen2Config:
 
     def to_dict(self) -> dict:
         d = asdict(self)
+        if self.rope_scaling is not None:
+            y = self.rope_scaling
+            d["rope_scaling"] = {"type": "yarn", "factor": y.factor, "original_max_position_embeddings": y.original_max_positions,
+                                 "beta_fast": y.beta_fast, "beta_slow": y.beta_slow, "mscale": y.mscale,
+                                 "mscale_all_dim": y.mscale_all_dim}
         d["architectures"] = [ARCHITECTURE]
         d["model_type"] = "qwen2"
         d["hidden_act"] = "silu"
@@ -134,15 +166,25 @@ class Qwen2Config:
             return self.sliding_window
         return None
 
+    def attention_scale(self) -> Optional[float]:
+        """What the scores are multiplied by: ``head_dim ** -0.5`` (None: the part's own default), times the square of
+        YaRN's ``0.1 mscale_all_dim ln(factor) + 1`` where that applies (``crates/mach-model/src/config.rs:218-234``)."""
+        y = self.rope_scaling
+        if y is None or y.mscale_all_dim <= 0.0:
+            return None
+        import math
+        m = 0.1 * y.mscale_all_dim * math.log(y.factor) + 1.0
+        return m * m / math.sqrt(self.head_dim)
+
     def to_spec(self) -> ModelSpec:
         """Tensor names: ``crates/mach-model/src/loader.rs:1023-1037, 1189-1231``."""
         layers = []
         for i in range(self.num_hidden_layers):
             p = f"model.layers.{i}."
-            rotary = RotarySpec("rotary", self.head_dim, self.rope_theta)
+            rotary = RotarySpec("rotary", self.head_dim, self.rope_theta, yarn=self.rope_scaling)
             mixer = AttentionSpec(
                 "attention", self.hidden_size, self.num_attention_heads, self.num_key_value_heads, self.head_dim,
-                rotary, window=self.layer_window(i),
+                rotary, window=self.layer_window(i), scale=self.attention_scale(),
                 tensors={"q.weight": p + "self_attn.q_proj.weight", "k.weight": p + "self_attn.k_proj.weight",
                          "v.weight": p + "self_attn.v_proj.weight", "o.weight": p + "self_attn.o_proj.weight",
                          "q.bias": p + "self_attn.q_proj.bias", "k.bias": p + "self_attn.k_proj.bias",

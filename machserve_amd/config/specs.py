@@ -29,12 +29,28 @@ class NormSpec:
 
 
 @dataclass(frozen=True)
+class YarnSpec:
+    """YaRN scaling of a rotation's frequencies (``crates/mach-server/src/startup.rs:172-199``): between the
+    pair indices that ``beta_fast`` and ``beta_slow`` rotations over ``original_max_positions`` mark, a frequency
+    goes over from its own value to ``1 / factor`` of it; cosines and sines are multiplied by
+    ``mscale(factor, mscale) / mscale(factor, mscale_all_dim)`` with ``mscale(f, m) = 0.1 m ln f + 1``."""
+    factor: float
+    original_max_positions: int
+    beta_fast: float = 32.0
+    beta_slow: float = 1.0
+    mscale: float = 1.0
+    mscale_all_dim: float = 0.0
+
+
+@dataclass(frozen=True)
 class RotarySpec:
-    """Rotation of pairs ``(j, j + rotary_dim/2)`` with ``freq_j = theta^(-2j/rotary_dim)``."""
+    """Rotation of pairs ``(j, j + rotary_dim/2)`` with ``freq_j = theta^(-2j/rotary_dim)``, or those frequencies
+    scaled as ``yarn`` says."""
     kind: str
     head_dim: int
     theta: float
     tensors: Mapping[str, str] = field(default_factory=dict)
+    yarn: Optional[YarnSpec] = None
 
 
 @dataclass(frozen=True)

@@ -30,6 +30,8 @@ class Attention(Mixer):
         scale = getattr(s, "scale", None)
         self.scale = float(s.head_dim) ** -0.5 if scale is None else float(scale)
         self.position = POSITION_ENCODINGS.build(s.position, rt) if s.position is not None else None
+        if self.position is not None:
+            self.scale *= float(self.position.score_factor())
         self.writes_cache = s.kv_source is None
         self.group = None
         self.kpool = self.vpool = None

@@ -213,6 +213,10 @@ class PositionEncoding(Part):
         """Encode positions in place into ``q [T, H, hd]`` and ``k [T, KV, hd]`` (float32 views)."""
         raise NotImplementedError
 
+    def score_factor(self) -> float:
+        """What the encoding multiplies every score by, beside what it does to q and k (1: nothing)."""
+        return 1.0
+
 
 class Mixer(Part):
     """Mixes information between positions of one request (attention, or a recurrence)."""

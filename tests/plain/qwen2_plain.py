@@ -37,28 +37,83 @@ def linear(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None = None) -> t
     return y
 
 
-def rope_angles(positions: torch.Tensor, head_dim: int, theta: float, dtype=torch.float32) -> torch.Tensor:
-    """``ang[p, j] = float(pos_p) * (1 / theta^(2j / head_dim))`` for ``j < head_dim/2``,
-    every step in ``dtype`` as the reference does it in f32.
+def yarn_of(rope_scaling):
+    """``rope_scaling`` of config.json as the reference reads it: None unless its ``type`` is "yarn"; then
+    ``(factor, original_max_position_embeddings, beta_fast = 32, beta_slow = 1, mscale = 1, mscale_all_dim = 0)``.
+    crates/mach-server/src/startup.rs:172-199."""
+    if not rope_scaling or rope_scaling.get("type", rope_scaling.get("rope_type")) != "yarn":
+        return None
+    return (float(rope_scaling.get("factor", 1.0)), int(rope_scaling.get("original_max_position_embeddings", 0)),
+            float(rope_scaling.get("beta_fast", 32.0)), float(rope_scaling.get("beta_slow", 1.0)),
+            float(rope_scaling.get("mscale", 1.0)), float(rope_scaling.get("mscale_all_dim", 0.0)))
 
-    crates/mach-model/src/ref_model.rs:636-643 (rope_freq, yarn off) and 679-681.
+
+def rope_freq(head_dim: int, theta: float, dtype=torch.float32, yarn=None) -> torch.Tensor:
+    """Inverse frequency of every pair index ``j < head_dim/2``: ``theta^(-2j / head_dim)``; with YaRN
+    ``freq_inter * ramp + freq_extra * (1 - ramp)``, ``freq_inter = freq_extra / factor``,
+    ``ramp = clamp((j - low) / (high - low), 0, 1)``,
+    ``low = floor(head_dim ln(orig / (beta_fast 2 pi)) / (2 ln theta))`` not below 0,
+    ``high = ceil(the same with beta_slow)`` not above ``head_dim - 1`` (and 0.001 more if equal to ``low``).
+
+    crates/mach-model/src/ref_model.rs:636-667 (rope_freq).
     """
     j = torch.arange(head_dim // 2, dtype=dtype)
-    freq = 1.0 / torch.pow(torch.tensor(float(theta), dtype=dtype), 2.0 * j / head_dim)
-    return positions.to(dtype)[:, None] * freq[None, :]
+    th = torch.tensor(float(theta), dtype=dtype)
+    extra = 1.0 / torch.pow(th, 2.0 * j / head_dim)
+    if yarn is None:
+        return extra
+    factor, orig, beta_fast, beta_slow = yarn[:4]
+    inter = 1.0 / (factor * torch.pow(th, 2.0 * j / head_dim))
+
+    def pair(rotations):
+        return head_dim * math.log(orig / (rotations * 2.0 * math.pi)) / (2.0 * math.log(theta))
+    low, high = max(math.floor(pair(beta_fast)), 0.0), min(math.ceil(pair(beta_slow)), head_dim - 1.0)
+    if high == low:
+        high += 0.001
+    ramp = ((j - low) / (high - low)).clamp(0.0, 1.0)
+    return inter * ramp + extra * (1.0 - ramp)
 
 
-def rope(x: torch.Tensor, positions: torch.Tensor, theta: float) -> torch.Tensor:
+def yarn_attention_factor(yarn) -> float:
+    """What YaRN multiplies every cosine and sine by: ``mscale(factor, mscale) / mscale(factor, mscale_all_dim)``
+    with ``mscale(f, m) = 0.1 m ln f + 1``.  crates/mach-model/src/config.rs:242-253."""
+    if yarn is None:
+        return 1.0
+    ln = math.log(yarn[0])
+    return (0.1 * yarn[4] * ln + 1.0) / (0.1 * yarn[5] * ln + 1.0)
+
+
+def attn_scale(head_dim: int, yarn=None) -> float:
+    """``m^2 / sqrt(head_dim)`` with ``m = 0.1 mscale_all_dim ln(factor) + 1`` under YaRN with ``mscale_all_dim > 0``,
+    else ``m = 1``.  crates/mach-model/src/config.rs:218-234."""
+    m = 1.0
+    if yarn is not None and yarn[5] > 0.0:
+        m = 0.1 * yarn[5] * math.log(yarn[0]) + 1.0
+    return m * m / math.sqrt(head_dim)
+
+
+def rope_angles(positions: torch.Tensor, head_dim: int, theta: float, dtype=torch.float32, yarn=None) -> torch.Tensor:
+    """``ang[p, j] = float(pos_p) * freq_j`` for ``j < head_dim/2``, every step in ``dtype`` as the
+    reference does it in f32.
+
+    crates/mach-model/src/ref_model.rs:636-643 (rope_freq) and 679-681.
+    """
+    return positions.to(dtype)[:, None] * rope_freq(head_dim, theta, dtype, yarn)[None, :]
+
+
+def rope(x: torch.Tensor, positions: torch.Tensor, theta: float, yarn=None) -> torch.Tensor:
     """Rotate pairs ``(j, j + head_dim/2)`` (rotate_half pairing, whole head rotated):
-    ``a' = a cos - b sin``, ``b' = a sin + b cos``.  ``x`` is ``[T, heads, head_dim]``.
+    ``a' = a cos - b sin``, ``b' = a sin + b cos``, cosine and sine times YaRN's factor if there is one.
+    ``x`` is ``[T, heads, head_dim]``.
 
     crates/mach-model/src/ref_model.rs:669-704 (apply_rope, interleave=false), tools/ref_llama.py:56-67.
     """
     hd = x.shape[-1]
     half = hd // 2
-    ang = rope_angles(positions, hd, theta, x.dtype)
-    c = torch.cos(ang)[:, None, :]
-    s = torch.sin(ang)[:, None, :]
+    ang = rope_angles(positions, hd, theta, x.dtype, yarn)
+    f = yarn_attention_factor(yarn)
+    c = torch.cos(ang)[:, None, :] * f
+    s = torch.sin(ang)[:, None, :] * f
     a = x[..., :half]
     b = x[..., half:]
     return torch.cat([a * c - b * s, a * s + b * c], dim=-1)
@@ -78,7 +133,8 @@ def to_f16_and_back(x: torch.Tensor) -> torch.Tensor:
     return x.to(torch.float16).to(x.dtype)
 
 
-def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int | None = None, rounded=same) -> torch.Tensor:
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int | None = None, rounded=same,
+              scale: float | None = None) -> torch.Tensor:
     """Causal grouped-query attention over a whole sequence.
 
     ``q`` is ``[T, H, hd]``, ``k``/``v`` are ``[T, KV, hd]``.  Query head ``h`` reads
@@ -92,7 +148,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int | N
     T, H, hd = q.shape
     KV = k.shape[1]
     g = H // KV
-    scale = hd ** -0.5
+    scale = hd ** -0.5 if scale is None else scale
     out = torch.zeros_like(q)
     for h in range(H):
         kv = h // g
@@ -129,9 +185,10 @@ def attention_block(x, w, prefix, positions, sizes, window=None, rounded=same):
     q = linear(x, w[prefix + "q_proj.weight"], w.get(prefix + "q_proj.bias"))
     k = linear(x, w[prefix + "k_proj.weight"], w.get(prefix + "k_proj.bias"))
     v = linear(x, w[prefix + "v_proj.weight"], w.get(prefix + "v_proj.bias"))
-    q = rounded(rope(q.view(T, H, hd), positions, sizes["theta"]))
-    k = rounded(rope(k.view(T, KV, hd), positions, sizes["theta"]))
-    o = rounded(attention(q, k, rounded(v.view(T, KV, hd)), window, rounded))
+    yarn = yarn_of(sizes.get("rope_scaling"))
+    q = rounded(rope(q.view(T, H, hd), positions, sizes["theta"], yarn))
+    k = rounded(rope(k.view(T, KV, hd), positions, sizes["theta"], yarn))
+    o = rounded(attention(q, k, rounded(v.view(T, KV, hd)), window, rounded, attn_scale(hd, yarn)))
     return linear(o.reshape(T, H * hd), w[prefix + "o_proj.weight"])
 
 
@@ -188,6 +245,7 @@ def sizes_from_config(cfg: dict) -> dict:
         "vocab": cfg["vocab_size"],
         "eps": cfg.get("rms_norm_eps", 1e-6),
         "theta": cfg.get("rope_theta", 10000.0),
+        "rope_scaling": cfg.get("rope_scaling"),
         "tied": cfg.get("tie_word_embeddings", False),
         "use_sliding_window": cfg.get("use_sliding_window", False),
         "sliding_window": cfg.get("sliding_window"),

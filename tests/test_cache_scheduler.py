@@ -382,6 +382,32 @@ def test_a_step_filled_up_to_a_shared_size_gives_the_same_logits(tmp_path, which
     assert all(g.pool.available() == g.pool.num_pages for g in lm.cache.groups.values())
 
 
+@pytest.mark.parametrize("mscale_all_dim", [0.0, 0.707])
+def test_yarn_through_the_engine_equals_the_plain_model(tmp_path, mscale_all_dim):
+    """A configuration with YaRN (crates/mach-model/src/ref_model.rs:636-704): scaled frequencies, the factor on
+    cosines and sines (which the engine puts on the scores, squared) and mscale_all_dim's square on the scores'
+    scale; positions far beyond the original context, in portions and token by token."""
+    from machserve_amd.engine import StepEntry, load_model
+    from machserve_amd.weights import write_random_model
+    from tiny_configs import TINY_A, sharpen_attention
+    raw = dict(TINY_A, max_position_embeddings=512,
+               rope_scaling={"type": "yarn", "factor": 8.0, "original_max_position_embeddings": 32, "mscale_all_dim": mscale_all_dim})
+    d = write_random_model(raw, 3, str(tmp_path / "yarn"))
+    sharpen_attention(d, 4.0)
+    w, sizes = read_for_plain(d)
+    assert sizes["rope_scaling"]["factor"] == 8.0
+    toks = random_prompt(300, 512, 5)
+    ref = P.forward(w, sizes, toks)
+    without = P.forward(w, dict(sizes, rope_scaling=None), toks)
+    assert (ref - without).abs().max() > 1e-2 * ref.abs().max(), "the test must tell YaRN from plain rotation"
+    lm = load_model(d, dtype="float32", device="cpu", page_size=16, num_pages=20, max_requests=1, ops=EmulatedOps())
+    slot = lm.cache.admit()
+    got = [lm.step([StepEntry(slot, toks[:170], list(range(170)))]), lm.step([StepEntry(slot, toks[170:290], list(range(120)))])]
+    got += [lm.step([StepEntry(slot, toks[i:i + 1], [0])]) for i in range(290, 300)]
+    got = torch.cat(got)
+    assert (got - ref).abs().max() <= 2e-5 * (1 + ref.abs().max())
+
+
 def test_a_refused_step_takes_no_pages(tmp_path):
     """A step with a bad token, a slot twice, a place beyond its tokens, or a slot that no request holds is refused
     before anything is taken: the tables, the free pages and the lengths are what they were."""

@@ -30,12 +30,35 @@ def test_qwen2_config_reads_its_keys():
     assert c.max_position_embeddings == 77 and c.rms_norm_eps == 2e-6
 
 
+def test_yarn_rope_scaling_is_read_with_the_reference_s_keys_and_defaults():
+    """crates/mach-server/src/startup.rs:172-199: type yarn, factor, original_max_position_embeddings, beta_fast 32,
+    beta_slow 1, mscale 1, mscale_all_dim 0; the scores' scale takes mscale_all_dim's square only when it is set."""
+    import math
+    from machserve_amd.config import YarnSpec, config_from_dict
+    raw = dict(TINY_A, rope_scaling={"type": "yarn", "factor": 4.0, "original_max_position_embeddings": 64})
+    c = config_from_dict(raw)
+    assert c.rope_scaling == YarnSpec(4.0, 64, 32.0, 1.0, 1.0, 0.0) and c.attention_scale() is None
+    spec = c.to_spec()
+    assert all(l.mixer.position.yarn == c.rope_scaling and l.mixer.scale is None for l in spec.layers)
+    assert config_from_dict(c.to_dict()) == c
+    c2 = config_from_dict(dict(TINY_A, rope_scaling={"rope_type": "yarn", "factor": 40.0, "original_max_position_embeddings": 4096,
+                                                      "beta_fast": 16, "beta_slow": 2, "mscale": 0.9, "mscale_all_dim": 0.707}))
+    assert c2.rope_scaling == YarnSpec(40.0, 4096, 16.0, 2.0, 0.9, 0.707)
+    m = 0.1 * 0.707 * math.log(40.0) + 1
+    assert abs(c2.attention_scale() - m * m / 4.0) < 1e-12      # head size 16
+    assert config_from_dict(dict(TINY_A, rope_scaling=None)).rope_scaling is None
+    assert config_from_dict(dict(TINY_A, rope_scaling={"type": "default"})).rope_scaling is None
+
+
 @pytest.mark.parametrize("change,match", [
     ({"hidden_size": None}, "missing key 'hidden_size'"),
     ({"num_hidden_layers": 0}, "num_hidden_layers"),
     ({"num_key_value_heads": 3}, "not a multiple"),
     ({"hidden_act": "gelu"}, "hidden_act"),
-    ({"rope_scaling": {"type": "yarn"}}, "rope_scaling"),
+    ({"rope_scaling": {"type": "yarn"}}, "factor > 1"),
+    ({"rope_scaling": {"type": "yarn", "factor": 4.0}}, "original_max_position_embeddings"),
+    ({"rope_scaling": {"type": "linear", "factor": 2.0}}, "only yarn"),
+    ({"rope_scaling": {"rope_type": "llama3", "factor": 8.0}}, "only yarn"),
     ({"use_sliding_window": True}, "sliding_window"),
     ({"architectures": ["LlamaForCausalLM"]}, "not supported"),
     ({"hidden_size": 66}, "head_dim"),

@@ -60,6 +60,41 @@ def test_rope_is_rotate_half_and_not_interleaved():
     assert not torch.allclose(inter[1:], P.rope(x, pos, theta)[1:], atol=1e-3)
 
 
+def test_yarn_frequencies_and_factors_are_the_reference_s_own_vectors():
+    """The numbers that the reference's tests hold for YaRN (crates/mach-model/src/ref_model.rs:1330-1560): with head
+    size 64, theta 10,000, factor 40 over 4,096 positions, beta 32 / 1 the ramp runs from pair 10 to pair 23 (clamped to
+    the head size, not to the number of pairs); pair 0 keeps its own frequency, pair 31 has 1 / factor of it; the
+    factor on cosines and sines is mscale(1.0) / mscale(0.707); the scores' scale has mscale(0.707)^2.  And the
+    formulas written out once more, in 64-bit, as the library that the checkpoints come from writes them."""
+    import math
+    yarn = P.yarn_of({"type": "yarn", "factor": 40.0, "original_max_position_embeddings": 4096, "mscale": 1.0, "mscale_all_dim": 0.707})
+    assert yarn == (40.0, 4096, 32.0, 1.0, 1.0, 0.707)
+    assert P.yarn_of(None) is None and P.yarn_of({"type": "linear", "factor": 2.0}) is None
+    f = P.rope_freq(64, 1e4, torch.float64, yarn)
+    assert abs(f[0].item() - 1.0) < 1e-12 and abs(f[31].item() - 1.0 / (40.0 * 1e4 ** (62 / 64))) < 1e-15
+    dim, base, factor, orig = 64, 1e4, 40.0, 4096.0
+    corr = lambda rot: dim * math.log(orig / (rot * 2 * math.pi)) / (2 * math.log(base))
+    low, high = max(math.floor(corr(32.0)), 0), min(math.ceil(corr(1.0)), dim - 1)
+    assert (low, high) == (10, 23)
+    for d in range(32):
+        extra = 1.0 / base ** (2 * d / dim)
+        mask = 1.0 - min(max((d - low) / (high - low), 0.0), 1.0)
+        want = extra / factor * (1 - mask) + extra * mask
+        assert abs(f[d].item() - want) <= 1e-12 * want, d
+    assert torch.equal(P.rope_freq(64, 1e4, torch.float64, None), 1.0 / torch.pow(torch.tensor(1e4, dtype=torch.float64), torch.arange(0, 64, 2, dtype=torch.float64) / 64))
+    ln = math.log(40.0)
+    assert abs(P.yarn_attention_factor(yarn) - (0.1 * ln + 1) / (0.1 * 0.707 * ln + 1)) < 1e-12
+    assert P.yarn_attention_factor(yarn[:4] + (0.707, 0.707)) == 1.0 and P.yarn_attention_factor(None) == 1.0
+    m = 0.1 * 0.707 * ln + 1
+    assert abs(P.attn_scale(192, yarn) - m * m / math.sqrt(192)) < 1e-12
+    assert P.attn_scale(192, yarn[:5] + (0.0,)) == 1 / math.sqrt(192) and P.attn_scale(64) == 0.125
+    # rotation with the factor: every pair's norm grows by it, position 0 is the identity times it
+    x = rnd(3, 2, 64, seed=21)
+    y = P.rope(x, torch.tensor([0, 5, 9000]), 1e4, yarn)
+    af = P.yarn_attention_factor(yarn)
+    assert torch.allclose(y[0], x[0] * af) and torch.allclose((y[..., :32] ** 2 + y[..., 32:] ** 2), (x[..., :32] ** 2 + x[..., 32:] ** 2) * af * af)
+
+
 def test_rope_scores_depend_on_distance_only():
     q, k = rnd(1, 1, 32, seed=9), rnd(1, 1, 32, seed=10)
     def score(p, s, theta=1e6):

@@ -8,7 +8,7 @@ import torch
 
 from gpu_util import DEV
 from plain import qwen2_plain as P
-from tiny_configs import CONFIGS, TINY_A, make_model_dir, random_prompt, read_for_plain
+from tiny_configs import CONFIGS, TINY_A, make_model_dir, random_prompt, read_for_plain, sharpen_attention
 
 pytestmark = pytest.mark.gpu
 
@@ -289,3 +289,27 @@ def test_long_prompts_at_head_size_64(tmp_path, dtype):
         allowed = {torch.float32: 1e-4 + 1e-4 * scale, torch.bfloat16: 3e-2 * scale, torch.float16: 3e-2 / 8 * scale}[dtype]
         err = (got - ref[where]).abs().max().item()
         assert err <= allowed, f"max error {err:.3e}, allowed {allowed:.3e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_yarn_on_the_gpu(tmp_path, dtype):
+    """YaRN through the kernels (crates/mach-model/src/ref_model.rs:636-704): the scaled frequencies go to the rotation
+    kernels as their table, the factors to the attention kernels as the scores' scale; a prompt in portions, then
+    decoded tokens (the fused decode kernel rotates by the same table), positions far beyond the original context."""
+    from machserve_amd.engine import StepEntry, load_model
+    from machserve_amd.weights import write_random_model
+    raw = dict(TINY_A, max_position_embeddings=1024,
+               rope_scaling={"type": "yarn", "factor": 8.0, "original_max_position_embeddings": 64, "mscale": 0.8, "mscale_all_dim": 0.707})
+    d = write_random_model(raw, 3, str(tmp_path / "yarn"))
+    sharpen_attention(d, 4.0)
+    w, sizes = read_for_plain(d)
+    toks = random_prompt(620, 512, 5)
+    ref = P.forward(_stored(w, dtype), sizes, toks)
+    lm = load_model(d, dtype=dtype, device=DEV, page_size=16, num_pages=40, max_requests=1)
+    slot = lm.cache.admit()
+    got = [lm.step([StepEntry(slot, toks[:400], list(range(400)))]), lm.step([StepEntry(slot, toks[400:600], list(range(200)))])]
+    got += [lm.step([StepEntry(slot, toks[i:i + 1], [0])]) for i in range(600, 620)]
+    got = torch.cat(got).float().cpu()
+    scale = ref.abs().max().item()
+    err = (got - ref).abs().max().item()
+    assert err <= _bound(dtype, scale), f"max error {err:.3e}"

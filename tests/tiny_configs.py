@@ -52,3 +52,16 @@ def read_for_plain(model_dir: str):
 def random_prompt(length: int, vocab: int, seed: int):
     g = torch.Generator().manual_seed(seed)
     return torch.randint(0, vocab, (length,), generator=g).tolist()
+
+
+def sharpen_attention(model_dir: str, by: float) -> None:
+    """Multiplies the query and key projections (weights and biases) of a written model by `by`: the scores grow by
+    its square, the softmax stops being nearly flat, and what changes a score (a rotation angle, a scale) shows in
+    the logits, which it hardly does with small random weights."""
+    from safetensors.torch import load_file, save_file
+    path = os.path.join(model_dir, "model.safetensors")
+    w = load_file(path)
+    for name in w:
+        if ".q_proj." in name or ".k_proj." in name:
+            w[name] = (w[name].float() * by).to(w[name].dtype)
+    save_file(w, path)
