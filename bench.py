@@ -217,7 +217,7 @@ def measured_peaks(dtype_name):
         best = min(best, a.elapsed_time(b))
     out["copy_GBs"] = round(2 * (1 << 30) / (best * 1e-3) / 1e9, 1)
     del src, dst
-    lib = ctypes.CDLL(build.ensure_library("probe", dtype_name))
+    lib = ctypes.CDLL(build_probe(dtype_name))
     blocks, iters = 4096, 2048 if dtype_name == "bf16" else 1024
     buf = torch.empty(blocks * 256, dtype=torch.float32, device="cuda:0")
     flops = ctypes.c_double(0.0)
@@ -233,6 +233,14 @@ def measured_peaks(dtype_name):
         best = min(best, a.elapsed_time(b))
     out["mfma_TFLOPs"] = round(flops.value / (best * 1e-3) / 1e12, 1)
     return out
+
+
+def build_probe(dtype_name, force=False):
+    """The matrix-core measurement beside this file, compiled into a library of its own (this benchmark's, not the
+    package's: nothing on the product path loads it)."""
+    from machserve_amd.kernels import build
+    here = os.path.dirname(os.path.abspath(__file__))
+    return build.ensure_extra_library("bench_mfma_probe", dtype_name, os.path.join(here, "bench_mfma_probe.hip"), force)
 
 
 def main() -> int:

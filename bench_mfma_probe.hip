@@ -1,6 +1,6 @@
 // What the matrix cores of the device at hand give a loop of nothing but matrix instructions: the
 // denominator "measured on the box" beside the published peak that the benchmark prices against.
-// Built as a library of its own, loaded by bench.py only; nothing on the product path calls it.
+// Built by bench.py as a library of its own; nothing on the product path calls it.
 //
 // Role in the reference: none (its benchmarks report times only, docs/benchmark-protocol.md:43-75).
 #include "common.cuh"

@@ -143,6 +143,19 @@ __device__ __forceinline__ void arguments_now(T... v) {
     (argument_now(v), ...);
 }
 
+// ---- the activation of a gated feed-forward ----------------------------------------
+// act(g) = g * sigmoid(u): u = g is SiLU; u = 2 sqrt(2 / pi) (g + 0.044715 g^3) is the tanh form of GELU,
+// since 0.5 g (1 + tanh(z)) = g * sigmoid(2 z).  Which one is an argument of the products that apply it.
+enum GateActivation { ACT_SILU = 0, ACT_GELU_TANH = 1, ACT_COUNT = 2 };
+__device__ __forceinline__ float gate_activation(float g, int act) {
+    const float u = act == ACT_GELU_TANH ? 1.5957691216057308f * (g + 0.044715f * g * g * g) : g;
+#ifdef MS_ELEM_HALF
+    return g / (1.0f + __expf(-u));
+#else
+    return g / (1.0f + expf(-u));
+#endif
+}
+
 // ---- reductions -----------------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

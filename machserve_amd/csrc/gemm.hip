@@ -44,15 +44,8 @@ struct EpiArgs {
     const float* row_ss;  // [ss_parts, M] or null
     int ss_parts;
     float ss_eps;
+    int act;            // SWIGLU: the activation on the gate (GateActivation)
 };
-
-__device__ __forceinline__ float silu_f(float g) {
-#ifdef MS_ELEM_HALF
-    return g / (1.0f + __expf(-g));
-#else
-    return g / (1.0f + expf(-g));
-#endif
-}
 
 template <int BM, int BN, int WM, int WN, int BK, int EPI, int STAGES = 2, bool SCALED = false>
 __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A, const elem_t* __restrict__ W,
@@ -328,7 +321,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
                             gv *= f[e];
                             uv *= f[e];
                         }
-                        out[(size_t)row * ep.ldo + col] = from_f32<elem_t>(silu_f(gv) * uv);
+                        out[(size_t)row * ep.ldo + col] = from_f32<elem_t>(gate_activation(gv, ep.act) * uv);
                     }
                 }
             }
@@ -508,12 +501,13 @@ extern "C" int ms_linear_residual(const void* a, const void* w, float* x, int M,
     return launch_gemm<EPI_RESIDUAL>((const elem_t*)a, (const elem_t*)w, M, N, K, ep, stream);
 }
 
-// out[M, I] = silu(a g^T) * (a u^T) where w holds gate and up rows interleaved in blocks of 16:
+// out[M, I] = act(a g^T) * (a u^T) where w holds gate and up rows interleaved in blocks of 16:
 // rows [32 t, 32 t + 16) are gate rows [16 t, 16 t + 16), rows [32 t + 16, 32 t + 32) the same
 // up rows; w has 2 * ceil16(I) rows, the padding rows being zero.
-extern "C" int ms_linear_swiglu(const void* a, const void* w, void* out, int M, int I, int K, hipStream_t stream) {
+extern "C" int ms_linear_swiglu(const void* a, const void* w, void* out, int M, int I, int K, int act, hipStream_t stream) {
+    MS_REQUIRE(act >= 0 && act < ACT_COUNT, "gated product: no activation %d", act);
     const int n = 2 * ceil_div(I, 16) * 16;
-    EpiArgs ep{out, nullptr, I, I, 0, 0};
+    EpiArgs ep{out, nullptr, I, I, 0, 0, nullptr, 0, 0.f, act};
     return launch_gemm<EPI_SWIGLU>((const elem_t*)a, (const elem_t*)w, M, n, K, ep, stream);
 }
 
@@ -531,18 +525,19 @@ extern "C" int ms_swiglu_scaled_takes(int M, int I, int K) {
 // ms_linear_swiglu for rows that came in multiplied by a norm's weight only: both products of a row are
 // divided by the row's root mean square, 1 / sqrt(sum_p row_ss[p, row] / K + eps), before the activation.
 extern "C" int ms_linear_swiglu_scaled(const void* a, const float* row_ss, int ss_parts, float eps, const void* w, void* out, int M, int I,
-                                       int K, hipStream_t stream) {
+                                       int K, int act, hipStream_t stream) {
 #ifdef MS_ELEM_HALF
+    MS_REQUIRE(act >= 0 && act < ACT_COUNT, "gated product: no activation %d", act);
     MS_REQUIRE(ms_swiglu_scaled_takes(M, I, K), "gated product with row factors: M=%d K=%d is not taken", M, K);
     MS_REQUIRE(row_ss && ss_parts >= 1, "gated product with row factors: the rows' sums of squares are missing");
     MS_REQUIRE((reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0, "gemm: operands must be 16-byte aligned");
     const int n = 2 * ceil_div(I, 16) * 16;
-    EpiArgs ep{out, nullptr, I, I, K, 0, row_ss, ss_parts, eps};
+    EpiArgs ep{out, nullptr, I, I, K, 0, row_ss, ss_parts, eps, act};
     hipLaunchKernelGGL((gemm_kernel<64, 64, 2, 2, 64, EPI_SWIGLU, 4, true>), dim3((unsigned)ceil_div(n, 64), 1), dim3(256), 0, stream,
                        (const elem_t*)a, (const elem_t*)w, M, n, K, ep);
     return check_launch("gemm 64x64x64 deep, row factors");
 #else
-    (void)a; (void)row_ss; (void)ss_parts; (void)eps; (void)w; (void)out; (void)M; (void)I; (void)K; (void)stream;
+    (void)a; (void)row_ss; (void)ss_parts; (void)eps; (void)w; (void)out; (void)M; (void)I; (void)K; (void)act; (void)stream;
     MS_REQUIRE(false, "gated product with row factors: built for bfloat16 only");
 #endif
 }

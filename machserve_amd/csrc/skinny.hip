@@ -39,15 +39,8 @@ struct SkinnyArgs {
     const float* row_ss;  // [ss_parts, M] or null
     int ss_parts;
     float ss_eps;
+    int act;          // SK_SWIGLU: the activation on the gate (GateActivation)
 };
-
-__device__ __forceinline__ float silu_sk(float g) {
-#ifdef MS_ELEM_HALF
-    return g / (1.0f + __expf(-g));
-#else
-    return g / (1.0f + expf(-g));
-#endif
-}
 
 // A block of eight waves puts two on every SIMD; with more than 128 registers a wave a CU then holds one
 // block, and a grid of more blocks than CUs (the gated product: 304 for 9,728 columns) runs in two rounds
@@ -59,7 +52,7 @@ constexpr int skinny_waves_per_simd() { return (WN * KSI == 8 && MT == 1 && NT <
 template <int MT, int NT, int WN, int KSI, int EPI>
 __global__ __launch_bounds__(64 * WN * KSI, (skinny_waves_per_simd<MT, NT, WN, KSI, EPI>())) void gemm_skinny_kernel(SkinnyArgs a) {
     arguments_now(a.A, a.W, a.out, a.M, a.N, a.K, a.k_per_wave);
-    if constexpr (EPI == SK_SWIGLU) arguments_now(a.n_out, a.row_ss, a.ss_parts, a.ss_eps);
+    if constexpr (EPI == SK_SWIGLU) arguments_now(a.n_out, a.row_ss, a.ss_parts, a.ss_eps, a.act);
     if constexpr (EPI == SK_RESIDUAL_PRENORM) arguments_now(a.norm_w, a.hn, a.ss_part);
     __shared__ float red[(KSI > 1 ? (KSI - 1) : 1) * WN * NT * 4 * 64];  // one row tile of every slice at a time
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -249,7 +242,7 @@ __global__ __launch_bounds__(64 * WN * KSI, (skinny_waves_per_simd<MT, NT, WN, K
                 for (int e = 0; e < 4; ++e) {
                     const int row = i * 16 + grp * 4 + e;
                     if (row < a.M && col < a.n_out)
-                        out[(size_t)row * a.n_out + col] = from_f32<elem_t>(silu_sk(acc[i][j][e] * f[e]) * (acc[i][j + 1][e] * f[e]));
+                        out[(size_t)row * a.n_out + col] = from_f32<elem_t>(gate_activation(acc[i][j][e] * f[e], a.act) * (acc[i][j + 1][e] * f[e]));
                 }
             }
     } else if constexpr (EPI == SK_RESIDUAL_PRENORM) {
@@ -329,11 +322,12 @@ struct SkinnyNormArgs {
     void* out;              // SK_STORE_F32: float [M, N]; SK_SWIGLU: elem [M, n_out]
     int M, N, K, k_per_wave, n_out;
     float eps;
+    int act;                // SK_SWIGLU: the activation on the gate (GateActivation)
 };
 
 template <int NT, int KSI, int EPI, int NP>
 __global__ __launch_bounds__(64 * KSI) void gemm_skinny_norm_kernel(SkinnyNormArgs a) {
-    arguments_now(a.x, a.partials, a.partial_stride, a.norm_w, a.x_out, a.W, a.out, a.M, a.N, a.K, a.k_per_wave, a.n_out, a.eps);
+    arguments_now(a.x, a.partials, a.partial_stride, a.norm_w, a.x_out, a.W, a.out, a.M, a.N, a.K, a.k_per_wave, a.n_out, a.eps, a.act);
     static_assert(KSI > 1, "the slices of K are waves of one block");
     __shared__ float red[(KSI - 1) * NT * 4 * 64];
     __shared__ float ss_part[KSI][16];
@@ -443,7 +437,7 @@ __global__ __launch_bounds__(64 * KSI) void gemm_skinny_norm_kernel(SkinnyNormAr
             for (int e = 0; e < 4; ++e) {
                 const int r = grp * 4 + e;
                 if (r < a.M && col < a.n_out)
-                    out[(size_t)r * a.n_out + col] = from_f32<elem_t>(silu_sk(acc[j][e] * inv[e]) * (acc[j + 1][e] * inv[e]));
+                    out[(size_t)r * a.n_out + col] = from_f32<elem_t>(gate_activation(acc[j][e] * inv[e], a.act) * (acc[j + 1][e] * inv[e]));
             }
         }
     } else {
@@ -602,10 +596,11 @@ extern "C" int ms_linear_skinny(const void* a, const void* w, float* out, int M,
     return launch_skinny<SK_STORE_F32>(args, plan_skinny(M, N, K, allow_partials != 0), stream);
 }
 
-// out[M, I] = silu(a g^T) * (a u^T), gate and up rows interleaved in blocks of 16 (see ms_linear_swiglu).
-extern "C" int ms_linear_swiglu_skinny(const void* a, const void* w, void* out, int M, int I, int K, hipStream_t stream) {
+// out[M, I] = act(a g^T) * (a u^T), gate and up rows interleaved in blocks of 16 (see ms_linear_swiglu).
+extern "C" int ms_linear_swiglu_skinny(const void* a, const void* w, void* out, int M, int I, int K, int act, hipStream_t stream) {
+    MS_REQUIRE(act >= 0 && act < ACT_COUNT, "gated product: no activation %d", act);
     const int n = 2 * ceil_div(I, 16) * 16;
-    SkinnyArgs args{(const elem_t*)a, (const elem_t*)w, out, M, n, K, 0, I};
+    SkinnyArgs args{(const elem_t*)a, (const elem_t*)w, out, M, n, K, 0, I, nullptr, nullptr, nullptr, nullptr, 0, 0.f, act};
     return launch_skinny<SK_SWIGLU>(args, plan_skinny(M, n, K, false, true), stream);
 }
 
@@ -624,11 +619,12 @@ extern "C" int ms_swiglu_scaled_skinny_takes(int M, int I, int K) {
 // ms_linear_swiglu_skinny for rows that came in multiplied by a norm's weight only: both products of a row are
 // divided by the row's root mean square, 1 / sqrt(sum_p row_ss[p, row] / K + eps), before the activation.
 extern "C" int ms_linear_swiglu_scaled_skinny(const void* a, const float* row_ss, int ss_parts, float eps, const void* w, void* out,
-                                              int M, int I, int K, hipStream_t stream) {
+                                              int M, int I, int K, int act, hipStream_t stream) {
+    MS_REQUIRE(act >= 0 && act < ACT_COUNT, "gated product: no activation %d", act);
     MS_REQUIRE(ms_swiglu_scaled_skinny_takes(M, I, K), "few-rows gated product with row factors: M=%d I=%d K=%d is not taken", M, I, K);
     MS_REQUIRE(row_ss && ss_parts >= 1, "few-rows gated product with row factors: the rows' sums of squares are missing");
     const int n = 2 * ceil_div(I, 16) * 16;
-    SkinnyArgs args{(const elem_t*)a, (const elem_t*)w, out, M, n, K, 0, I, nullptr, nullptr, nullptr, row_ss, ss_parts, eps};
+    SkinnyArgs args{(const elem_t*)a, (const elem_t*)w, out, M, n, K, 0, I, nullptr, nullptr, nullptr, row_ss, ss_parts, eps, act};
     return launch_skinny<SK_SWIGLU>(args, plan_skinny(M, n, K, false, true), stream);
 }
 
@@ -649,12 +645,13 @@ extern "C" int ms_linear_norm_skinny(const float* x, const float* partials, int 
     return launch_skinny_norm<SK_STORE_F32>(a, n_partials, stream);
 }
 
-// out[M, I] = silu(h g^T) * (h u^T) with h = rmsnorm(x + sum partials), gate and up rows interleaved in blocks of 16.
+// out[M, I] = act(h g^T) * (h u^T) with h = rmsnorm(x + sum partials), gate and up rows interleaved in blocks of 16.
 extern "C" int ms_linear_swiglu_norm_skinny(const float* x, const float* partials, int n_partials, int T, const float* norm_w,
-                                            float eps, float* x_out, const void* w, void* out, int M, int I, int K,
+                                            float eps, float* x_out, const void* w, void* out, int M, int I, int K, int act,
                                             hipStream_t stream) {
+    MS_REQUIRE(act >= 0 && act < ACT_COUNT, "gated product: no activation %d", act);
     const int n = 2 * ceil_div(I, 16) * 16;
-    SkinnyNormArgs a{x, partials ? partials : x, (size_t)T * K, norm_w, n_partials ? x_out : nullptr, (const elem_t*)w, out, M, n, K, 0, I, eps};
+    SkinnyNormArgs a{x, partials ? partials : x, (size_t)T * K, norm_w, n_partials ? x_out : nullptr, (const elem_t*)w, out, M, n, K, 0, I, eps, act};
     return launch_skinny_norm<SK_SWIGLU>(a, n_partials, stream);
 }
 

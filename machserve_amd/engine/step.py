@@ -362,7 +362,8 @@ class StepFunction:
         taken on the device: the host need not have seen them.  None if the step cannot take this
         path or its shape has not come often enough to be captured; ``OutOfPages`` before anything
         ran if the pages are not there."""
-        if not (self.use_graphs and all(len(e.tokens) == 1 and e.positions is None for e in entries)
+        if not (self.use_graphs and self.model.observer is None
+                and all(len(e.tokens) == 1 and e.positions is None for e in entries)
                 and len({e.slot for e in entries}) == len(entries)):
             return None
         slots = [e.slot for e in entries]
@@ -410,7 +411,8 @@ class StepFunction:
         cache = self.cache
         checked = self._check_entries(entries)  # a step that is refused has taken nothing
         self._take_pages(entries)
-        graphs = self.use_graphs and all(e.positions is None for e in entries)  # a captured step takes positions from the cache
+        # a captured step takes positions from the cache, and shows no layer's stream to an observer
+        graphs = self.use_graphs and self.model.observer is None and all(e.positions is None for e in entries)
         if graphs and all(len(e.tokens) == 1 for e in entries) and len({e.slot for e in entries}) == len(entries):
             built, key, pad = self._decode_shape(checked, False)
             if self._ready(key, self.DECODE_CAPTURE_AFTER):

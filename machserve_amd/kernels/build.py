@@ -67,8 +67,6 @@ def _hipcc() -> str:
 def _sources_of(kind: str):
     if kind == "core":
         return list(CORE_SOURCES)
-    if kind == "probe":  # the benchmark's measurement of the matrix cores; nothing on the product path loads it
-        return ["errors.hip", "probe.hip"]
     return ["errors.hip", "attention.hip"]
 
 
@@ -86,8 +84,8 @@ def _digest(sources, defines) -> str:
     h.update(" ".join(FLAGS + defines).encode())
     headers = {f for f in os.listdir(CSRC) if f.endswith((".cuh", ".h"))}
     for f in sorted(set(sources) | headers):
-        with open(os.path.join(CSRC, f), "rb") as fh:
-            h.update(f.encode())
+        with open(os.path.join(CSRC, f), "rb") as fh:   # a source outside the folder is given by its full path
+            h.update(os.path.basename(f).encode())
             h.update(fh.read())
     return h.hexdigest()
 
@@ -124,6 +122,16 @@ def _lock_of(name: str) -> threading.Lock:
 def ensure_library(kind: str, elem: str, nd: int | None = None, force: bool = False) -> str:
     """Path of the built library; compiles it first if it is missing or stale (or ``force``)."""
     name, sources, defines = _spec(kind, elem, nd)
+    return _ensure(name, sources, defines, force)
+
+
+def ensure_extra_library(name: str, elem: str, source: str, force: bool = False) -> str:
+    """A library of the caller's own: one HIP source given by its path, which may include this package's
+    headers and is linked with its error channel; built with the same flags and kept beside the others."""
+    return _ensure(f"{name}_{elem}", ["errors.hip", os.path.abspath(source)], [ELEM_DEFINE[elem]], force)
+
+
+def _ensure(name: str, sources, defines, force: bool) -> str:
     libdir = _lib_dir()
     so = os.path.join(libdir, f"lib{name}.so")
     stamp = so + ".stamp"
@@ -138,12 +146,12 @@ def ensure_library(kind: str, elem: str, nd: int | None = None, force: bool = Fa
         os.makedirs(objdir, exist_ok=True)
         _say(f"compiling {name} for {ARCH} ({len(sources)} files)")
         t0 = time.time()
-        objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in sources]
+        objs = [os.path.join(objdir, os.path.basename(s).replace(".hip", ".o")) for s in sources]
 
         def one(pair):
             src, obj = pair
-            cmd = [hipcc, *FLAGS, *[f"-D{d}" for d in defines], "-c", os.path.join(CSRC, src), "-o", obj]
-            _run_with_heartbeat(cmd, f"{name}/{src}")
+            cmd = [hipcc, *FLAGS, *[f"-D{d}" for d in defines], f"-I{CSRC}", "-c", os.path.join(CSRC, src), "-o", obj]
+            _run_with_heartbeat(cmd, f"{name}/{os.path.basename(src)}")
 
         with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
             list(pool.map(one, zip(sources, objs)))
@@ -214,7 +222,6 @@ def build_all(force: bool = True, workers: int = 4) -> list:
     jobs = []
     for elem in ELEM_DEFINE:
         jobs.append(("core", elem, None))
-        jobs.append(("probe", elem, None))
         for nd in ATTENTION_TILES:
             jobs.append(("attention", elem, nd))
     with ThreadPoolExecutor(max_workers=workers) as pool:

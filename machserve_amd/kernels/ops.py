@@ -284,9 +284,10 @@ class HipOps:
         return hn, ss
 
     def linear_swiglu_scaled(self, hn: torch.Tensor, row_ss: torch.Tensor, eps: float, w_gate_up: torch.Tensor,
-                             intermediate: int) -> torch.Tensor:
+                             intermediate: int, activation: str = "silu") -> torch.Tensor:
         """:meth:`linear_swiglu` of rows ``hn`` that lack their norm's division: both products of a row are
         divided by ``sqrt(sum(row_ss[:, row]) / K + eps)`` before the activation."""
+        act = gate_activation_code(activation)
         M, N, K = self._mm_operands(hn, w_gate_up, "linear_swiglu_scaled")
         if N != 2 * ((intermediate + 15) // 16) * 16:
             raise KernelError(f"linear_swiglu_scaled: interleaved weight has {N} rows for intermediate size {intermediate}")
@@ -295,19 +296,21 @@ class HipOps:
         few_rows = bool(self._plan("ms_swiglu_scaled_skinny_takes", M, intermediate, K))
         fn = self._core.ms_linear_swiglu_scaled_skinny if few_rows else self._core.ms_linear_swiglu_scaled
         self._check(self._core, fn(_ptr(hn), _ptr(row_ss), _c_int(row_ss.shape[0]), _c_float(eps), _ptr(w_gate_up), _ptr(out),
-                                   _c_int(M), _c_int(intermediate), _c_int(K), self._stream()))
+                                   _c_int(M), _c_int(intermediate), _c_int(K), _c_int(act), self._stream()))
         return out
 
-    def linear_swiglu(self, a: torch.Tensor, w_gate_up: torch.Tensor, intermediate: int) -> torch.Tensor:
-        """``silu(a @ gate.T) * (a @ up.T)`` with gate and up rows interleaved in blocks of 16
-        (see :func:`interleave_gate_up`)."""
+    def linear_swiglu(self, a: torch.Tensor, w_gate_up: torch.Tensor, intermediate: int, activation: str = "silu") -> torch.Tensor:
+        """``act(a @ gate.T) * (a @ up.T)`` with gate and up rows interleaved in blocks of 16
+        (see :func:`interleave_gate_up`); ``activation`` is one of :data:`GATE_ACTIVATIONS` (SiLU gives the
+        method its name)."""
+        act = gate_activation_code(activation)
         M, N, K = self._mm_operands(a, w_gate_up, "linear_swiglu")
         if N != 2 * ((intermediate + 15) // 16) * 16:
             raise KernelError(f"linear_swiglu: interleaved weight has {N} rows for intermediate size {intermediate}")
         out = torch.empty((M, intermediate), dtype=self.dtype, device=a.device)
         fn = self._core.ms_linear_swiglu if self._tiled(M, N, K) else self._core.ms_linear_swiglu_skinny
         self._check(self._core, fn(_ptr(a), _ptr(w_gate_up), _ptr(out), _c_int(M), _c_int(intermediate), _c_int(K),
-                                   self._stream()))
+                                   _c_int(act), self._stream()))
         return out
 
     # ------------------------------------------------------------------ products with the norm folded in
@@ -343,16 +346,17 @@ class HipOps:
         return out, x_new
 
     def linear_swiglu_normed(self, x: torch.Tensor, partials: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float,
-                             w_gate_up: torch.Tensor, intermediate: int):
-        """``silu(h @ gate.T) * (h @ up.T)`` for ``h = rmsnorm(x + sum(partials))`` (see
+                             w_gate_up: torch.Tensor, intermediate: int, activation: str = "silu"):
+        """``act(h @ gate.T) * (h @ up.T)`` for ``h = rmsnorm(x + sum(partials))`` (see
         :meth:`linear_swiglu`), and the stream with the pending sums added (or None)."""
+        act = gate_activation_code(activation)
         M, N, K, P, x_new = self._normed_operands(x, partials, norm_w, w_gate_up, "linear_swiglu_normed")
         if N != 2 * ((intermediate + 15) // 16) * 16:
             raise KernelError(f"linear_swiglu_normed: interleaved weight has {N} rows for intermediate size {intermediate}")
         out = torch.empty((M, intermediate), dtype=self.dtype, device=x.device)
         self._check(self._core, self._core.ms_linear_swiglu_norm_skinny(
             _ptr(x), _ptr(partials), _c_int(P), _c_int(M), _ptr(norm_w), _c_float(eps), _ptr(x_new), _ptr(w_gate_up), _ptr(out),
-            _c_int(M), _c_int(intermediate), _c_int(K), self._stream()))
+            _c_int(M), _c_int(intermediate), _c_int(K), _c_int(act), self._stream()))
         return out, x_new
 
     # ------------------------------------------------------------------ attention
@@ -551,6 +555,18 @@ class HipOps:
         self._want(delta, torch.float32, "logit_edit deltas", n)
         self._check(self._core, self._core.ms_logit_edit(_ptr(logits), _c_int(logits.shape[1]), _ptr(row_of), _ptr(token),
                                                          _ptr(delta), _c_int(n), self._stream()))
+
+
+# The activations a gated product applies to its gate branch, by the name a specification gives them, and the
+# number the kernels know them by.
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def gate_activation_code(name: str) -> int:
+    try:
+        return GATE_ACTIVATIONS[name]
+    except KeyError:
+        raise KernelError(f"gated product: activation {name!r} is not built (built: {', '.join(sorted(GATE_ACTIVATIONS))})") from None
 
 
 def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:

@@ -160,9 +160,9 @@ class PendingNorm:
         """``norm(x) @ w.T`` as float32 ``[P, T, N]`` partial sums."""
         return self.stream.ops.linear_split(self.tensor(), w)
 
-    def linear_swiglu(self, w_gate_up: torch.Tensor, intermediate: int) -> torch.Tensor:
-        """``silu(h @ gate.T) * (h @ up.T)`` for ``h = norm(x)``."""
-        return self.stream.ops.linear_swiglu(self.tensor(), w_gate_up, intermediate)
+    def linear_swiglu(self, w_gate_up: torch.Tensor, intermediate: int, activation: str = "silu") -> torch.Tensor:
+        """``act(h @ gate.T) * (h @ up.T)`` for ``h = norm(x)``."""
+        return self.stream.ops.linear_swiglu(self.tensor(), w_gate_up, intermediate, activation)
 
 
 def require_kernel_sizes(rt: "Runtime", what: str, reductions=(), head_dim: Optional[int] = None,

@@ -74,6 +74,10 @@ class DecoderModel:
         self.final_norm = NORMS.build(spec.final_norm, rt)
         self.head = HEADS.build(spec.head, rt, self.embedding)
         self._bindings, self._rebind = [], False
+        # Debugging aid: a callable (name, float32 stream [rows, width]) that sees the residual stream after the
+        # embedding and after every run of a layer (crates/mach-model/src/batched.rs:3040-3088 dumps the same
+        # points).  While it is set the step function runs every step as it is, from no captured graph.
+        self.observer = None
 
     # ------------------------------------------------------------------ structure
     def parts(self) -> List[Part]:
@@ -139,10 +143,15 @@ class DecoderModel:
         """Run the step's rows through the layers in ``order``; float32 logits ``[W, vocab]`` of
         the wanted rows, or None when none is wanted."""
         stream = ResidualStream(self.embedding.forward(ctx.tokens), self.rt.ops)
+        watch = self.observer
+        if watch is not None:
+            watch("embedding", stream.value())
         for p, i in enumerate(self.order):
             if self._rebind and self._bindings[p] is not None:
                 self.blocks[i].bind_cache(self._bindings[p])
             self.blocks[i].forward(stream, ctx)
+            if watch is not None:  # the sums still pending are added first: the value is the whole stream
+                watch(f"layer{p:02d}", stream.value())
         if ctx.want_rows.numel() == 0:
             return None
         return self.head.forward(self.final_norm.forward(stream, rows=ctx.want_rows))

@@ -47,7 +47,7 @@ class PendingRMSNorm(PendingNorm):
             return out
         return ops.linear_split(self.tensor(), w)
 
-    def linear_swiglu(self, w_gate_up, intermediate):
+    def linear_swiglu(self, w_gate_up, intermediate, activation="silu"):
         stream, ops, weight, eps = self.stream, self.stream.ops, self.norm.weight, self.norm.spec.eps
         if stream.deferred is not None and stream.pending is None:
             # a product that is still to be added: where the kernels can, it leaves what the norm needs beside its
@@ -57,13 +57,13 @@ class PendingRMSNorm(PendingNorm):
             if takes is not None and takes(a.shape[0], w.shape[0], w.shape[1], w_gate_up.shape[0]):
                 stream.deferred = None
                 hn, row_ss = ops.linear_residual_prenorm(a, w, stream.x, weight)
-                return ops.linear_swiglu_scaled(hn, row_ss, eps, w_gate_up, intermediate)
+                return ops.linear_swiglu_scaled(hn, row_ss, eps, w_gate_up, intermediate, activation)
         stream.launch_deferred()
         T, K = stream.x.shape
         P = 0 if stream.pending is None else stream.pending.shape[0]
         if ops.norm_folds_into(T, w_gate_up.shape[0], K, P):
-            out, x_new = ops.linear_swiglu_normed(stream.x, stream.pending, weight, eps, w_gate_up, intermediate)
+            out, x_new = ops.linear_swiglu_normed(stream.x, stream.pending, weight, eps, w_gate_up, intermediate, activation)
             if x_new is not None:
                 stream.x, stream.pending = x_new, None
             return out
-        return ops.linear_swiglu(self.tensor(), w_gate_up, intermediate)
+        return ops.linear_swiglu(self.tensor(), w_gate_up, intermediate, activation)

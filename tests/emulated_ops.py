@@ -14,6 +14,15 @@ import torch
 MASK64 = (1 << 64) - 1
 
 
+def _act(g, activation):
+    """The activation on the gate branch of a gated product, in its textbook form."""
+    if activation == "silu":
+        return g / (1.0 + torch.exp(-g))
+    if activation == "gelu_tanh":
+        return 0.5 * g * (1.0 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g * g * g)))
+    raise ValueError(f"no activation {activation!r}")
+
+
 class EmulatedOps:
 
     def __init__(self, dtype=torch.float32, device="cpu"):
@@ -65,13 +74,13 @@ class EmulatedOps:
         a, inv, x_new = self._normed(x, partials, norm_w, eps)
         return ((a.float() @ w.float().t()) * inv).unsqueeze(0), x_new
 
-    def linear_swiglu_normed(self, x, partials, norm_w, eps, w_gate_up, intermediate):
+    def linear_swiglu_normed(self, x, partials, norm_w, eps, w_gate_up, intermediate, activation="silu"):
         a, inv, x_new = self._normed(x, partials, norm_w, eps)
         Ip = w_gate_up.shape[0] // 2
         w = w_gate_up.float().view(Ip // 16, 2, 16, -1)
         gate = (a.float() @ w[:, 0].reshape(Ip, -1).t()) * inv
         up = (a.float() @ w[:, 1].reshape(Ip, -1).t()) * inv
-        return self._r((gate / (1.0 + torch.exp(-gate)) * up)[:, :intermediate]), x_new
+        return self._r((_act(gate, activation) * up)[:, :intermediate]), x_new
 
     def linear_residual(self, a, w, x):
         if a.shape[0] <= self.SKINNY_ROWS:
@@ -79,12 +88,12 @@ class EmulatedOps:
         x += a.float() @ w.float().t()
         return None
 
-    def linear_swiglu(self, a, w_gate_up, intermediate):
+    def linear_swiglu(self, a, w_gate_up, intermediate, activation="silu"):
         Ip = w_gate_up.shape[0] // 2
         w = w_gate_up.float().view(Ip // 16, 2, 16, -1)
         gate = a.float() @ w[:, 0].reshape(Ip, -1).t()
         up = a.float() @ w[:, 1].reshape(Ip, -1).t()
-        return self._r((gate / (1.0 + torch.exp(-gate)) * up)[:, :intermediate])
+        return self._r((_act(gate, activation) * up)[:, :intermediate])
 
     def rope_kv_write(self, qkv, bias, positions, inv_freq, slot_map, kpool, vpool, H, KV, hd, page_size):
         qkv = qkv if qkv.dim() == 2 else qkv.sum(0)

@@ -203,12 +203,14 @@ def layer_windows(sizes) -> list:
     return [sizes["sliding_window"] if i >= sizes["max_window_layers"] else None for i in range(L)]
 
 
-def forward(weights: dict, sizes: dict, tokens, compute=torch.float32, start_pos: int = 0, rounded=same) -> torch.Tensor:
+def forward(weights: dict, sizes: dict, tokens, compute=torch.float32, start_pos: int = 0, rounded=same,
+            streams: list = None) -> torch.Tensor:
     """Logits ``[T, vocab]`` at every position of one whole sequence.  ``rounded`` is applied wherever a
     reduced-precision run of the same formulas stores a value in its element type: the inputs of every matrix
     product (the norms' outputs, the attention output, SiLU(gate) * up), q, and the keys and values of the
     cache, and the probabilities that multiply the values; the stream, the sums, the softmax and its
-    statistics stay as computed.  The default rounds nothing.
+    statistics stay as computed.  The default rounds nothing.  A list given as ``streams`` receives the residual
+    stream after the embedding and after every layer (crates/mach-model/src/batched.rs:3040-3088).
 
     Pre-norm blocks ``x += attn(norm(x)); x += mlp(norm(x))``, final norm, head =
     ``lm_head.weight`` when the tensor exists, else the embedding table.
@@ -219,6 +221,8 @@ def forward(weights: dict, sizes: dict, tokens, compute=torch.float32, start_pos
     toks = torch.as_tensor(tokens, dtype=torch.long)
     positions = torch.arange(start_pos, start_pos + len(toks))
     x = w["model.embed_tokens.weight"][toks]
+    keep = streams.append if streams is not None else (lambda t: None)
+    keep(x)
     windows = layer_windows(sizes)
     for i in range(sizes["layers"]):
         p = f"model.layers.{i}."
@@ -226,6 +230,7 @@ def forward(weights: dict, sizes: dict, tokens, compute=torch.float32, start_pos
         x = x + attention_block(xn, w, p + "self_attn.", positions, sizes, windows[i], rounded)
         xn = rounded(rms_norm(x, w[p + "post_attention_layernorm.weight"], sizes["eps"]))
         x = x + swiglu(xn, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"], rounded)
+        keep(x)
     xf = rounded(rms_norm(x, w["model.norm.weight"], sizes["eps"]))
     head = w["lm_head.weight"] if "lm_head.weight" in w and not sizes.get("tied", False) else w["model.embed_tokens.weight"]
     return linear(xf, head)

@@ -408,6 +408,44 @@ def test_yarn_through_the_engine_equals_the_plain_model(tmp_path, mscale_all_dim
     assert (got - ref).abs().max() <= 2e-5 * (1 + ref.abs().max())
 
 
+def test_replay_writes_every_layer_s_stream_at_the_wanted_places(tmp_path):
+    """The replay program's debugging aid (crates/mach-model/src/batched.rs:3040-3088): the residual stream after the
+    embedding and after every layer, at the wanted places of a step, equals the plain model's; a fault put into one
+    layer's weights shows in that layer's file first."""
+    import json
+    import numpy as np
+    from machserve_amd.engine import load_model
+    from machserve_amd.engine.replay import replay
+    d = make_model_dir(tmp_path, "C")
+    w, sizes = read_for_plain(d)
+    toks = random_prompt(70, sizes["vocab"], 9)
+    lm = load_model(d, dtype="float32", device="cpu", page_size=16, num_pages=12, max_requests=2, ops=EmulatedOps())
+    lines = [json.dumps({"step": 0, "entries": [{"id": "a", "tokens": toks[:50], "want": []}], "end": []}),
+             json.dumps({"step": 1, "entries": [{"id": "a", "tokens": toks[50:], "want": [3, 19]}], "end": ["a"]})]
+    out, layers = tmp_path / "out", tmp_path / "layers"
+    out.mkdir(), layers.mkdir()
+    replay(lm, lines, str(out), say=lambda m: None, layers_dir=str(layers))
+    streams = []
+    ref = P.forward(w, sizes, toks, streams=streams)
+    rows = [53, 69]
+    got = np.fromfile(out / "1.f32", dtype="<f4").reshape(2, -1)
+    assert np.abs(got - ref[rows].numpy()).max() <= 2e-5 * (1 + ref.abs().max().item())
+    names = ["embedding"] + [f"layer{i:02d}" for i in range(sizes["layers"])]
+    assert sorted(f.name for f in layers.iterdir()) == sorted(f"1_{n}.f32" for n in names)   # step 0 wanted nothing
+    for n, want in zip(names, streams):
+        g = np.fromfile(layers / f"1_{n}.f32", dtype="<f4").reshape(2, sizes["hidden"])
+        assert np.abs(g - want[rows].numpy()).max() <= 2e-5 * (1 + want.abs().max().item()), n
+    # a changed weight in layer 2: layers 0 and 1 still agree, layer 2 is the first that does not
+    w2 = dict(w)
+    w2["model.layers.2.mlp.down_proj.weight"] = w["model.layers.2.mlp.down_proj.weight"] * 1.5
+    streams2 = []
+    P.forward(w2, sizes, toks, streams=streams2)
+    differs = [n for n, want in zip(names, streams2)
+               if np.abs(np.fromfile(layers / f"1_{n}.f32", dtype="<f4").reshape(2, -1) - want[rows].numpy()).max() > 1e-4]
+    assert differs == ["layer02", "layer03"]
+    assert lm.model.observer is not None and lm.step.use_graphs is False
+
+
 def test_a_refused_step_takes_no_pages(tmp_path):
     """A step with a bad token, a slot twice, a place beyond its tokens, or a slot that no request holds is refused
     before anything is taken: the tables, the free pages and the lengths are what they were."""

@@ -245,6 +245,42 @@ def test_a_large_or_tiny_stream_goes_through_the_norm_and_its_reader(dtype, scal
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,I,K", [(1, 4864, 896), (9, 168, 64), (16, 4864, 896), (200, 328, 192), (40, 1000, 576)])
+def test_gated_products_with_another_activation(dtype, M, I, K):
+    """The activation on the gate is an argument: the tanh form of GELU (crates/mach-model/src/kernels.rs:199-208)
+    against the library's own, through every kernel that applies an activation: the tiled and the few-rows gated
+    product, the one that applies the stream's norm itself, and the one that divides its finished sums."""
+    import torch.nn.functional as F
+    from machserve_amd.kernels import KernelError, interleave_gate_up
+    ops = ops_for(dtype)
+    gelu = lambda t: F.gelu(t, approximate="tanh")
+    a, g, u = rnd((M, K), dtype, 9), rnd((I, K), dtype, 10, K ** -0.5), rnd((I, K), dtype, 11, K ** -0.5)
+    gate, up = P.linear(a.double(), g.double()), P.linear(a.double(), u.double())
+    ref = gelu(gate) * up
+    assert (ref - P.silu(gate) * up).abs().max() > 0.03 * ref.abs().max(), "the test must tell the activations apart"
+    w = interleave_gate_up(g, u).to(DEV)
+    assert_close(ops.linear_swiglu(a.to(DEV), w, I, "gelu_tanh"), ref, dtype, "gated product, GELU")
+    assert_close(ops.linear_swiglu(a.to(DEV), w, I, "silu"), P.silu(gate) * up, dtype, "gated product, SiLU by name")
+    with pytest.raises(KernelError, match="gelu_erf"):
+        ops.linear_swiglu(a.to(DEV), w, I, "gelu_erf")
+    eps = 1e-5
+    x, nw = rnd((M, K), torch.float32, 12, 2.0), 1 + rnd((K,), torch.float32, 13, 0.1)
+    h = P.rms_norm(x, nw, eps).double()
+    ref = gelu(P.linear(h, g.double())) * P.linear(h, u.double())
+    if ops.norm_folds_into(M, w.shape[0], K, 0):
+        got, _ = ops.linear_swiglu_normed(x.to(DEV), None, nw.to(DEV), eps, w, I, "gelu_tanh")
+        assert_close(got, ref, dtype, "gated product of the normed stream, GELU")
+    Ka = 72
+    if ops.prenorm_swiglu_takes(M, K, Ka, w.shape[0]):
+        b, wo = rnd((M, Ka), dtype, 14), rnd((K, Ka), dtype, 15, Ka ** -0.5)
+        xd = x.to(DEV).clone()
+        hn, ss = ops.linear_residual_prenorm(b.to(DEV), wo.to(DEV), xd, nw.to(DEV))
+        h = P.rms_norm(xd.cpu(), nw, eps).double()
+        ref = gelu(P.linear(h, g.double())) * P.linear(h, u.double())
+        assert_close(ops.linear_swiglu_scaled(hn, ss, eps, w, I, "gelu_tanh"), ref, dtype, "gated product with row factors, GELU")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,I,K", [(1, 16, 8), (9, 160, 64), (70, 328, 192), (200, 4864, 896), (64, 4864, 896), (33, 264, 136),
                                    (64, 328, 256), (50, 1000, 576),
                                    # tiles of 128x160 (five pairs of gate and up tiles): whole, and ragged at both edges

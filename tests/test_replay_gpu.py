@@ -409,5 +409,41 @@ def test_the_four_ways_through_the_program(models, which, dtype, tmp_path):
             at += hi - lo
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_the_program_writes_every_layer_s_stream(models, dtype, tmp_path):
+    """``bin/trace_run --dump-layers``: the residual stream after the embedding and after every layer at the wanted
+    places (crates/mach-model/src/batched.rs:3040-3088 dumps the same points), from the kernels, a prompt portion
+    beside decoded tokens of another request; the logits of the same run are those of a run without the dump."""
+    import json, os, subprocess, sys
+    import numpy as np
+    d, w, sizes, prompts, _ = models["C"]
+    a, b = prompts[2], prompts[3]                       # 130 and 47 tokens
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:100], "want": []}, {"id": "b", "tokens": b[:46], "want": []}], "end": []},
+             {"step": 1, "entries": [{"id": "b", "tokens": b[46:], "want": [0]}, {"id": "a", "tokens": a[100:], "want": [0, 29]}], "end": ["a", "b"]}]
+    root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..")
+    name = {torch.float32: "float32", torch.bfloat16: "bfloat16"}[dtype]
+    outs = {}
+    for how in ("plainly", "dumping"):
+        out = tmp_path / how
+        cmd = [sys.executable, os.path.join(root, "bin", "trace_run"), "--model", d, "--dtype", name, "--out", str(out), "--max-tokens", "256"]
+        if how == "dumping":
+            cmd += ["--dump-layers", str(tmp_path / "layers")]
+        r = subprocess.run(cmd, input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600)
+        assert r.returncode == 0, r.stderr[-2000:]
+        outs[how] = np.fromfile(out / "1.f32", dtype="<f4").reshape(3, sizes["vocab"])
+    scale = np.abs(outs["plainly"]).max()
+    assert np.abs(outs["plainly"] - outs["dumping"]).max() <= (1e-5 if dtype == torch.float32 else 1e-2) * scale
+    ww = w if dtype == torch.float32 else {k: v.to(dtype).float() if v.dim() == 2 else v for k, v in w.items()}
+    sa, sb = [], []
+    P.forward(ww, sizes, a, streams=sa)
+    P.forward(ww, sizes, b, streams=sb)
+    names = ["embedding"] + [f"layer{i:02d}" for i in range(sizes["layers"])]
+    for n, xa, xb in zip(names, sa, sb):
+        want = torch.stack([xb[46], xa[100], xa[129]]).numpy()
+        got = np.fromfile(tmp_path / "layers" / f"1_{n}.f32", dtype="<f4").reshape(3, sizes["hidden"])
+        bound = (2e-5 if dtype == torch.float32 else 3e-2) * (1 + np.abs(want).max())
+        assert np.abs(got - want).max() <= bound, f"{n}: {np.abs(got - want).max():.3e}"
+
+
 def test_zz_report_worst_bfloat16_error():
     print("largest errors of the reduced-precision runs, in units of the logits' scale:", WORST)

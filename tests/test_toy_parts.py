@@ -538,7 +538,7 @@ class SandwichToyConfig:
         norm = lambda name: NormSpec("rmsnorm", WIDTH, 1e-5, {"weight": name})
         names = lambda i: {k: f"l{i}.att.{k}" for k in ("q.weight", "k.weight", "v.weight", "o.weight", "q.bias", "k.bias", "v.bias")}
         att0 = AttentionSpec("attention", WIDTH, HEADS, KV, HD, RotarySpec("rotary", HD, 1e4), tensors=names(0), scale=SANDWICH_SCALE)
-        ff0 = GatedMlpSpec("gated_mlp", WIDTH, INTER, "silu", {k: f"l0.ff.{k}" for k in ("gate.weight", "up.weight", "down.weight")})
+        ff0 = GatedMlpSpec("gated_mlp", WIDTH, INTER, "gelu_tanh", {k: f"l0.ff.{k}" for k in ("gate.weight", "up.weight", "down.weight")})
         layers = (SandwichSpec("toy_sandwich", att0, ff0, (norm("l0.n1"), norm("l0.n2"), norm("l1.n1"), norm("l1.n2"))),
                   MixerOnlySpec("toy_mixer_only", AttentionSpec("attention", WIDTH, HEADS, KV, HD, RotarySpec("rotary", HD, 1e4),
                                                                 tensors=names(2)), norm("l2.n1")))
@@ -549,7 +549,7 @@ class SandwichToyConfig:
 register_architecture("SandwichToyForCausalLM", SandwichToyConfig)
 
 
-def plain_sandwich_toy(t, toks, scale0=SANDWICH_SCALE):
+def plain_sandwich_toy(t, toks, scale0=SANDWICH_SCALE, act=lambda g: torch.nn.functional.gelu(g, approximate="tanh")):
     T = len(toks)
     pos = torch.arange(T)
     x = t["emb"][torch.tensor(toks)]
@@ -565,7 +565,8 @@ def plain_sandwich_toy(t, toks, scale0=SANDWICH_SCALE):
     for i in (0, 1, 0):
         if i == 0:
             x = x + P.rms_norm(att(0, P.rms_norm(x, t["l0.n1"], 1e-5), scale0), t["l0.n2"], 1e-5)
-            y = P.swiglu(P.rms_norm(x, t["l1.n1"], 1e-5), t["l0.ff.gate.weight"], t["l0.ff.up.weight"], t["l0.ff.down.weight"])
+            xn = P.rms_norm(x, t["l1.n1"], 1e-5)
+            y = P.linear(act(P.linear(xn, t["l0.ff.gate.weight"])) * P.linear(xn, t["l0.ff.up.weight"]), t["l0.ff.down.weight"])
             x = x + P.rms_norm(y, t["l1.n2"], 1e-5)
         else:
             x = x + att(2, P.rms_norm(x, t["l2.n1"], 1e-5), HD ** -0.5)
@@ -573,8 +574,9 @@ def plain_sandwich_toy(t, toks, scale0=SANDWICH_SCALE):
 
 
 def _check_sandwich(device, ops):
-    """Blocks that build parts of their own (four norms; no feed-forward), and an attention whose scale the spec gives:
-    a request in portions beside one token by token, against the plain parts."""
+    """Blocks that build parts of their own (four norms; no feed-forward), an attention whose scale the spec gives and a
+    gated feed-forward whose activation it gives (the tanh form of GELU, the library's own as the plain one): a request
+    in portions beside one token by token, against the plain parts."""
     from machserve_amd.config import config_from_dict
     from machserve_amd.engine import StepEntry, load_model
     t = {k: v for k, v in toy_tensors().items() if k.startswith(("emb", "nf", "l0.", "l1.n", "l2.n1", "l2.att"))}
@@ -602,6 +604,9 @@ def _check_sandwich(device, ops):
         assert (out - refs[r]).abs().max() <= 2e-4 * (1 + refs[r].abs().max()), f"request {r}"
     # the test can tell the scale: with the usual one the plain model is far from this
     usual = plain_sandwich_toy(t, seqs[0], HD ** -0.5)
+    assert (usual - refs[0]).abs().max() > 50 * 2e-4 * (1 + refs[0].abs().max())
+    # ... and the activation
+    usual = plain_sandwich_toy(t, seqs[0], act=P.silu)
     assert (usual - refs[0]).abs().max() > 50 * 2e-4 * (1 + refs[0].abs().max())
 
 
