@@ -48,9 +48,10 @@ struct EpiArgs {
 };
 
 template <int BM, int BN, int WM, int WN, int BK, int EPI, int STAGES = 2, bool SCALED = false>
-__global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A, const elem_t* __restrict__ W,
+__global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const elem_t* __restrict__ A, const elem_t* __restrict__ W,
                                                    int M, int N, int K, EpiArgs ep) {
-    static_assert(WM * WN == 4, "four waves");
+    static_assert(WM * WN == 4 || WM * WN == 8, "four waves, or eight for the widest tiles");
+    constexpr int NT = 64 * WM * WN;  // threads of the block
     arguments_now(A, W, M, N, K, ep.out, ep.bias, ep.ldo, ep.n_out, ep.k_per_split, ep.split_stride);
     if constexpr (SCALED) arguments_now(ep.row_ss, ep.ss_parts, ep.ss_eps);
     static_assert(BK % 32 == 0, "K step in MFMA steps of 32");
@@ -64,8 +65,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
     // where chunk `chunk` of tile row `row` lies in a buffer
     auto at = [](int row, int chunk) { return row * LDS_LD + (DIRECT ? (chunk ^ (row & 7)) : chunk) * EPC; };
     constexpr int TM = BM / WM / 16, TN = BN / WN / 16;
-    constexpr int A_CHUNKS = BM * CPR / 256, W_CHUNKS = BN * CPR / 256;
-    static_assert(BM * CPR % 256 == 0 && BN * CPR % 256 == 0, "tile loads divide over the block");
+    constexpr int A_CHUNKS = BM * CPR / NT, W_CHUNKS = BN * CPR / NT;
+    static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0, "tile loads divide over the block");
+    static_assert(NT == 256 || !SCALED, "the row factors' shares are dealt to four waves");
     static_assert(STAGES == 2 || DIRECT, "more than two LDS buffers only with direct loads");
     static_assert(!SCALED || (STAGES > 2 && EPI == EPI_SWIGLU), "row factors: built for the gated product with several steps in flight");
     static_assert(256 % BM == 0 || !SCALED, "threads are dealt to the rows");
@@ -89,17 +91,17 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
     u32x4 ra[A_CHUNKS], rw[W_CHUNKS];
     const elem_t* pa[A_CHUNKS];
     const elem_t* pw[W_CHUNKS];
-    // Thread t owns position (t + i * 256) % CPR of tile row (t + i * 256) / CPR; with swizzled rows that
-    // position holds another chunk of K, the same one for every i (256 / CPR rows on is a multiple of 8).
+    // Thread t owns position (t + i * NT) % CPR of tile row (t + i * NT) / CPR; with swizzled rows that
+    // position holds another chunk of K, the same one for every i (NT / CPR rows on is a multiple of 8).
     const int my_chunk = DIRECT ? (tid % CPR) ^ ((tid / CPR) & 7) : tid % CPR;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
-        const int c = tid + i * 256;
+        const int c = tid + i * NT;
         pa[i] = A + (size_t)min(m0 + c / CPR, M - 1) * K + my_chunk * EPC;
     }
 #pragma unroll
     for (int i = 0; i < W_CHUNKS; ++i) {
-        const int c = tid + i * 256;
+        const int c = tid + i * NT;
         pw[i] = W + (size_t)min(n0 + c / CPR, N - 1) * K + my_chunk * EPC;
     }
     auto load_global = [&](int k0) {
@@ -126,12 +128,12 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
     auto store_lds = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < A_CHUNKS; ++i) {
-            const int c = tid + i * 256, row = c / CPR;
+            const int c = tid + i * NT, row = c / CPR;
             *reinterpret_cast<u32x4*>(&As[buf][at(row, my_chunk)]) = ra[i];
         }
 #pragma unroll
         for (int i = 0; i < W_CHUNKS; ++i) {
-            const int c = tid + i * 256, row = c / CPR;
+            const int c = tid + i * NT, row = c / CPR;
             *reinterpret_cast<u32x4*>(&Ws[buf][at(row, my_chunk)]) = rw[i];
         }
     };
@@ -146,9 +148,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(const elem_t* __restrict__ A,
             asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(base) : "memory", "m0");
         };
 #pragma unroll
-        for (int i = 0; i < A_CHUNKS; ++i) issue(pa[i] + k0, &As[buf][(i * 256 + wave * 64) * EPC]);
+        for (int i = 0; i < A_CHUNKS; ++i) issue(pa[i] + k0, &As[buf][(i * NT + wave * 64) * EPC]);
 #pragma unroll
-        for (int i = 0; i < W_CHUNKS; ++i) issue(pw[i] + k0, &Ws[buf][(i * 256 + wave * 64) * EPC]);
+        for (int i = 0; i < W_CHUNKS; ++i) issue(pw[i] + k0, &Ws[buf][(i * NT + wave * 64) * EPC]);
     };
 #endif
     // End of a K step: this wave's loads and LDS accesses have completed, then everybody's.
@@ -375,14 +377,14 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
 #define MS_GEMM_DEEP(BM_, BN_, WM_, WN_, BK_, ST_)                                                                         \
     do {                                                                                                                  \
         const long nb = (long)ceil_div(M, BM_) * ceil_div(N, BN_);                                                        \
-        hipLaunchKernelGGL((gemm_kernel<BM_, BN_, WM_, WN_, BK_, EPI, ST_>), dim3((unsigned)nb, ns), dim3(256), 0, stream, \
+        hipLaunchKernelGGL((gemm_kernel<BM_, BN_, WM_, WN_, BK_, EPI, ST_>), dim3((unsigned)nb, ns), dim3(64 * WM_ * WN_), 0, stream, \
                            A, W, M, N, K, ep);                                                                            \
         return check_launch("gemm " #BM_ "x" #BN_ "x" #BK_ " deep");                                                      \
     } while (0)
 #define MS_GEMM(BM_, BN_, WM_, WN_, BK_)                                                                              \
     do {                                                                                                              \
         const long nb = (long)ceil_div(M, BM_) * ceil_div(N, BN_);                                                    \
-        hipLaunchKernelGGL((gemm_kernel<BM_, BN_, WM_, WN_, BK_, EPI>), dim3((unsigned)nb, ns), dim3(256), 0, stream, \
+        hipLaunchKernelGGL((gemm_kernel<BM_, BN_, WM_, WN_, BK_, EPI>), dim3((unsigned)nb, ns), dim3(64 * WM_ * WN_), 0, stream, \
                            A, W, M, N, K, ep);                                                                        \
         return check_launch("gemm " #BM_ "x" #BN_ "x" #BK_);                                                          \
     } while (0)
@@ -394,12 +396,27 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
     if (forced == 6) MS_GEMM(64, 64, 2, 2, 64);
     const bool whole_steps = ep.k_per_split % 64 == 0 && K % 64 == 0;
     if (forced == 8 && whole_steps) MS_GEMM_DEEP(64, 64, 2, 2, 64, 4);
+    if (forced == 9) MS_GEMM(256, 256, 2, 4, 64);
     // The largest tile that still gives every CU of the chip a block or two, with K steps of 64 (half
-    // the barriers of steps of 32).  Measured on M = 512..8192 of the 0.5B shapes; larger wave tiles
-    // (256x128) lose: their accumulators no longer fit the registers of two blocks a CU.
+    // the barriers of steps of 32).  Measured on M = 512..8192 of the 0.5B shapes; larger tiles under
+    // four waves (256x128) lose: their accumulators no longer fit the registers of two blocks a CU.
     // two 128x128 blocks a CU are a round of the chip (512 on 256 CUs); a tile is taken when its blocks fill
     // six tenths of a round
     const long round_blocks = 2L * compute_units(), enough = round_blocks * 300 / 512;
+    if (M > 64 && ns == 1 && ep.k_per_split >= 128 && forced == 0) {
+        // Tiles of 256x256 under eight waves (each 128 rows by 64 columns: 128 accumulator registers, 220 in all, two
+        // waves a SIMD; 128 KB of LDS: one block a CU) bring half the bytes of two 128x128 tiles from the L2 into the CUs,
+        // which is what bounds the large products (every variant of the 128x128 loop pulls 13 to 15 TB/s).  They pay
+        // where the last of their rounds of one block a CU is well filled: measured against the choice below at the
+        // 0.5B, 1.5B and 7B layer sizes with 1,024 to 8,192 rows, +4 to +18 % from 0.72 of the rounds' blocks upwards
+        // (7B gate/up at 2,048 rows 604 -> 511 us, at 8,192 rows 2,167 -> 1,818 us = 1.22 PFLOP/s; 7B down at 4,096
+        // rows 588 -> 496), -15 to -44 % below 0.63; a short K (the 0.5B model's 896: fourteen steps between a tile's
+        // start and its 256x256 stores) wants the rounds nearly full (0.95: +16 %, 0.79: -5 %).  Three LDS stages
+        // (256x128, 128x256) and four of K = 32 (256x256) were slower than this.
+        const long t256 = (long)ceil_div(M, 256) * ceil_div(N, 256), cus = compute_units();
+        const long rounds = ceil_div(t256, cus);
+        if (t256 * 100 >= rounds * cus * (K >= 1536 ? 72 : 90)) MS_GEMM(256, 256, 2, 4, 64);
+    }
     if (M > 64) {
         const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128), b12864 = (long)ceil_div(M, 128) * ceil_div(N, 64);
         // The chip holds a round of such blocks at a time and a round that is nearly empty takes as long as a full one:

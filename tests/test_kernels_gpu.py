@@ -75,7 +75,10 @@ def test_rmsnorm(dtype, T, d, eps):
                                    # few tiles, whole K steps: four LDS buffers in turn, with four, five, seven and nineteen steps
                                    (64, 200, 256), (48, 264, 320), (40, 130, 448), (100, 72, 1216),
                                    # so many tiles that tiles of 128x160 save a round: whole tiles, and ragged rows and columns
-                                   (1024, 9728, 136), (1000, 9700, 264)])
+                                   (1024, 9728, 136), (1000, 9700, 264),
+                                   # tiles of 256x256 under eight waves, taken where they fill their rounds of a block a CU: whole
+                                   # tiles with two whole K steps; ragged rows and columns with a partial last step; a long K
+                                   (4096, 4096, 128), (4000, 4090, 136), (3840, 3584, 1600)])
 def test_linear(dtype, M, N, K):
     ops = ops_for(dtype)
     a, w = rnd((M, K), dtype, 5), rnd((N, K), dtype, 6, K ** -0.5)
@@ -284,7 +287,9 @@ def test_gated_products_with_another_activation(dtype, M, I, K):
 @pytest.mark.parametrize("M,I,K", [(1, 16, 8), (9, 160, 64), (70, 328, 192), (200, 4864, 896), (64, 4864, 896), (33, 264, 136),
                                    (64, 328, 256), (50, 1000, 576),
                                    # tiles of 128x160 (five pairs of gate and up tiles): whole, and ragged at both edges
-                                   (2048, 4864, 896), (1000, 4850, 200)])
+                                   (2048, 4864, 896), (1000, 4850, 200),
+                                   # tiles of 256x256 (two pairs of gate and up tiles a wave): whole, and ragged at both edges
+                                   (4096, 2048, 128), (4000, 2040, 200)])
 def test_linear_swiglu(dtype, M, I, K):
     from machserve_amd.kernels import interleave_gate_up
     ops = ops_for(dtype)
