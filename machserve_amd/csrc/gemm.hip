@@ -412,7 +412,8 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
         // (7B gate/up at 2,048 rows 604 -> 511 us, at 8,192 rows 2,167 -> 1,818 us = 1.22 PFLOP/s; 7B down at 4,096
         // rows 588 -> 496), -15 to -44 % below 0.63; a short K (the 0.5B model's 896: fourteen steps between a tile's
         // start and its 256x256 stores) wants the rounds nearly full (0.95: +16 %, 0.79: -5 %).  Three LDS stages
-        // (256x128, 128x256) and four of K = 32 (256x256) were slower than this.
+        // (256x128, 128x256), four of K = 32 (256x256: 1.13 against 1.22 PFLOP/s) and four waves of 128x128 each with
+        // their sums in the accumulation registers (1.06) were slower than this.
         const long t256 = (long)ceil_div(M, 256) * ceil_div(N, 256), cus = compute_units();
         const long rounds = ceil_div(t256, cus);
         if (t256 * 100 >= rounds * cus * (K >= 1536 ? 72 : 90)) MS_GEMM(256, 256, 2, 4, 64);
