@@ -40,6 +40,7 @@ PEAK_FLOPS = {"bf16": 2.5e15, "f16": 2.5e15, "f32": 157.3e12}
 # the reference's own numbers for this model on its hardware (RX 7900 XTX, fp16)
 REF_DECODE_B64_CTX2048 = 4777.0   # README.md:15, docs/benchmark-protocol.md:74-75
 REF_PREFILL_2048 = 2048 / 0.289   # README.md:18
+REF_DECODE_B256_SHORT = 29273.0   # docs/roadmap.md:324-325 (short contexts)
 
 QWEN25_05B = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_size": 896, "num_hidden_layers": 24,
@@ -482,6 +483,11 @@ def main() -> int:
             # the first token of a prompt of a length not seen before (the reference quotes 512 tokens, docs/roadmap.md:260-261)
             for n, (v, d) in first_token_points(args.shape, (128, 500, 512)).items():
                 points[f"first_token_{n}"], detail[f"first_token_{n}"] = round(v, 1), d
+            # many requests at short contexts, as the reference's own sweep over the batch has them (docs/roadmap.md:324-325)
+            v, detail["decode_b256_ctx512"] = decode_point(args.shape, 256, 512)
+            points["decode_b256_ctx512"] = round(v, 1)
+            if "vs_reference" in out:
+                out["vs_reference"]["decode_b256_short_contexts"] = round(v / REF_DECODE_B256_SHORT, 2)
             # the same configuration in the reference's own fast precision and in true 32-bit
             for dtn in ("f16", "f32"):
                 v, detail[f"{dtn}_decode_b8"] = decode_point(args.shape, args.batch, ctx, dtn)

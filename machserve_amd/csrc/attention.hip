@@ -1350,8 +1350,10 @@ using namespace ms;
 #define MS_CAT2(a, b) a##b
 #define MS_CAT(a, b) MS_CAT2(a, b)
 
-// Attention of a mixed batch.  `work` lists (request index, first flat row) for every block
-// of 64 flat rows; see the file comment.  window = 0 means all keys.  max_key_groups = 0 lets the
+// Attention of a mixed batch.  `work` lists (request index, first flat row) for every ROWS_PER_BLOCK
+// flat rows of a request (ms_attention_rows_per_block_nd<N>() tells the caller the number; the general kernel
+// takes an item as SUB_BLOCKS blocks of 64 rows, the kernel of 32-row tiles as one block); an item of
+// request -1 only fills a list up and is skipped; see the file comment.  window = 0 means all keys.  max_key_groups = 0 lets the
 // launcher choose how many key groups share a block (1, 2 or 4) from the width of the block tables;
 // a positive value asks for that many (as far as this tile has them).  nsplit > 1 cuts every block's
 // keys over that many blocks (few blocks of rows over long contexts would leave most of the chip idle
