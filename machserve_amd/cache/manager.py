@@ -24,7 +24,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Tuple
 
-from . import CacheCore, CacheError, OutOfPages
+from . import CacheCore, CacheError
 
 
 def group_name(window: Optional[int]) -> str:

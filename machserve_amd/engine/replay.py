@@ -21,7 +21,6 @@ import json
 import os
 import sys
 
-import numpy as np
 
 from .loading import load_model
 from .step import StepEntry

@@ -5,7 +5,7 @@ may name a layer twice.  Only the rows whose logits are wanted reach the head
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional
+from typing import List, Optional
 
 import torch
 

@@ -7,7 +7,7 @@ draw per sampled row, greedy rows included (``crates/mach-model/src/sampling.rs:
 1026-1030``)."""
 from __future__ import annotations
 
-from typing import Dict, List, Sequence
+from typing import Dict, Sequence
 
 import numpy as np
 import torch

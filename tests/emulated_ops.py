@@ -6,9 +6,6 @@ the GPU tests.  Nothing in the package imports this file.
 """
 from __future__ import annotations
 
-import math
-
-import numpy as np
 import torch
 
 MASK64 = (1 << 64) - 1

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from emulated_ops import EmulatedOps
-from tiny_configs import CONFIGS, TINY_A, TINY_B, TINY_C, make_model_dir
+from tiny_configs import TINY_A, TINY_B, TINY_C, make_model_dir
 
 
 def test_qwen2_config_reads_its_keys():

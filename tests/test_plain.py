@@ -9,7 +9,7 @@ import torch
 import torch.nn.functional as F
 
 from plain import qwen2_plain as P
-from tiny_configs import CONFIGS, make_model_dir, random_prompt, read_for_plain
+from tiny_configs import make_model_dir, random_prompt, read_for_plain
 
 
 def rnd(*shape, seed=0, dtype=torch.float64):
