@@ -406,6 +406,40 @@ def main() -> int:
         torch.cuda.empty_cache()
         return out
 
+    def mixed_load_point(shape, n_requests=256, running=64, budget=2048, arrive=4):
+        """The whole engine under a load as a server has it: requests of 64 to 640 prompt tokens and 32 to 256 new tokens,
+        ``arrive`` of them a step, at most ``running`` at a time, prompts fed in portions beside the decoding requests
+        under a budget of ``budget`` tokens a step, to the end.  Tokens a second, prompt and generated together, from
+        the first arrival to the last token on the host; the sizes that steps are filled up to were captured before
+        (``Engine.warm_up``), the decode steps' shapes are captured as they come."""
+        import random
+        cfg, tensors, _ = model_of(shape)
+        lm = load_model(config=cfg, tensors=tensors, dtype=DT[args.dtype], page_size=args.page_size, max_tokens=running * 1024,
+                        max_requests=running)
+        eng = Engine(lm, max_batch_tokens=budget, max_running=running)
+        eng.warm_up(range(64, budget + 1, 64))
+        rng = random.Random(0)
+        reqs = [([rng.randrange(cfg.vocab_size) for _ in range(rng.randint(64, 640))], rng.randint(32, 256)) for _ in range(n_requests)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        added = produced = steps = 0
+        while added < n_requests or eng.has_work():
+            for p, m in reqs[added:added + arrive]:
+                eng.add(p, m, SamplingParams())
+            added = min(n_requests, added + arrive)
+            em, _ = eng.step_pipelined()
+            produced += len(em)
+            steps += 1
+        torch.cuda.synchronize()
+        dt_s = time.perf_counter() - t0
+        prompt_tokens = sum(len(p) for p, _ in reqs)
+        assert produced == sum(m for _, m in reqs), "every request ran to its last token"
+        del eng, lm
+        torch.cuda.empty_cache()
+        return (prompt_tokens + produced) / dt_s, {"s": round(dt_s, 3), "requests": n_requests, "prompt_tokens": prompt_tokens,
+                                                   "generated": produced, "generated_tok_s": round(produced / dt_s, 1),
+                                                   "steps": steps, "ms_per_step": round(dt_s / steps * 1e3, 3)}
+
     shape_name = SHAPES[args.shape][0]
     cfg, _, full_layers = model_of(args.shape)
     ctx = args.context
@@ -483,6 +517,9 @@ def main() -> int:
             # the first token of a prompt of a length not seen before (the reference quotes 512 tokens, docs/roadmap.md:260-261)
             for n, (v, d) in first_token_points(args.shape, (128, 500, 512)).items():
                 points[f"first_token_{n}"], detail[f"first_token_{n}"] = round(v, 1), d
+            # the engine whole: arrivals, portions of prompts beside decoding requests, ends
+            v, detail["mixed_load_256_requests"] = mixed_load_point(args.shape)
+            points["mixed_load_256_requests"] = round(v, 1)
             # many requests at short contexts, as the reference's own sweep over the batch has them (docs/roadmap.md:324-325)
             v, detail["decode_b256_ctx512"] = decode_point(args.shape, 256, 512)
             points["decode_b256_ctx512"] = round(v, 1)

@@ -76,13 +76,14 @@ class StepFunction:
     # A larger step keeps the device busy about as long as the host needs to launch it (2,048 rows of the 0.5B sizes:
     # 4.06 ms launched, 3.95 ms replayed).
     CAPTURE_MAX_ROWS = 2048
-    # A capture costs 7 ms; a replayed step is 0.9 ms shorter than a launched one with a few requests, 0.3 to
-    # 0.4 ms with 64 requests or a few hundred rows.  While requests end one by one most shapes last a few
-    # steps, so a shape is captured only when it has come this often before: at worst that doubles what the
-    # better choice would have cost.
+    # A capture costs 7 ms; a replayed step is about 1 ms shorter than a launched one (a decode step of the 0.5B sizes:
+    # 1.03 against 2.17 ms).  A step in a shape of its own is captured only when that shape has come often (most never come
+    # again); the sizes that steps are filled up to, and the decode steps' few sizes, keep coming in a server, so they are
+    # captured the second time they are seen.  (256 and 1,024 requests of 64 to 640 prompt tokens and 32 to 256 new
+    # ones, four arriving a step, 64 running: 1.28 -> 1.23 s and 4.50 -> 4.39 s against thresholds of 8 and 4.)
     CAPTURE_AFTER = 16        # a step other than plain decoding, in its own shape
-    FILLED_CAPTURE_AFTER = 4  # ... filled up to a size that many steps share: such a size keeps coming
-    DECODE_CAPTURE_AFTER = 8  # a decode step
+    FILLED_CAPTURE_AFTER = 2  # ... filled up to a size that many steps share
+    DECODE_CAPTURE_AFTER = 1  # a decode step
 
     def __init__(self, model, cache: CacheManager, rt, attention_rows_per_block: int = 64, use_graphs: bool = True):
         self.model, self.cache, self.rt = model, cache, rt
