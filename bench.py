@@ -136,15 +136,16 @@ def by_name(rows, n):
     return sorted(((nm, c, t / c, t) for nm, (c, t) in names.items()), key=lambda r: -r[3])
 
 
-def write_summary(path, title, command, kinds, names, n_steps):
-    """A short text summary of one traced run: what it ran, the kinds of kernels, the kernels by name."""
+def write_summary(path, title, command, kinds, names, n_steps, work_of=None):
+    """A short text summary of one traced run: what it ran, the kinds of kernels, the kernels by name (with the rate of
+    those whose bytes or operations ``work_of`` knows: name -> (amount over the listed calls, unit))."""
     lines = [f"# {title}", "", "Command (on an MI355X, from the repository root; the summary is written by the command itself):", "",
              f"    {command}", "",
              "The work is run a second time under `rocprofv3 --kernel-trace`; the dispatches of the last steps are matched, in order, with",
              "the operations one step issues.  Times are the kernels' own durations as the profiler reports them.", "",
              "| kind of kernel | launches a step | us a step | rate | of the published peak | of what the box gives |", "|---|---|---|---|---|---|"]
     for kind, r in kinds.items():
-        if kind == "all" or not isinstance(r, dict):
+        if kind == "all" or kind.startswith("_") or not isinstance(r, dict):
             continue
         rate = f"{r['rate']} {r['unit']}" if "rate" in r else ""
         lines.append(f"| {kind} | {r['launches']} | {r['us']} | {rate} | {r.get('frac', '')} | {r.get('frac_of_measured', '')} |")
@@ -152,9 +153,13 @@ def write_summary(path, title, command, kinds, names, n_steps):
         a = kinds["all"]
         lines += ["", f"All: {a['launches']} launches a step, {a['us_in_kernels']} us inside kernels, {a['us_first_to_last']} us from the first "
                       f"kernel's start to the last one's end under the profiler (which slows the replay of a captured step)."]
-    lines += ["", f"| kernel | calls in {n_steps} step{'s' if n_steps != 1 else ''} | mean us | total us |", "|---|---|---|---|"]
+    lines += ["", f"| kernel | calls in {n_steps} step{'s' if n_steps != 1 else ''} | mean us | total us | rate |", "|---|---|---|---|---|"]
     for nm, c, mean, total in names[:14]:
-        lines.append(f"| `{nm[:110]}` | {c} | {mean:.2f} | {total:.1f} |")
+        rate = ""
+        if work_of and nm in work_of and total > 0:
+            amount, unit = work_of[nm]
+            rate = f"{amount / (total * 1e-6) / (1e9 if unit == 'GB/s' else 1e12):.0f} {unit}"
+        lines.append(f"| `{nm[:110]}` | {c} | {mean:.2f} | {total:.1f} | {rate} |")
     with open(path, "w") as f:
         f.write("\n".join(lines) + "\n")
 
@@ -169,9 +174,19 @@ def account(calls, rows, n_steps, peak_of, measured_of, extra):
         return {"error": f"{len(rows)} traced dispatches for {n_steps} steps of {L} launches"}
     rows = rows[-n_steps * L:]
     kinds = {}
-    for i, (start, end, _) in enumerate(rows):
-        k = kinds.setdefault(per_launch[i % L][0], {"launches": 0, "us": 0.0})
+    # what the dispatches of a kernel name moved or computed, where an operation is one launch (a product) or its
+    # work is given for the kind (attention)
+    work_of, kind_us = {}, {}
+    for i, (start, end, name) in enumerate(rows):
+        call = per_launch[i % L]
+        k = kinds.setdefault(call[0], {"launches": 0, "us": 0.0})
         k["us"] += (end - start) / 1e3 / n_steps
+        unit = peak_of.get(call[0])
+        if unit and call[1] == 1 and call[0] not in extra:
+            w = work_of.setdefault(name, [0.0, unit])
+            w[0] += call[2] if unit == "GB/s" else call[3]
+        elif unit and call[0] in extra:
+            kind_us.setdefault(call[0], {}).setdefault(name, [0.0])[0] += (end - start) / 1e3
     for c in calls:
         k = kinds.setdefault(c[0], {"launches": 0, "us": 0.0})
         k["launches"] += c[1]
@@ -196,6 +211,12 @@ def account(calls, rows, n_steps, peak_of, measured_of, extra):
     busy = sum(k["us"] for k in kinds.values())
     out["all"] = {"launches": L, "us_in_kernels": round(busy, 2), "us_first_to_last": round(span, 2),
                   "us_between_kernels": round(span - busy, 2)}
+    for kind, per_name in kind_us.items():
+        unit = peak_of[kind]
+        amount = (extra[kind][0] if unit == "GB/s" else extra[kind][1]) * n_steps
+        main = max(per_name, key=lambda n: per_name[n][0])  # the kind's work is its main kernel's (a merge moves next to nothing)
+        work_of[main] = [amount, unit]
+    out["_work_of"] = {k: (v[0], "GB/s" if v[1] == "GB/s" else "TFLOP/s") for k, v in work_of.items()}
     return out
 
 
@@ -604,7 +625,9 @@ def kernels_by_kind(args, cfg, dt, peaks, ctx, prefill_tokens):
                 name += ("" if args.shape == "0.5b" else "_" + args.shape) + ("" if args.dtype == "bf16" else "_" + args.dtype)
                 command = "python bench.py " + " ".join(a for a in sys.argv[1:])
                 write_summary(os.path.join(args.profile_out, name + ".md"), f"{title} ({shape} shape, {args.dtype}, random weights)", command,
-                              out[kind], by_name(rows, n_steps * out[kind]["all"]["launches"]), n_steps)
+                              out[kind], by_name(rows, n_steps * out[kind]["all"]["launches"]), n_steps, out[kind].get("_work_of"))
+            if isinstance(out[kind], dict):
+                out[kind].pop("_work_of", None)  # for the summaries only: the record keeps to the kinds
     return out
 
 
