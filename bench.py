@@ -78,8 +78,10 @@ def prefill_flops(cfg, T):
 PRODUCT_OPS = {  # name -> positions of (rows operand, weight) among the arguments
     "linear_split": (0, 1), "linear": (0, 1), "linear_residual": (0, 1), "linear_residual_prenorm": (0, 1),
     "linear_swiglu": (0, 1), "linear_swiglu_scaled": (0, 3), "linear_split_normed": (0, 4), "linear_swiglu_normed": (0, 4),
+    "linear_qkv_rope": (0, 1),
 }
 OTHER_OPS = {"embed": "embedding", "rmsnorm": "norm", "add_partials": "norm", "rope_kv_write": "rotation and cache write",
+             "rope_table": "rotation and cache write",
              "paged_attention": "attention", "decode_attention_fused": "attention", "decode_attention": "attention",
              "sample": "sampling", "sample_packed": "sampling", "top_logprobs": "sampling", "logit_edit": "sampling"}
 

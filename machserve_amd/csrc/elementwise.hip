@@ -194,6 +194,20 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(RopeArgs a) {
     }
 }
 
+// cs[t, j] = (cos, sin) of positions[t] * inv_freq[j]: the angles of a step's rows, once for every layer that rotates
+// by these frequencies, for the product that rotates in its own epilogue (it cannot share a row's sines among its
+// lanes as the kernels here do).  The same expression as above: the same values.
+__global__ __launch_bounds__(256) void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                                         float* __restrict__ cs, int n, int half) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int t = i / half, j = i - t * half;
+    float c, s;
+    sincosf((float)positions[t] * inv_freq[j], &s, &c);
+    cs[2 * (size_t)i] = c;
+    cs[2 * (size_t)i + 1] = s;
+}
+
 // The same in quads: head sizes that are multiples of 8, rows whose stride is a multiple of 4 and
 // 16-byte aligned buffers.  A thread takes four neighbouring pairs (j .. j + 3, j + half .. + 3) of one
 // head: two 16-byte loads per partial sum, all asked for before the first is used, and two 8-byte
@@ -273,6 +287,15 @@ using namespace ms;
 constexpr int MAX_ROW_FLOATS = 15000;
 extern "C" int ms_max_norm_width() { return MAX_ROW_FLOATS; }
 extern "C" int ms_max_rope_row() { return MAX_ROW_FLOATS; }
+
+// cs [T, half, 2] (float) = cosine and sine of positions[t] * inv_freq[j].
+extern "C" int ms_rope_table(const int* positions, const float* inv_freq, float* cs, int T, int half, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && half > 0 && positions && inv_freq && cs, "rope table: T=%d, %d frequencies", T, half);
+    MS_REQUIRE((long)T * half < 2147483647L, "rope table: %d rows of %d frequencies", T, half);
+    const int n = T * half;
+    hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, stream, positions, inv_freq, cs, n, half);
+    return check_launch("rope_table");
+}
 
 extern "C" int ms_embed(const int* tokens, const void* table, float* x, int T, int d, float scale, hipStream_t stream) {
     MS_REQUIRE(T > 0 && d > 0, "embed: empty problem T=%d d=%d", T, d);

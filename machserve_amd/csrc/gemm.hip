@@ -30,7 +30,7 @@ constexpr int EPC = 4;
 constexpr int KPAD = 8;  // rows of 160 bytes (BK 32)
 #endif
 
-enum EpiKind { EPI_STORE_F32 = 0, EPI_STORE_ELEM = 1, EPI_RESIDUAL = 2, EPI_SWIGLU = 3 };
+enum EpiKind { EPI_STORE_F32 = 0, EPI_STORE_ELEM = 1, EPI_RESIDUAL = 2, EPI_SWIGLU = 3, EPI_QKV_ROPE = 4 };
 
 struct EpiArgs {
     void* out;          // [M, ldo]
@@ -45,6 +45,14 @@ struct EpiArgs {
     int ss_parts;
     float ss_eps;
     int act;            // SWIGLU: the activation on the gate (GateActivation)
+    // QKV_ROPE: the columns are H query heads, KV key heads and KV value heads of the tile's width; bias added, queries
+    // and keys rotated by the rows' angles (pairs (j, j + half a head)), queries to `out` [M, H * hd], keys and values
+    // into their pages
+    const float* rope_cs;  // [M, hd / 2, 2]: cosine and sine of each row's angles
+    const int* slot_map;   // [M]: page * ps + offset of each row's key and value, or negative: not written
+    elem_t* kpool;         // [pages, KV, ps, hd]
+    elem_t* vpool;         // [pages, KV, hd, ps]
+    int H, KV, ps;
 };
 
 template <int BM, int BN, int WM, int WN, int BK, int EPI, int STAGES = 2, bool SCALED = false>
@@ -327,6 +335,55 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(const elem_t* __rest
                     }
                 }
             }
+        } else if constexpr (EPI == EPI_QKV_ROPE) {
+            // The tile's columns are one head (the launcher sees to it), and a wave holds all of them: lane (r16, grp)
+            // has columns r16 + 16 j of rows grp * 4 + e, so both elements of a pair (j, j + TN / 2) are its own.
+            static_assert(WN == 1 && TN % 2 == 0, "a wave holds whole heads");
+            constexpr int HT = TN / 2, hd = BN, half = BN / 2;
+            const int head = n0 / hd;
+            const int kind = head < ep.H ? 0 : (head < ep.H + ep.KV ? 1 : 2);  // query, key or value head
+            float bias_j[TN];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) bias_j[j] = ep.bias ? ep.bias[n0 + j * 16 + r16] : 0.f;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int row = row_base + i * 16 + e;
+                    if (row >= M) continue;
+                    float x[TN];
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) x[j] = bias_j[j] + acc[i][j][e];
+                    if (kind < 2) {
+                        const float* cs = ep.rope_cs + (size_t)row * (2 * half);
+#pragma unroll
+                        for (int j = 0; j < HT; ++j) {
+                            const float c = cs[2 * (j * 16 + r16)], sn = cs[2 * (j * 16 + r16) + 1];
+                            const float x0 = x[j], x1 = x[j + HT];
+                            x[j] = x0 * c - x1 * sn;
+                            x[j + HT] = x0 * sn + x1 * c;
+                        }
+                    }
+                    if (kind == 0) {
+                        elem_t* o = reinterpret_cast<elem_t*>(ep.out) + ((size_t)row * ep.H + head) * hd + r16;
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) o[j * 16] = from_f32<elem_t>(x[j]);
+                    } else {
+                        const int slot = ep.slot_map[row];
+                        if (slot < 0) continue;
+                        const int page = slot / ep.ps, off = slot - page * ep.ps;
+                        if (kind == 1) {
+                            elem_t* o = ep.kpool + (((size_t)page * ep.KV + (head - ep.H)) * ep.ps + off) * hd + r16;
+#pragma unroll
+                            for (int j = 0; j < TN; ++j) o[j * 16] = from_f32<elem_t>(x[j]);
+                        } else {
+                            elem_t* o = ep.vpool + (((size_t)page * ep.KV + (head - ep.H - ep.KV)) * hd + r16) * ep.ps + off;
+#pragma unroll
+                            for (int j = 0; j < TN; ++j) o[(size_t)(j * 16) * ep.ps] = from_f32<elem_t>(x[j]);
+                        }
+                    }
+                }
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
@@ -557,6 +614,64 @@ extern "C" int ms_linear_swiglu_scaled(const void* a, const float* row_ss, int s
 #else
     (void)a; (void)row_ss; (void)ss_parts; (void)eps; (void)w; (void)out; (void)M; (void)I; (void)K; (void)act; (void)stream;
     MS_REQUIRE(false, "gated product with row factors: built for bfloat16 only");
+#endif
+}
+
+// Whether ms_linear_qkv_rope takes this shape: two-byte elements, more rows than the few-rows kernels take, heads of
+// 64 or 128 (a tile's columns are one head, so that both elements of a rotated pair lie in one lane), K in whole chunks.
+extern "C" int ms_qkv_rope_takes(int M, int H, int KV, int hd, int K) {
+#ifdef MS_ELEM_HALF
+    return M > 64 && H > 0 && KV > 0 && (hd == 64 || hd == 128) && K % 8 == 0 && K >= 128;
+#else
+    (void)M; (void)H; (void)KV; (void)hd; (void)K;
+    return 0;
+#endif
+}
+
+// The q/k/v projection of a step of many rows with what follows it in its epilogue: w [(H + 2 KV) * hd, K] holds the
+// query heads, the key heads and the value heads; bias [(H + 2 KV) * hd] or null is added, queries and keys are rotated
+// by the rows' angles (rope_cs [M, hd / 2, 2], cosine and sine, as ms_rope_table makes them), queries go to q_out
+// [M, H * hd], keys and values into their pages at slot_map[row] (a negative slot is not written).  The same values as
+// ms_linear (32-bit output) followed by ms_rope_kv_write, without the 32-bit sums' trip through memory and without
+// the second launch.
+extern "C" int ms_linear_qkv_rope(const void* a, const void* w, const float* bias, const float* rope_cs, const int* slot_map,
+                                  void* q_out, void* kpool, void* vpool, int M, int H, int KV, int hd, int ps, int K,
+                                  hipStream_t stream) {
+#ifdef MS_ELEM_HALF
+    MS_REQUIRE(ms_qkv_rope_takes(M, H, KV, hd, K), "q/k/v product with rotation: M=%d, %d + 2 x %d heads of %d, K=%d is not taken", M, H, KV, hd, K);
+    MS_REQUIRE(rope_cs && slot_map && q_out && kpool && vpool && ps > 0, "q/k/v product with rotation: a buffer is missing");
+    MS_REQUIRE((reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0, "gemm: operands must be 16-byte aligned");
+    const int N = (H + 2 * KV) * hd;
+    EpiArgs ep{q_out, bias, H * hd, N, K, 0, nullptr, 0, 0.f, 0, rope_cs, slot_map, (elem_t*)kpool, (elem_t*)vpool, H, KV, ps};
+    const long round_blocks = 2L * compute_units();
+#define MS_QKV(BM_, BN_)                                                                                                 \
+    do {                                                                                                                 \
+        const long nb = (long)ceil_div(M, BM_) * (N / BN_);                                                              \
+        hipLaunchKernelGGL((gemm_kernel<BM_, BN_, 4, 1, 64, EPI_QKV_ROPE>), dim3((unsigned)nb, 1), dim3(256), 0, stream, \
+                           (const elem_t*)a, (const elem_t*)w, M, N, K, ep);                                             \
+        return check_launch("gemm q/k/v with rotation " #BM_ "x" #BN_);                                                  \
+    } while (0)
+    // rows in tiles of 128 where that still gives the chip a round of blocks, else of 64
+    const bool tall = (long)ceil_div(M, 128) * (N / hd) >= round_blocks * 300 / 512;
+    if (hd == 64) {
+        if (tall) MS_QKV(128, 64);
+        if (K % 64 == 0 && K >= 256) {
+            // three LDS buffers in turn (two K steps in flight, three blocks a CU): 0.5B, 2,048 rows, 17.0 -> 16.4 us; tiles of
+            // 128x64 take 20.3 (288 blocks, barely one a CU, each step a trip to the L2)
+            const long nb = (long)ceil_div(M, 64) * (N / 64);
+            hipLaunchKernelGGL((gemm_kernel<64, 64, 4, 1, 64, EPI_QKV_ROPE, 3>), dim3((unsigned)nb, 1), dim3(256), 0, stream,
+                               (const elem_t*)a, (const elem_t*)w, M, N, K, ep);
+            return check_launch("gemm q/k/v with rotation 64x64 deep");
+        }
+        MS_QKV(64, 64);
+    }
+    if (tall) MS_QKV(128, 128);
+    MS_QKV(64, 128);
+#undef MS_QKV
+#else
+    (void)a; (void)w; (void)bias; (void)rope_cs; (void)slot_map; (void)q_out; (void)kpool; (void)vpool; (void)M; (void)H; (void)KV;
+    (void)hd; (void)ps; (void)K; (void)stream;
+    MS_REQUIRE(false, "q/k/v product with rotation: built for two-byte elements only");
 #endif
 }
 

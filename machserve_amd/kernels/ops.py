@@ -181,6 +181,42 @@ class HipOps:
             _ptr(kpool), _ptr(vpool), _c_int(T), _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), self._stream()))
         return q
 
+    def rope_table(self, positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+        """Float32 ``[T, hd / 2, 2]``: cosine and sine of ``positions[t] * inv_freq[j]``, as the rotation kernels
+        compute them; for :meth:`linear_qkv_rope`."""
+        T, half = positions.numel(), inv_freq.numel()
+        self._want(positions, torch.int32, "rope table positions", T)
+        self._want(inv_freq, torch.float32, "rope table inv_freq", half)
+        cs = torch.empty((T, half, 2), dtype=torch.float32, device=inv_freq.device)
+        self._check(self._core, self._core.ms_rope_table(_ptr(positions), _ptr(inv_freq), _ptr(cs), _c_int(T), _c_int(half), self._stream()))
+        return cs
+
+    def qkv_rope_takes(self, M: int, H: int, KV: int, hd: int, K: int) -> bool:
+        """Whether :meth:`linear_qkv_rope` takes this shape (else: :meth:`linear_split` and :meth:`rope_kv_write`)."""
+        return bool(self._plan("ms_qkv_rope_takes", M, H, KV, hd, K))
+
+    def linear_qkv_rope(self, a: torch.Tensor, w_qkv: torch.Tensor, bias: Optional[torch.Tensor], rope_cs: torch.Tensor,
+                        slot_map: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, H: int, KV: int, hd: int,
+                        page_size: int) -> torch.Tensor:
+        """The q/k/v projection ``a @ w_qkv.T + bias`` of a step of many rows with the rotation of queries and keys
+        (by ``rope_cs`` of :meth:`rope_table`) and the write of keys and values into their pages in the product's own
+        epilogue.  Returns q ``[T, H * hd]`` in the element type."""
+        M, N, K = self._mm_operands(a, w_qkv, "linear_qkv_rope")
+        if N != (H + 2 * KV) * hd:
+            raise KernelError(f"linear_qkv_rope: weight of {N} rows for {H} + 2 x {KV} heads of {hd}")
+        if bias is not None:
+            self._want(bias, torch.float32, "linear_qkv_rope bias", N)
+        self._want(rope_cs, torch.float32, "linear_qkv_rope angles", M, hd // 2, 2)
+        self._want(slot_map, torch.int32, "linear_qkv_rope slot_map", M)
+        pages = kpool.shape[0]
+        self._want(kpool, self.dtype, "key pool", pages, KV, page_size, hd)
+        self._want(vpool, self.dtype, "value pool", pages, KV, hd, page_size)
+        q = torch.empty((M, H * hd), dtype=self.dtype, device=a.device)
+        self._check(self._core, self._core.ms_linear_qkv_rope(
+            _ptr(a), _ptr(w_qkv), _ptr(bias), _ptr(rope_cs), _ptr(slot_map), _ptr(q), _ptr(kpool), _ptr(vpool), _c_int(M), _c_int(H),
+            _c_int(KV), _c_int(hd), _c_int(page_size), _c_int(K), self._stream()))
+        return q
+
     # ------------------------------------------------------------------ matrix products
     def _mm_operands(self, a: torch.Tensor, w: torch.Tensor, what: str):
         self._want(a, self.dtype, f"{what} input")

@@ -79,6 +79,23 @@ class Attention(Mixer):
     def forward(self, h, stream, ctx):
         s, ops = self.spec, self.rt.ops
         view = ctx.groups[self.group]
+        g = self.attention_rows_per_token()
+        # A step of many rows: the q/k/v product rotates and writes the cache in its own epilogue, where the kernels have
+        # that form (the rows' angles come from a table that the step's layers share).
+        takes = getattr(ops, "qkv_rope_takes", None)
+        if (takes is not None and self.writes_cache and self.position is not None and not (ctx.decode_only and g <= ops.DECODE_MAX_GROUP)
+                and takes(ctx.n_rows, s.heads, s.kv_heads, s.head_dim, self.w_qkv.shape[1])):
+            inv_freq = self.position.rotary_inv_freq()
+            if inv_freq is not None:
+                key = ("rope table", inv_freq.data_ptr())
+                if key not in ctx.shared:
+                    ctx.shared[key] = ops.rope_table(ctx.position_axis(0), inv_freq)
+                q = ops.linear_qkv_rope(h.tensor() if isinstance(h, PendingNorm) else h, self.w_qkv, self.b_qkv, ctx.shared[key],
+                                        view.slot_map, self.kpool, self.vpool, s.heads, s.kv_heads, s.head_dim, view.page_size)
+                o = ops.paged_attention(q, self.kpool, self.vpool, view.block_table, ctx.seq_q_start, ctx.seq_q_len, ctx.seq_pos0,
+                                        ctx.attention_work[g], s.heads, s.kv_heads, s.head_dim, view.page_size, s.window, self.scale)
+                stream.add_linear(o, self.w_o)
+                return
         # [P, T, nq (+ 2 nkv)] partial sums, bias not yet added
         qkv = h.linear_split(self.w_qkv) if isinstance(h, PendingNorm) else ops.linear_split(h, self.w_qkv)
         inv_freq = self.position.rotary_inv_freq() if self.position is not None else None
@@ -93,7 +110,6 @@ class Attention(Mixer):
             q = qkv[0, :, :self.nq].unflatten(1, (s.heads, s.head_dim))
             k = qkv[0, :, self.nq:self.nq + self.nkv].unflatten(1, (s.kv_heads, s.head_dim)) if self.writes_cache else None
             self.position.apply(q, k, ctx)
-        g = self.attention_rows_per_token()
         decode = ctx.decode_only and g <= ops.DECODE_MAX_GROUP
         # the fused decode kernel rotates by the row's place in the cache: only where that is its position
         if decode and self.writes_cache and (self.position is None or (inv_freq is not None and ctx.positions_sequential)):

@@ -91,6 +91,8 @@ class StepContext:
     # True: every row's position is, on every axis, its index in its request's cache (``seq_pos0`` onwards), so a
     # kernel may take positions from there; False: the caller gave positions of its own for some rows
     positions_sequential: bool = True
+    # what parts have worked out from this step's rows and share between layers (a table of the rows' rotation angles)
+    shared: Dict[object, object] = field(default_factory=dict)
 
     def position_axis(self, axis: int = 0) -> torch.Tensor:
         """``[T]`` positions along one axis, contiguous."""

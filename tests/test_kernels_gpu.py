@@ -759,3 +759,53 @@ def test_logit_edit():
     ref = torch.zeros(2, 10)
     ref[0, 3], ref[1, 0], ref[1, 9] = 1.5, -2.0, 4.0
     assert torch.equal(x.cpu(), ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,H,KV,hd,K,ps", [(100, 3, 1, 64, 136, 16), (300, 14, 2, 64, 896, 64), (130, 4, 4, 128, 264, 32),
+                                            (2048, 14, 2, 64, 896, 64), (1100, 12, 2, 128, 200, 64)])
+def test_qkv_product_that_rotates_and_writes_the_cache(dtype, M, H, KV, hd, K, ps):
+    """The q/k/v projection of a step of many rows with bias, rotation and cache write in its epilogue: the same queries
+    and the same pages as the plain product (32-bit sums) followed by the rotation kernel, and as the plain formulas
+    (crates/mach-model/src/batched.rs:3566-3679); rows with a negative slot leave the pages alone; positions that are
+    not the rows' indices."""
+    ops = ops_for(dtype)
+    assert ops.qkv_rope_takes(M, H, KV, hd, K) and not ops.qkv_rope_takes(64, H, KV, hd, K) and not ops.qkv_rope_takes(M, H, KV, 80, K)
+    N = (H + 2 * KV) * hd
+    a, w, bias = rnd((M, K), dtype, 1), rnd((N, K), dtype, 2, K ** -0.5), rnd((N,), torch.float32, 3)
+    gen = torch.Generator().manual_seed(4)
+    positions = torch.randint(0, 5000, (M,), generator=gen, dtype=torch.int32)
+    pages = -(-M // ps) + 2
+    slots = torch.randperm(pages * ps, generator=gen)[:M].to(torch.int32)
+    slots[5] = -1                                    # a row that writes nothing
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(hd // 2, dtype=torch.float32) * 2 / hd)))
+    dev = lambda t: t.to(DEV)
+    kp0, vp0 = rnd((pages, KV, ps, hd), dtype, 5), rnd((pages, KV, hd, ps), dtype, 6)
+    # the two kernels it replaces
+    kp1, vp1 = dev(kp0).clone(), dev(vp0).clone()
+    sums = ops.linear(dev(a), dev(w), None, out_f32=True)
+    q1 = ops.rope_kv_write(sums, dev(bias), dev(positions), dev(inv_freq), dev(slots), kp1, vp1, H, KV, hd, ps)
+    # the one kernel
+    kp2, vp2 = dev(kp0).clone(), dev(vp0).clone()
+    table = ops.rope_table(dev(positions), dev(inv_freq))
+    ang = positions.double()[:, None] * inv_freq.double()[None, :]
+    assert (table[..., 0].cpu().double() - torch.cos(ang)).abs().max() < 1e-3 and (table[..., 1].cpu().double() - torch.sin(ang)).abs().max() < 1e-3
+    q2 = ops.linear_qkv_rope(dev(a), dev(w), dev(bias), table, dev(slots), kp2, vp2, H, KV, hd, ps)
+    assert_close(q2, q1.double(), dtype, "queries against the two kernels")
+    assert_close(kp2, kp1.double(), dtype, "key pages against the two kernels")
+    assert_close(vp2, vp1.double(), dtype, "value pages against the two kernels")
+    # the plain formulas
+    x = P.linear(a.double(), w.double(), bias.double())
+    qr = P.rope(x[:, :H * hd].view(M, H, hd).float(), positions.long(), 10000.0).reshape(M, H * hd)
+    assert_close(q2, qr.double(), dtype, "queries against the plain rotation")
+    kr = P.rope(x[:, H * hd:(H + KV) * hd].view(M, KV, hd).float(), positions.long(), 10000.0)
+    t = 17
+    page, off = int(slots[t]) // ps, int(slots[t]) % ps
+    assert_close(kp2[page, :, off, :], kr[t].double(), dtype, "a key in its page")
+    assert_close(vp2[page, :, :, off], x[t, (H + KV) * hd:].view(KV, hd), dtype, "a value in its page")
+    # what no row writes stays as it was (the row with the negative slot, and the slots nobody has)
+    written = torch.zeros(pages * ps, dtype=torch.bool)
+    written[slots[slots >= 0].long()] = True
+    keep = (~written).view(pages, ps)
+    assert torch.equal(kp2.cpu().permute(0, 2, 1, 3)[keep], kp0.permute(0, 2, 1, 3)[keep])
+    assert torch.equal(vp2.cpu().permute(0, 3, 1, 2)[keep], vp0.permute(0, 3, 1, 2)[keep])
