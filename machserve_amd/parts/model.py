@@ -142,6 +142,10 @@ class DecoderModel:
     def forward(self, ctx: StepContext) -> Optional[torch.Tensor]:
         """Run the step's rows through the layers in ``order``; float32 logits ``[W, vocab]`` of
         the wanted rows, or None when none is wanted."""
+        # What the layers of one pass share (a table of the rows' rotation angles) is made anew in every pass: a context
+        # is run once to load everything and once more under capture, and what the first run left would be missing
+        # from the captured graph, which would then rotate every later step by the first step's positions.
+        ctx.shared.clear()
         stream = ResidualStream(self.embedding.forward(ctx.tokens), self.rt.ops)
         watch = self.observer
         if watch is not None:

@@ -223,6 +223,40 @@ def test_steps_of_any_mix_run_from_graphs_of_shared_sizes(tmp_path, which, dtype
     assert all(g.pool.available() == g.pool.num_pages for g in lm.cache.groups.values())
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("head_dim,heads,kv", [(64, 6, 2), (128, 32, 2)])
+def test_prompts_of_one_size_from_one_graph_at_head_sizes_64_and_128(tmp_path, dtype, head_dim, heads, kv):
+    """At head sizes 64 and 128 the q/k/v product of a step of many rows rotates by a table of the rows' angles that the
+    step's layers share.  Prompts of several lengths that are filled up to one size run from one captured graph: the
+    table is made inside the graph, from the positions of the step at hand (captured from the first prompt's, every
+    later prompt's rows beyond the first one's length would be rotated by the angles of the rows that filled the first
+    step up).  Every position's logits against the plain model."""
+    from machserve_amd.engine import StepEntry, load_model
+    from machserve_amd.weights import write_random_model
+    raw = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_size": 200, "num_hidden_layers": 2,
+           "num_attention_heads": heads, "num_key_value_heads": kv, "head_dim": head_dim, "intermediate_size": 160, "vocab_size": 512,
+           "max_position_embeddings": 512, "rms_norm_eps": 1e-5, "rope_theta": 10000.0, "tie_word_embeddings": False,
+           "hidden_act": "silu", "attention_bias": True}
+    d = write_random_model(raw, 11, str(tmp_path / "m"))
+    sharpen_attention(d, 3.0)                        # so that a wrong angle shows in the logits
+    w, sizes = read_for_plain(d)
+    ww = _stored(w, dtype)
+    lm = load_model(d, dtype=dtype, device=DEV, page_size=64, num_pages=12, max_requests=2)
+    assert lm.rt.ops.qkv_rope_takes(128, heads, kv, head_dim, 200)
+    bound = 3e-2 if dtype == torch.bfloat16 else 3e-2 / 8
+    lm.step.FILLED_CAPTURE_AFTER = 0
+    for n in (68, 101, 76, 66, 127, 120):            # all of them filled up to 128 rows
+        prompt = random_prompt(n, 512, 300 + n)
+        ref = P.forward(ww, sizes, prompt)
+        slot = lm.cache.admit()
+        got = lm.step([StepEntry(slot, prompt, list(range(n)))]).float().cpu()
+        lm.cache.release(slot)
+        err = (got - ref).abs().max().item()
+        assert err <= bound * ref.abs().max().item(), f"a prompt of {n} tokens: error {err:.3e} of {ref.abs().max().item():.3f}"
+    filled = [k for k in lm.step._graphs if k[0] == "filled"]
+    assert len(filled) == 1, "the prompts shared one captured graph"
+
+
 def test_warm_up_captures_the_sizes_that_prompts_will_come_in(tmp_path):
     """After ``Engine.warm_up`` the first prompt of a length is replayed from a graph captured before any request came,
     and the tokens are the plain model's."""
