@@ -325,8 +325,9 @@ def test_long_prompts_at_head_size_64(tmp_path, dtype):
         assert err <= allowed, f"max error {err:.3e}, allowed {allowed:.3e}"
 
 
+@pytest.mark.parametrize("head_dim", [None, 64])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_yarn_on_the_gpu(tmp_path, dtype):
+def test_yarn_on_the_gpu(tmp_path, dtype, head_dim):
     """YaRN through the kernels (crates/mach-model/src/ref_model.rs:636-704): the scaled frequencies go to the rotation
     kernels as their table, the factors to the attention kernels as the scores' scale; a prompt in portions, then
     decoded tokens (the fused decode kernel rotates by the same table), positions far beyond the original context."""
@@ -334,6 +335,8 @@ def test_yarn_on_the_gpu(tmp_path, dtype):
     from machserve_amd.weights import write_random_model
     raw = dict(TINY_A, max_position_embeddings=1024,
                rope_scaling={"type": "yarn", "factor": 8.0, "original_max_position_embeddings": 64, "mscale": 0.8, "mscale_all_dim": 0.707})
+    if head_dim:  # a head size at which the q/k/v product of the prompt's portions rotates in its own epilogue (two-byte elements)
+        raw["head_dim"] = head_dim
     d = write_random_model(raw, 3, str(tmp_path / "yarn"))
     sharpen_attention(d, 4.0)
     w, sizes = read_for_plain(d)
