@@ -68,3 +68,37 @@ def test_real_layer_sizes(name, dtype):
         assert err <= allowed, f"{name} {dtype}: max error {err:.3e}, allowed {allowed:.3e}"
         if dtype == torch.float32:
             assert torch.equal(got.argmax(-1), ref[:n].argmax(-1))
+
+
+@pytest.mark.timeout(300)
+@pytest.mark.parametrize("T,dtype", [(2000, torch.bfloat16), (2048, torch.float16), (8192, torch.bfloat16)])
+def test_long_prompts_at_the_0_5b_layer_sizes(T, dtype):
+    """A prompt of thousands of tokens in one step at the 0.5B layer sizes (two layers, a small vocabulary), then decoded
+    tokens, against the plain model: what only such sizes reach inside the engine: the widest tiles of the products (128x160,
+    and 256x256 at 8,192 rows), the down projection cut along K, the q/k/v product that rotates and writes the cache, the
+    attention in 32-row tiles over several rounds of blocks, a step filled up and captured."""
+    from machserve_amd.config import config_from_dict
+    from machserve_amd.engine import StepEntry, load_model
+    from machserve_amd.weights import random_tensor_dict
+    raw = config("0.5B")
+    raw.update(vocab_size=8000, max_position_embeddings=16384)
+    cfg = config_from_dict(raw)
+    tensors = random_tensor_dict(cfg, 3)
+    sizes = P.sizes_from_config(raw)
+    ww = {k: v.to(dtype).float() if v.dim() == 2 else v for k, v in tensors.items()}
+    toks = random_prompt(T + 6, 8000, T)
+    ref = P.forward(ww, sizes, toks)
+    lm = load_model(config=cfg, tensors=tensors, dtype=dtype, device=DEV, page_size=64, num_pages=T // 64 + 3, max_requests=1)
+    lm.step.FILLED_CAPTURE_AFTER = 0
+    rows = [0, 63, 64, T // 2, T - 130, T - 2, T - 1]
+    slot = lm.cache.admit()
+    got = [lm.step([StepEntry(slot, toks[:T], rows)])]
+    got += [lm.step([StepEntry(slot, toks[T + i:T + i + 1], [0])]) for i in range(6)]
+    lm.cache.release(slot)
+    lm.cache.check()
+    got = torch.cat(got).float().cpu()
+    want = torch.cat([ref[rows], ref[T:T + 6]])
+    scale = want.abs().max().item()
+    err = (got - want).abs().max().item()
+    allowed = (3e-2 if dtype == torch.bfloat16 else 3e-2 / 8) * scale
+    assert err <= allowed, f"{T} tokens, {dtype}: max error {err:.3e}, allowed {allowed:.3e}"
