@@ -460,7 +460,7 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
     // two 128x128 blocks a CU are a round of the chip (512 on 256 CUs); a tile is taken when its blocks fill
     // six tenths of a round
     const long round_blocks = 2L * compute_units(), enough = round_blocks * 300 / 512;
-    if (M > 64 && ns == 1 && ep.k_per_split >= 128 && forced == 0) {
+    if (M > 64 && (ns == 1 || K >= 16384) && ep.k_per_split >= 128 && forced == 0) {
         // Tiles of 256x256 under eight waves (each 128 rows by 64 columns: 128 accumulator registers, 220 in all, two
         // waves a SIMD; 128 KB of LDS: one block a CU) bring half the bytes of two 128x128 tiles from the L2 into the CUs,
         // which is what bounds the large products (every variant of the 128x128 loop pulls 13 to 15 TB/s).  They pay
@@ -471,7 +471,8 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
         // start and its 256x256 stores) wants the rounds nearly full (0.95: +16 %, 0.79: -5 %).  Three LDS stages
         // (256x128, 128x256), four of K = 32 (256x256: 1.13 against 1.22 PFLOP/s) and four waves of 128x128 each with
         // their sums in the accumulation registers (1.06) were slower than this.
-        const long t256 = (long)ceil_div(M, 256) * ceil_div(N, 256), cus = compute_units();
+        // (with K cut over `ns` blocks - a very long K under few tiles, see plan_tiled_splits - the slices fill the round)
+        const long t256 = (long)ceil_div(M, 256) * ceil_div(N, 256) * ns, cus = compute_units();
         const long rounds = ceil_div(t256, cus);
         if (t256 * 100 >= rounds * cus * (K >= 1536 ? 72 : 90)) MS_GEMM(256, 256, 2, 4, 64);
     }
@@ -519,6 +520,17 @@ static int plan_tiled_splits(int M, int N, int K) {
 #ifdef MS_ELEM_HALF
     const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128);
     const long round_blocks = 2L * compute_units();  // two 128x128 blocks a CU
+    // A very long K under few output tiles (the 7B down projection: K = 18,944, 14 column tiles of 256): tiles of 256x256
+    // bring half the bytes of 128x128 tiles from the L2, but one or two thousand rows of them do not fill the chip's round of
+    // one block a CU; with K cut in two to four they do, and the norm that follows adds the slices.  Measured with that
+    // norm: 2,048 rows 374 -> 330 us in two slices (320 in four), 1,024 rows 198 -> 158 in four; shorter K (the 1.5B down
+    // projection, 8,960) and the 0.5B sizes lose by it, and from 4,096 rows on the uncut tiles fill the round themselves.
+    if (M > 64 && K >= 16384 && g_force_splits == 0) {
+        const long t256 = (long)ceil_div(M, 256) * ceil_div(N, 256), cus = compute_units();
+        if (t256 * 100 < 72 * cus)
+            for (int sl = 2; sl <= 4; ++sl)
+                if (t256 * sl * 100 >= 85 * cus && t256 * sl <= cus) return ceil_div(K, ceil_div(ceil_div(K, sl), 64) * 64);
+    }
     if (b128 >= round_blocks * 300 / 512 && g_force_splits == 0) return 1;
     // More than six slices cost more in the consumer's sums than they gain here (with very few tiles - a
     // portion of a few hundred rows - slices of 256 still pay).  With few rows the partial sums are small
@@ -618,10 +630,13 @@ extern "C" int ms_linear_swiglu_scaled(const void* a, const float* row_ss, int s
 }
 
 // Whether ms_linear_qkv_rope takes this shape: two-byte elements, more rows than the few-rows kernels take, heads of
-// 64 or 128 (a tile's columns are one head, so that both elements of a rotated pair lie in one lane), K in whole chunks.
+// 64 (a tile's columns are one head, so that both elements of a rotated pair lie in one lane), K in whole chunks.
+// Heads of 128 are left to the plain product and the rotation kernel: tiles of one head's width, four waves above one
+// another, give those shapes a worse count of blocks and less reuse in a wave than the plain product's wider tiles
+// (7B layer sizes, 2,048 rows: 133 us in one launch against 81 + 17 in two; 1.5B, 512 rows: the step 6 % longer).
 extern "C" int ms_qkv_rope_takes(int M, int H, int KV, int hd, int K) {
 #ifdef MS_ELEM_HALF
-    return M > 64 && H > 0 && KV > 0 && (hd == 64 || hd == 128) && K % 8 == 0 && K >= 128;
+    return M > 64 && H > 0 && KV > 0 && hd == 64 && K % 8 == 0 && K >= 128;
 #else
     (void)M; (void)H; (void)KV; (void)hd; (void)K;
     return 0;
@@ -653,20 +668,16 @@ extern "C" int ms_linear_qkv_rope(const void* a, const void* w, const float* bia
     } while (0)
     // rows in tiles of 128 where that still gives the chip a round of blocks, else of 64
     const bool tall = (long)ceil_div(M, 128) * (N / hd) >= round_blocks * 300 / 512;
-    if (hd == 64) {
-        if (tall) MS_QKV(128, 64);
-        if (K % 64 == 0 && K >= 256) {
-            // three LDS buffers in turn (two K steps in flight, three blocks a CU): 0.5B, 2,048 rows, 17.0 -> 16.4 us; tiles of
-            // 128x64 take 20.3 (288 blocks, barely one a CU, each step a trip to the L2)
-            const long nb = (long)ceil_div(M, 64) * (N / 64);
-            hipLaunchKernelGGL((gemm_kernel<64, 64, 4, 1, 64, EPI_QKV_ROPE, 3>), dim3((unsigned)nb, 1), dim3(256), 0, stream,
-                               (const elem_t*)a, (const elem_t*)w, M, N, K, ep);
-            return check_launch("gemm q/k/v with rotation 64x64 deep");
-        }
-        MS_QKV(64, 64);
+    if (tall) MS_QKV(128, 64);
+    if (K % 64 == 0 && K >= 256) {
+        // three LDS buffers in turn (two K steps in flight, three blocks a CU): 0.5B, 2,048 rows, 17.0 -> 16.4 us; tiles of
+        // 128x64 take 20.3 (288 blocks, barely one a CU, each step a trip to the L2)
+        const long nb = (long)ceil_div(M, 64) * (N / 64);
+        hipLaunchKernelGGL((gemm_kernel<64, 64, 4, 1, 64, EPI_QKV_ROPE, 3>), dim3((unsigned)nb, 1), dim3(256), 0, stream,
+                           (const elem_t*)a, (const elem_t*)w, M, N, K, ep);
+        return check_launch("gemm q/k/v with rotation 64x64 deep");
     }
-    if (tall) MS_QKV(128, 128);
-    MS_QKV(64, 128);
+    MS_QKV(64, 64);
 #undef MS_QKV
 #else
     (void)a; (void)w; (void)bias; (void)rope_cs; (void)slot_map; (void)q_out; (void)kpool; (void)vpool; (void)M; (void)H; (void)KV;

@@ -7,11 +7,17 @@ the kernel that also writes the cache."""
 from __future__ import annotations
 
 import math
+import weakref
 
 import torch
 
 from .base import PositionEncoding
 from .registry import register_position_encoding
+
+
+# Tables of equal frequencies on one device are one tensor: what a step's layers work out from the table (the rows'
+# cosines and sines) is then found again by the table's address and made once a step, not once a layer.
+_TABLES = weakref.WeakValueDictionary()
 
 
 @register_position_encoding("rotary")
@@ -41,7 +47,12 @@ class Rotary(PositionEncoding):
             inv = (1.0 / (f32(yarn.factor) * torch.pow(theta, 2.0 * j / hd))) * ramp + inv * (1.0 - ramp)
             ln = math.log(yarn.factor)
             self.factor = (0.1 * yarn.mscale * ln + 1.0) / (0.1 * yarn.mscale_all_dim * ln + 1.0)
-        self.inv_freq = inv.to(rt.device)
+        key = (str(rt.device), inv.numpy().tobytes())
+        table = _TABLES.get(key)
+        if table is None:
+            table = inv.to(rt.device)
+            _TABLES[key] = table
+        self.inv_freq = table
 
     def rotary_inv_freq(self):
         return self.inv_freq

@@ -382,6 +382,21 @@ def test_a_step_filled_up_to_a_shared_size_gives_the_same_logits(tmp_path, which
     assert all(g.pool.available() == g.pool.num_pages for g in lm.cache.groups.values())
 
 
+def test_layers_of_equal_frequencies_share_one_rotation_table():
+    """Rotary parts of equal frequencies hold the same tensor (what a step works out from it is then made once for all
+    layers); other frequencies, another table."""
+    from machserve_amd.config import RotarySpec, YarnSpec
+    from machserve_amd.parts import POSITION_ENCODINGS, Runtime
+    rt = Runtime(torch.device("cpu"), torch.float32, EmulatedOps())
+    a, b = (POSITION_ENCODINGS.build(RotarySpec("rotary", 64, 1e6), rt) for _ in range(2))
+    assert a is not b and a.rotary_inv_freq() is b.rotary_inv_freq()
+    for other in (RotarySpec("rotary", 64, 1e4), RotarySpec("rotary", 32, 1e6),
+                  RotarySpec("rotary", 64, 1e6, yarn=YarnSpec(4.0, 64, 32.0, 1.0, 1.0, 0.0))):
+        c = POSITION_ENCODINGS.build(other, rt)
+        assert c.rotary_inv_freq() is not a.rotary_inv_freq() and not (c.rotary_inv_freq().shape == a.rotary_inv_freq().shape
+                                                                         and torch.equal(c.rotary_inv_freq(), a.rotary_inv_freq()))
+
+
 @pytest.mark.parametrize("mscale_all_dim", [0.0, 0.707])
 def test_yarn_through_the_engine_equals_the_plain_model(tmp_path, mscale_all_dim):
     """A configuration with YaRN (crates/mach-model/src/ref_model.rs:636-704): scaled frequencies, the factor on

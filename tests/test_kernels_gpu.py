@@ -97,12 +97,16 @@ def test_linear(dtype, M, N, K):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(65, 896, 4864), (300, 130, 1096), (2048, 896, 4864), (200, 200, 520), (100, 1536, 8960),
-                                   (100, 1536, 1536), (130, 136, 264)])
+                                   (100, 1536, 1536), (130, 136, 264),
+                                   # a very long K under few tiles of 256x256: K cut so that the slices fill the chip's round
+                                   (1000, 3584, 16448)])
 def test_linear_many_rows_cut_along_k(dtype, M, N, K):
     """A product with too few tiles to fill the chip is cut along K into ordered partial sums."""
     ops = ops_for(dtype)
     a, w = rnd((M, K), dtype, 41), rnd((N, K), dtype, 42, K ** -0.5)
     parts = ops.linear_split(a.to(DEV), w.to(DEV))
+    if K >= 16384:
+        assert parts.shape[0] == (1 if dtype == torch.float32 else 4), "56 tiles of 256x256 in four slices are a round of the chip"
     assert parts.shape[1:] == (M, N) and (dtype != torch.float32 or parts.shape[0] == 1)
     assert_close(parts.sum(0), P.linear(a.double(), w.double()), torch.float32 if dtype == torch.float32 else dtype)
     assert ops.linear_split(a.to(DEV), w.to(DEV), allow_partials=False).shape[0] == 1
@@ -762,15 +766,16 @@ def test_logit_edit():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,H,KV,hd,K,ps", [(100, 3, 1, 64, 136, 16), (300, 14, 2, 64, 896, 64), (130, 4, 4, 128, 264, 32),
-                                            (2048, 14, 2, 64, 896, 64), (1100, 12, 2, 128, 200, 64)])
+@pytest.mark.parametrize("M,H,KV,hd,K,ps", [(100, 3, 1, 64, 136, 16), (300, 14, 2, 64, 896, 64), (130, 4, 4, 64, 264, 32),
+                                            (2048, 14, 2, 64, 896, 64), (1100, 12, 3, 64, 200, 64)])
 def test_qkv_product_that_rotates_and_writes_the_cache(dtype, M, H, KV, hd, K, ps):
     """The q/k/v projection of a step of many rows with bias, rotation and cache write in its epilogue: the same queries
     and the same pages as the plain product (32-bit sums) followed by the rotation kernel, and as the plain formulas
     (crates/mach-model/src/batched.rs:3566-3679); rows with a negative slot leave the pages alone; positions that are
     not the rows' indices."""
     ops = ops_for(dtype)
-    assert ops.qkv_rope_takes(M, H, KV, hd, K) and not ops.qkv_rope_takes(64, H, KV, hd, K) and not ops.qkv_rope_takes(M, H, KV, 80, K)
+    assert ops.qkv_rope_takes(M, H, KV, hd, K) and not ops.qkv_rope_takes(64, H, KV, hd, K)
+    assert not ops.qkv_rope_takes(M, H, KV, 80, K) and not ops.qkv_rope_takes(M, H, KV, 128, K)   # other heads: the two kernels
     N = (H + 2 * KV) * hd
     a, w, bias = rnd((M, K), dtype, 1), rnd((N, K), dtype, 2, K ** -0.5), rnd((N,), torch.float32, 3)
     gen = torch.Generator().manual_seed(4)

@@ -226,8 +226,8 @@ def test_steps_of_any_mix_run_from_graphs_of_shared_sizes(tmp_path, which, dtype
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("head_dim,heads,kv", [(64, 6, 2), (128, 32, 2)])
 def test_prompts_of_one_size_from_one_graph_at_head_sizes_64_and_128(tmp_path, dtype, head_dim, heads, kv):
-    """At head sizes 64 and 128 the q/k/v product of a step of many rows rotates by a table of the rows' angles that the
-    step's layers share.  Prompts of several lengths that are filled up to one size run from one captured graph: the
+    """At head size 64 the q/k/v product of a step of many rows rotates by a table of the rows' angles that the step's
+    layers share (at 128 the rotation kernel works the angles out itself).  Prompts of several lengths that are filled up to one size run from one captured graph: the
     table is made inside the graph, from the positions of the step at hand (captured from the first prompt's, every
     later prompt's rows beyond the first one's length would be rotated by the angles of the rows that filled the first
     step up).  Every position's logits against the plain model."""
@@ -242,9 +242,11 @@ def test_prompts_of_one_size_from_one_graph_at_head_sizes_64_and_128(tmp_path, d
     w, sizes = read_for_plain(d)
     ww = _stored(w, dtype)
     lm = load_model(d, dtype=dtype, device=DEV, page_size=64, num_pages=12, max_requests=2)
-    assert lm.rt.ops.qkv_rope_takes(128, heads, kv, head_dim, 200)
+    assert lm.rt.ops.qkv_rope_takes(128, heads, kv, head_dim, 200) == (head_dim == 64)
     bound = 3e-2 if dtype == torch.bfloat16 else 3e-2 / 8
     lm.step.FILLED_CAPTURE_AFTER = 0
+    tables, make_table = [], lm.rt.ops.rope_table
+    lm.rt.ops.rope_table = lambda *a: (tables.append(1), make_table(*a))[1]
     for n in (68, 101, 76, 66, 127, 120):            # all of them filled up to 128 rows
         prompt = random_prompt(n, 512, 300 + n)
         ref = P.forward(ww, sizes, prompt)
@@ -255,6 +257,8 @@ def test_prompts_of_one_size_from_one_graph_at_head_sizes_64_and_128(tmp_path, d
         assert err <= bound * ref.abs().max().item(), f"a prompt of {n} tokens: error {err:.3e} of {ref.abs().max().item():.3f}"
     filled = [k for k in lm.step._graphs if k[0] == "filled"]
     assert len(filled) == 1, "the prompts shared one captured graph"
+    # both layers rotate by one table: one for the run that warms the capture up and one inside the graph, none later
+    assert len(tables) == (2 if head_dim == 64 else 0), f"{len(tables)} tables of angles were made"
 
 
 def test_warm_up_captures_the_sizes_that_prompts_will_come_in(tmp_path):
