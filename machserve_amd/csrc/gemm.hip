@@ -634,9 +634,12 @@ extern "C" int ms_linear_swiglu_scaled(const void* a, const float* row_ss, int s
 // Heads of 128 are left to the plain product and the rotation kernel: tiles of one head's width, four waves above one
 // another, give those shapes a worse count of blocks and less reuse in a wave than the plain product's wider tiles
 // (7B layer sizes, 2,048 rows: 133 us in one launch against 81 + 17 in two; 1.5B, 512 rows: the step 6 % longer).
+// So are steps of up to 256 rows: their few tiles are each a chain of all K steps, which takes 10 us whatever the
+// number of LDS buffers, while the plain product cuts K over several blocks (0.5B sizes, 128 rows: 8.9 us in two
+// kernels, 9.7 to 11.8 in one; from 384 rows on the one kernel is ahead: 10.0 against 10.9).
 extern "C" int ms_qkv_rope_takes(int M, int H, int KV, int hd, int K) {
 #ifdef MS_ELEM_HALF
-    return M > 64 && H > 0 && KV > 0 && hd == 64 && K % 8 == 0 && K >= 128;
+    return M > 256 && H > 0 && KV > 0 && hd == 64 && K % 8 == 0 && K >= 128;
 #else
     (void)M; (void)H; (void)KV; (void)hd; (void)K;
     return 0;
@@ -671,8 +674,14 @@ extern "C" int ms_linear_qkv_rope(const void* a, const void* w, const float* bia
     if (tall) MS_QKV(128, 64);
     if (K % 64 == 0 && K >= 256) {
         // three LDS buffers in turn (two K steps in flight, three blocks a CU): 0.5B, 2,048 rows, 17.0 -> 16.4 us; tiles of
-        // 128x64 take 20.3 (288 blocks, barely one a CU, each step a trip to the L2)
+        // 128x64 take 20.3 (288 blocks, barely one a CU, each step a trip to the L2); four buffers where the blocks are
+        // at most two a CU (512 to 1,536 rows: 10.6 -> 10.0, 11.8 -> 11.4 us; at 2,048 rows 13.4 -> 17.9)
         const long nb = (long)ceil_div(M, 64) * (N / 64);
+        if (nb <= round_blocks) {
+            hipLaunchKernelGGL((gemm_kernel<64, 64, 4, 1, 64, EPI_QKV_ROPE, 4>), dim3((unsigned)nb, 1), dim3(256), 0, stream,
+                               (const elem_t*)a, (const elem_t*)w, M, N, K, ep);
+            return check_launch("gemm q/k/v with rotation 64x64 deeper");
+        }
         hipLaunchKernelGGL((gemm_kernel<64, 64, 4, 1, 64, EPI_QKV_ROPE, 3>), dim3((unsigned)nb, 1), dim3(256), 0, stream,
                            (const elem_t*)a, (const elem_t*)w, M, N, K, ep);
         return check_launch("gemm q/k/v with rotation 64x64 deep");

@@ -766,15 +766,15 @@ def test_logit_edit():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,H,KV,hd,K,ps", [(100, 3, 1, 64, 136, 16), (300, 14, 2, 64, 896, 64), (130, 4, 4, 64, 264, 32),
-                                            (2048, 14, 2, 64, 896, 64), (1100, 12, 3, 64, 200, 64)])
+@pytest.mark.parametrize("M,H,KV,hd,K,ps", [(260, 3, 1, 64, 136, 16), (300, 14, 2, 64, 896, 64), (530, 4, 4, 64, 264, 32),
+                                            (2048, 14, 2, 64, 896, 64), (1100, 12, 3, 64, 200, 64), (3000, 14, 2, 64, 896, 64)])
 def test_qkv_product_that_rotates_and_writes_the_cache(dtype, M, H, KV, hd, K, ps):
     """The q/k/v projection of a step of many rows with bias, rotation and cache write in its epilogue: the same queries
     and the same pages as the plain product (32-bit sums) followed by the rotation kernel, and as the plain formulas
     (crates/mach-model/src/batched.rs:3566-3679); rows with a negative slot leave the pages alone; positions that are
     not the rows' indices."""
     ops = ops_for(dtype)
-    assert ops.qkv_rope_takes(M, H, KV, hd, K) and not ops.qkv_rope_takes(64, H, KV, hd, K)
+    assert ops.qkv_rope_takes(M, H, KV, hd, K) and not ops.qkv_rope_takes(256, H, KV, hd, K)
     assert not ops.qkv_rope_takes(M, H, KV, 80, K) and not ops.qkv_rope_takes(M, H, KV, 128, K)   # other heads: the two kernels
     N = (H + 2 * KV) * hd
     a, w, bias = rnd((M, K), dtype, 1), rnd((N, K), dtype, 2, K ** -0.5), rnd((N,), torch.float32, 3)

@@ -242,12 +242,12 @@ def test_prompts_of_one_size_from_one_graph_at_head_sizes_64_and_128(tmp_path, d
     w, sizes = read_for_plain(d)
     ww = _stored(w, dtype)
     lm = load_model(d, dtype=dtype, device=DEV, page_size=64, num_pages=12, max_requests=2)
-    assert lm.rt.ops.qkv_rope_takes(128, heads, kv, head_dim, 200) == (head_dim == 64)
+    assert lm.rt.ops.qkv_rope_takes(320, heads, kv, head_dim, 200) == (head_dim == 64)
     bound = 3e-2 if dtype == torch.bfloat16 else 3e-2 / 8
     lm.step.FILLED_CAPTURE_AFTER = 0
     tables, make_table = [], lm.rt.ops.rope_table
     lm.rt.ops.rope_table = lambda *a: (tables.append(1), make_table(*a))[1]
-    for n in (68, 101, 76, 66, 127, 120):            # all of them filled up to 128 rows
+    for n in (260, 301, 276, 258, 318, 310):         # all of them filled up to 320 rows
         prompt = random_prompt(n, 512, 300 + n)
         ref = P.forward(ww, sizes, prompt)
         slot = lm.cache.admit()
