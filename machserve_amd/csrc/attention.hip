@@ -19,6 +19,7 @@
 //
 // Compiled once per MS_ATTN_ND (tile head size / 16); a smaller head size runs in the next
 // larger tile with the unused columns zero.
+#include <algorithm>
 #include <mutex>
 #include <type_traits>
 
@@ -1359,6 +1360,58 @@ using namespace ms;
 // keys over that many blocks (few blocks of rows over long contexts would leave most of the chip idle
 // and run as long as their chain of tiles); T is the number of rows, part_o [T, H, nsplit, hd] and
 // part_ml [T, H, nsplit, 2] are float workspaces.
+// Whether a launch with these sizes runs in the kernel of 32-row tiles: where the block tables allow contexts of
+// 2,048 keys and more (measured on one prompt of the 0.5B head shape: 512 tokens 13.9 against 11.9 us, 2,048 32.2
+// against 34.4, 4,096 60 against 83, 8,192 194 against 252), the head size is the tile's, and a block's share of the
+// block table fits its place in LDS (asked for by name with max_key_groups = 32).
+static bool takes_rows32(int hd, int ps, int table_stride, int window, int max_key_groups) {
+#ifdef MS_HAS_ROWS32
+    const long span = window > 0 ? (long)window + BKV : (long)table_stride * ps;
+    const long pages_of_span = window > 0 ? ((long)window + 2 * ROWS_PER_BLOCK + r32::ROUND) / ps + 2 : (long)table_stride;
+    return hd == HDT && pages_of_span <= r32::MAX_TABLE && (max_key_groups == 32 || (max_key_groups == 0 && span >= 2048));
+#else
+    (void)hd; (void)ps; (void)table_stride; (void)window; (void)max_key_groups;
+    return false;
+#endif
+}
+
+static int attention_compute_units() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
+        (void)hipGetLastError();
+        cus = n;
+    }
+    return cus;
+}
+
+// Into how many blocks ms_paged_attention should cut the keys of every block of rows (its `nsplit`) when the caller
+// leaves the choice to the library: n_work items of the work list, T rows in the step.  Few blocks of rows over long
+// contexts leave most of the chip idle and run as long as their chain of tiles; cutting the chain fills the chip, at
+// the price of the partial results' trip through memory and the merge's launch.  Block tables no wider than twice the
+// step's rows are (or may be) those of prompts that run whole, whose blocks walk half the keys on average and whose
+// longest block decides: cutting those only adds (0.5B heads, one prompt of 1,024 tokens 18.9 us uncut, 22.8 in two,
+// 31.9 in four; 1,536 tokens 24.4 / 32.3 / 36.8).  The kernel of 32-row tiles holds one block a CU: it is cut so that
+// blocks x splits stay within one round of the chip, at least 1,024 keys a split (256 rows behind 7,936 keys: 91 us
+// uncut, 25.8 in eight, 35.2 in sixteen; 512 rows behind 7,680: 90.6, 36.2 in four, 50.4 in six; 1,024 rows behind
+// 3,072: 49.4, 38.9 in two, 44.7 in four).  The cut depends on the batch, so results differ in rounding between batches.
+extern "C" int MS_CAT(ms_attention_splits_nd, MS_ATTN_ND)(int n_work, int KV, int T, int hd, int ps, int table_stride, int window) {
+    if (n_work < 1 || KV < 1 || ps < 1 || table_stride < 1) return 1;
+    const long blocks = (long)n_work * KV;
+    long span = (long)table_stride * ps;
+    if (window > 0 && span > (long)window + 64) span = (long)window + 64;
+    if (span <= 2L * T) return 1;
+    long n;
+    if (takes_rows32(hd, ps, table_stride, window, 0)) {
+        n = std::min((long)attention_compute_units() / blocks, span / 1024);
+    } else {
+        if (blocks >= 192) return 1;
+        n = std::min((384 + blocks - 1) / blocks, span / 512);
+    }
+    return (int)std::max(1L, std::min(n, (long)MAX_SPLITS));
+}
+
 extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
     const void* q, const void* kpool, const void* vpool, void* out, const int* block_table, int table_stride,
     const int* seq_q_start, const int* seq_q_len, const int* seq_pos0, const int* work, int n_work, int H, int KV,
@@ -1404,12 +1457,8 @@ extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
 #ifdef MS_HAS_ROWS32
     {
         // tiles of 32 rows by 32 keys under four key groups, a block a CU (the list's order, longest contexts first, is
-        // the order the blocks start in): where the block tables allow contexts of 2,048 keys and more (measured on
-        // one prompt of the 0.5B head shape: 512 tokens 13.9 against 11.9 us, 2,048 32.2 against 34.4, 4,096 60 against 83,
-        // 8,192 194 against 252), the head size is the tile's, and a block's share of the block table fits its
-        // place in LDS (asked for by name with max_key_groups = 32)
-        const long pages_of_span = window > 0 ? ((long)window + 2 * ROWS_PER_BLOCK + r32::ROUND) / ps + 2 : (long)table_stride;
-        if (hd == HDT && pages_of_span <= r32::MAX_TABLE && (max_key_groups == 32 || (max_key_groups == 0 && span >= 2048))) {
+        // the order the blocks start in)
+        if (takes_rows32(hd, ps, table_stride, window, max_key_groups)) {
             a.pair_span = 0;
             const dim3 grid32((unsigned)(n_work * KV), (unsigned)nsplit);
             hipLaunchKernelGGL(paged_attention_rows32_kernel, grid32, dim3(r32::KG * r32::GT), 0, stream, a);

@@ -468,13 +468,14 @@ static int launch_gemm(const elem_t* A, const elem_t* W, int M, int N, int K, Ep
         // 0.5B, 1.5B and 7B layer sizes with 1,024 to 8,192 rows, +4 to +18 % from 0.72 of the rounds' blocks upwards
         // (7B gate/up at 2,048 rows 604 -> 511 us, at 8,192 rows 2,167 -> 1,818 us = 1.22 PFLOP/s; 7B down at 4,096
         // rows 588 -> 496), -15 to -44 % below 0.63; a short K (the 0.5B model's 896: fourteen steps between a tile's
-        // start and its 256x256 stores) wants the rounds nearly full (0.95: +16 %, 0.79: -5 %).  Three LDS stages
+        // start and its 256x256 stores) wants the rounds fuller (0.95: +16 %; 0.89 - 1,536 and 3,072 rows of the 0.5B
+        // gate/up product - +24 and +7 %; 0.79: -5 to +6 %; 0.59: -20 %).  Three LDS stages
         // (256x128, 128x256), four of K = 32 (256x256: 1.13 against 1.22 PFLOP/s) and four waves of 128x128 each with
         // their sums in the accumulation registers (1.06) were slower than this.
         // (with K cut over `ns` blocks - a very long K under few tiles, see plan_tiled_splits - the slices fill the round)
         const long t256 = (long)ceil_div(M, 256) * ceil_div(N, 256) * ns, cus = compute_units();
         const long rounds = ceil_div(t256, cus);
-        if (t256 * 100 >= rounds * cus * (K >= 1536 ? 72 : 90)) MS_GEMM(256, 256, 2, 4, 64);
+        if (t256 * 100 >= rounds * cus * (K >= 1536 ? 72 : 85)) MS_GEMM(256, 256, 2, 4, 64);
     }
     if (M > 64) {
         const long b128 = (long)ceil_div(M, 128) * ceil_div(N, 128), b12864 = (long)ceil_div(M, 128) * ceil_div(N, 64);

@@ -228,11 +228,11 @@ class HipOps:
 
     SKINNY_ROWS = 64  # at most this many rows: the weight-streaming kernels
 
-    def _plan(self, what: str, *sizes: int) -> int:
+    def _plan(self, what: str, *sizes: int, lib=None) -> int:
         key = (what, sizes)
         v = self._plans.get(key)
         if v is None:
-            v = self._plans[key] = int(getattr(self._core, what)(*[_c_int(x) for x in sizes]))
+            v = self._plans[key] = int(getattr(lib or self._core, what)(*[_c_int(x) for x in sizes]))
         return v
 
     def _tiled(self, M: int, N: int, K: int) -> bool:
@@ -414,8 +414,8 @@ class HipOps:
                         work: torch.Tensor, H: int, KV: int, hd: int, page_size: int, window: Optional[int],
                         scale: float, max_key_groups: int = 0, key_splits: int = 0) -> torch.Tensor:
         """``max_key_groups`` asks for that many groups of waves sharing a block's keys (0: the kernel's
-        choice); ``key_splits`` for that many blocks sharing them (0: by the number of blocks of rows
-        and the width of the block tables), merged by a second kernel."""
+        choice); ``key_splits`` for that many blocks sharing them (0: the library's choice by the number of blocks
+        of rows, the step's rows and the width of the block tables), merged by a second kernel."""
         lib, fn = self._attention_lib(hd)[:2]
         T = q.shape[0]
         self._want(q, self.dtype, "attention q", T, H * hd)
@@ -432,7 +432,8 @@ class HipOps:
         if work.dim() != 2 or work.shape[1] != 2 or work.shape[0] == 0:
             raise KernelError(f"attention: work list of shape {tuple(work.shape)}")
         out = torch.empty((T, H * hd), dtype=self.dtype, device=q.device)
-        nsplit = key_splits or self._portion_splits(work.shape[0] * KV, block_table.shape[1] * page_size, window)
+        nsplit = key_splits or self._plan(f"ms_attention_splits_nd{build.attention_tile_for(hd)}", work.shape[0], KV, T, hd, page_size,
+                                          block_table.shape[1], window or 0, lib=lib)
         part_o = part_ml = None
         if nsplit > 1:
             part_o = torch.empty((T, H, nsplit, hd), dtype=torch.float32, device=q.device)
@@ -443,18 +444,6 @@ class HipOps:
                             _c_float(scale), _c_int(max_key_groups), _c_int(T), _c_int(nsplit), _ptr(part_o), _ptr(part_ml),
                             self._stream()))
         return out
-
-    @staticmethod
-    def _portion_splits(blocks: int, span: int, window: Optional[int]) -> int:
-        """Blocks sharing the keys of one block of rows.  Few blocks of rows (a short portion of a
-        prompt, or single rows) over long contexts leave most of the chip idle and take as long
-        as their chain of tiles; cutting the chain fills the chip.  One split has at least 512
-        keys; the cut depends on the batch, so results differ in rounding between batches."""
-        if blocks >= 192:
-            return 1
-        if window:
-            span = min(span, window + 64)
-        return max(1, min(-(-384 // blocks), span // 512, 64))
 
     DECODE_MAX_GROUP = 16  # query heads per key/value head the decode kernel takes
 

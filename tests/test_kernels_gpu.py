@@ -293,7 +293,9 @@ def test_gated_products_with_another_activation(dtype, M, I, K):
                                    # tiles of 128x160 (five pairs of gate and up tiles): whole, and ragged at both edges
                                    (2048, 4864, 896), (1000, 4850, 200),
                                    # tiles of 256x256 (two pairs of gate and up tiles a wave): whole, and ragged at both edges
-                                   (4096, 2048, 128), (4000, 2040, 200)])
+                                   (4096, 2048, 128), (4000, 2040, 200),
+                                   # the same tiles where they fill 0.89 of the chip under a short K
+                                   (1536, 4864, 896)])
 def test_linear_swiglu(dtype, M, I, K):
     from machserve_amd.kernels import interleave_gate_up
     ops = ops_for(dtype)
@@ -456,6 +458,30 @@ def test_attention_key_splits(dtype, splits, H, KV, hd, ps, window):
     seqs = [(0, 1), (0, 300), (517, 1), (1500, 37), (3, 2), (1023, 1), (128, 1), (127, 2)]
     got, ref = _attention_case(dtype, H, KV, hd, ps, window, seqs, 400 + hd + splits, peak=True, splits=splits)
     assert_close(got, ref, dtype, f"attention with the keys cut over {splits} blocks")
+
+
+def test_the_library_s_choice_of_key_splits():
+    """How many blocks share the keys of a block of rows when the caller leaves it to the library: none for block
+    tables that may belong to prompts running whole (no wider than twice the step's rows) and for a full chip; few rows
+    behind a long context are cut, in the kernel of 32-row tiles (head size 64, two-byte elements) so that blocks times
+    splits stay within the chip's CUs, at least 1,024 keys a split; a window bounds the keys that count."""
+    ops = ops_for(torch.bfloat16)
+    lib = ops._attention_lib(64)[0]
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    plan = lambda n_work, KV, T, hd, ps, width, window: lib.ms_attention_splits_nd4(n_work, KV, T, hd, ps, width, window)
+    assert plan(56, 2, 1024, 64, 64, 32, 0) == 1                     # a prompt of 1,024 tokens whole
+    assert plan(84, 2, 1536, 64, 64, 32, 0) == 1
+    assert plan(14, 2, 256, 64, 64, 256, 0) == min(cus // 28, 16)    # 256 rows behind thousands of keys
+    assert plan(28, 2, 512, 64, 64, 128, 0) == min(cus // 56, 8)
+    assert plan(56, 2, 1024, 64, 64, 64, 0) == min(cus // 112, 4)
+    assert plan(200, 2, 3600, 64, 64, 256, 0) == 1                   # the chip is full
+    assert plan(1, 2, 1, 64, 64, 4096, 0) == 64                      # never more than the kernels take
+    assert plan(14, 2, 256, 64, 64, 256, 500) == 1                   # a window of 500 keys: nothing to cut
+    assert plan(4, 2, 64, 64, 16, 64, 0) == min(-(-384 // 8), 1024 // 512)   # a short table: the general kernel's rule
+    lib128 = ops._attention_lib(128)[0]
+    assert lib128.ms_attention_splits_nd8(7, 4, 256, 128, 64, 128, 0) == min(-(-384 // 28), 8192 // 512)
+    f32 = ops_for(torch.float32)._attention_lib(64)[0]
+    assert f32.ms_attention_splits_nd4(14, 2, 256, 64, 64, 256, 0) == min(-(-384 // 28), 16384 // 512)   # no 32-row kernel in 32-bit
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
