@@ -41,6 +41,7 @@ PEAK_FLOPS = {"bf16": 2.5e15, "f16": 2.5e15, "f32": 157.3e12}
 REF_DECODE_B64_CTX2048 = 4777.0   # README.md:15, docs/benchmark-protocol.md:74-75
 REF_PREFILL_2048 = 2048 / 0.289   # README.md:18
 REF_DECODE_B256_SHORT = 29273.0   # docs/roadmap.md:324-325 (short contexts)
+REF_DECODE_B512_SHORT = 35251.0   # the same sweep's last entry
 
 QWEN25_05B = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_size": 896, "num_hidden_layers": 24,
@@ -548,6 +549,10 @@ def main() -> int:
             points["decode_b256_ctx512"] = round(v, 1)
             if "vs_reference" in out:
                 out["vs_reference"]["decode_b256_short_contexts"] = round(v / REF_DECODE_B256_SHORT, 2)
+            v, detail["decode_b512_ctx512"] = decode_point(args.shape, 512, 512)
+            points["decode_b512_ctx512"] = round(v, 1)
+            if "vs_reference" in out:
+                out["vs_reference"]["decode_b512_short_contexts"] = round(v / REF_DECODE_B512_SHORT, 2)
             # the same configuration in the reference's own fast precision and in true 32-bit
             for dtn in ("f16", "f32"):
                 v, detail[f"{dtn}_decode_b8"] = decode_point(args.shape, args.batch, ctx, dtn)
