@@ -751,6 +751,20 @@ def test_sampler_greedy_ties_and_spread():
     tok, _ = ops.sample(big.to(DEV), torch.zeros(5).to(DEV), torch.zeros(5, dtype=torch.int32, device=DEV), torch.ones(5).to(DEV),
                         torch.zeros(5, dtype=torch.int64, device=DEV))
     assert tok.cpu().tolist() == [int(big[i].argmax()) if i != 3 else 77 for i in range(5)]
+    # the maximum at the borders of the chunks that the first stage cuts a row into, with rows that are 16-byte aligned
+    # (a thread reads four entries at a time) and rows that are not
+    for V2 in (1000, 1001, 777, 4096, 6002):
+        chunk = -(-(-(-V2 // 64)) // 4) * 4
+        places = sorted({0, 1, 3, 4, chunk - 1, chunk, chunk + 1, 2 * chunk - 1, 5 * chunk, V2 - 5, V2 - 4, V2 - 1} & set(range(V2)))
+        rows = torch.randn(len(places), V2, generator=torch.Generator().manual_seed(V2))
+        for i, at in enumerate(places):
+            rows[i, at] = 30.0
+            if at + 2 < V2:
+                rows[i, at + 2] = 30.0           # a tie further on loses
+        n = len(places)
+        tok, _ = ops.sample(rows.to(DEV), torch.zeros(n).to(DEV), torch.zeros(n, dtype=torch.int32, device=DEV), torch.ones(n).to(DEV),
+                            torch.zeros(n, dtype=torch.int64, device=DEV))
+        assert tok.cpu().tolist() == places, f"vocabulary of {V2}"
     # a flat distribution is covered by different seeds
     flat = torch.zeros(64, V)
     st = torch.arange(1, 65, dtype=torch.int64).to(DEV)
