@@ -717,8 +717,11 @@ extern "C" int ms_prefers_tiled(int M, int N, int K) {
         // whole share at once and then waits.  From one row on (decode steps of the 1.5B and 7B layer sizes at
         // batch 1, 2, 4, 8: 7 to 12 % shorter; the vocabulary-sized head of every shape); a smaller weight
         // (0.5B gate/up) from 17 rows on, where the few-rows kernel can no longer apply the norm itself and
-        // re-reads its rows for every 32 columns (batch 32: 1.53 -> 1.40 ms a step).
-        return nk >= 10e6 || M >= 17;
+        // re-reads its rows for every 32 columns (batch 32: 1.53 -> 1.40 ms a step); from 9 rows on where the output
+        // is wide (0.5B gate/up, 9,728 columns), together with the narrow projections below: the norm between them
+        // then runs by itself and adds the K slices (0.5B decode step at batch 12 and 16: 1.085 -> 1.056 ms; a
+        // 2,048-wide output, the 1.5B q/k/v projection, loses 1 % by it and keeps the few-rows kernel up to 16 rows).
+        return nk >= 10e6 || M >= 17 || (M >= 9 && N >= 4096);
     }
     if (N >= 1024) {
         // a projection of the width (q/k/v, output): from 16 rows, or 8 if it is not small (batch 32: 1.40 ->
@@ -726,8 +729,10 @@ extern "C" int ms_prefers_tiled(int M, int N, int K) {
         // projection: 27 MB) from one row on (1.5B decode step at batch 1 and 4: 1.5 % shorter)
         return M >= 16 || (M >= 8 && nk >= 2e6) || nk >= 10e6;
     }
-    // a narrow output with a long K (a down projection): the tiled kernel cuts K over many blocks
-    return M >= 32 && K >= 4096;
+    // a narrow output (the 0.5B output and down projections, 896 columns): from 9 rows on the tiled kernel with K cut
+    // over many blocks (0.5B decode step at batch 24 and 32: 1.195 -> 1.129 and 1.200 -> 1.138 ms, all of it from the
+    // output projection; at 9 to 16 rows only together with the gate/up product above)
+    return M >= 9;
 #else
     return 0;
 #endif
