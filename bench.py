@@ -324,10 +324,15 @@ def main() -> int:
     recording = [False]
     recorders = []
 
+    def head_start(batch, ctx, budget):
+        """Tokens that the first request may decode while the last one's prompt is still being fed (a step takes every
+        decoding request's token and ``budget`` tokens in all): what a request is given beyond the timed steps."""
+        return max(2 * batch + 88, -(-batch * ctx // max(budget - batch, 1)) + batch + 24)
+
     def make_engine(shape, batch, budget, ctx, windows=1, dtn=None, page=None):
         cfg, tensors, _ = model_of(shape, dtn)
         page = page or args.page_size
-        per_req = -(-(ctx + args.warmup + windows * args.steps + 2 * batch + 96) // page)
+        per_req = -(-(ctx + args.warmup + windows * args.steps + head_start(batch, ctx, budget) + 8) // page)
         lm = load_model(config=cfg, tensors=tensors, dtype=DT[dtn or args.dtype], page_size=page, num_pages=batch * per_req + 4,
                         max_requests=batch)
         if args.record_calls and not recorders:
@@ -339,7 +344,7 @@ def main() -> int:
         cfg = model_of(shape, dtn)[0]
         eng = make_engine(shape, batch, 4096, ctx, windows, dtn, page)
         for p in prompts(cfg, batch, ctx):
-            eng.add(p, args.warmup + windows * args.steps + 2 * batch + 88, SamplingParams())  # early ones decode while later ones prefill
+            eng.add(p, args.warmup + windows * args.steps + head_start(batch, ctx, 4096), SamplingParams())  # early ones decode while later ones prefill
         while any(not r.decoding for r in eng.scheduler.running) or eng.scheduler.waiting:
             eng.step()
         # the engine's own loop (Engine.run): a step is launched while the tokens of the step before
