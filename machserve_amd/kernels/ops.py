@@ -62,6 +62,7 @@ class HipOps:
         self._libs: list = []
         self._core = self._load(build.ensure_library("core", self.elem))
         self._attn = {}
+        self._cus = torch.cuda.get_device_properties(self._index).multi_processor_count
         # what the library plans for a product depends on its sizes alone: asked once per size
         self._plans: dict = {}
 
@@ -447,15 +448,17 @@ class HipOps:
 
     DECODE_MAX_GROUP = 16  # query heads per key/value head the decode kernel takes
 
-    @staticmethod
-    def _decode_splits(S: int, KV: int, table_width: int, page_size: int, window: Optional[int], key_tile: int,
+    def _decode_splits(self, S: int, KV: int, table_width: int, page_size: int, window: Optional[int], key_tile: int,
                        hd: int = 64) -> int:
-        """Blocks sharing a request's keys: enough for two blocks a CU with small heads, one with heads
-        above 64 (measured at head sizes 64 and 128, 1 to 64 requests), at least four key tiles each."""
+        """Blocks sharing a request's keys: as many as stay within one round of the chip, which holds two blocks a CU
+        with small heads and one with heads above 64 (measured at head sizes 64 and 128, 1 to 200 requests: a split more
+        than that starts a second round of blocks, and every round has the kernel's whole chain of latencies in it: 7B
+        heads, 48 requests of 512 keys, 22 us uncut, 31 in two; 0.5B heads, 200 requests, 19 against 25), at least
+        four key tiles each."""
         span = table_width * page_size if not window else min(table_width * page_size, window + key_tile)
         tiles = max(1, -(-span // key_tile))
-        blocks = 512 if hd <= 64 else 256
-        return max(1, min(-(-blocks // (S * KV)), -(-tiles // 4), 64))
+        blocks = self._cus * (2 if hd <= 64 else 1)
+        return max(1, min(blocks // (S * KV), -(-tiles // 4), 64))
 
     def decode_attention_fused(self, qkv: torch.Tensor, bias: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor],
                                slot_map: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
