@@ -115,11 +115,9 @@ __global__ __launch_bounds__(256) void rmsnorm_wide_kernel(float* __restrict__ x
     for (int g = 0; g < G; ++g) {
         if (threadIdx.x + g * 256 >= ng) continue;
         const f32x4 o = v[g] * wv[g] * inv;
-        OutT* q = dst + (size_t)at[g] * 4;
-        q[0] = from_f32<OutT>(o.x);
-        q[1] = from_f32<OutT>(o.y);
-        q[2] = from_f32<OutT>(o.z);
-        q[3] = from_f32<OutT>(o.w);
+        typedef OutT out4_t __attribute__((ext_vector_type(4)));  // the group's four values in one store
+        const out4_t o4 = {from_f32<OutT>(o.x), from_f32<OutT>(o.y), from_f32<OutT>(o.z), from_f32<OutT>(o.w)};
+        *reinterpret_cast<out4_t*>(dst + (size_t)at[g] * 4) = o4;
     }
 }
 
