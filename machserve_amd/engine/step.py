@@ -236,18 +236,22 @@ class StepFunction:
     @staticmethod
     def _row_bucket(n: int) -> int:
         """Rows of the captured step that takes a step of ``n`` rows which is not plain decoding: multiples of 16 up
-        to 64 rows, of 64 up to 512, of 256 beyond (a step's time grows slowly with its rows while they are few:
-        1.25 ms at 16 rows of the 0.5B sizes, 1.35 at 64, 1.47 at 128, 1.52 at 256, 2.0 at 512)."""
+        to 64 rows, of 64 up to 512, of 128 up to 1,024, of 256 beyond (a step's time grows slowly with its rows while
+        they are few: 1.25 ms at 16 rows of the 0.5B sizes, 1.35 at 64, 1.47 at 128, 1.52 at 256, 2.0 at 512)."""
         if n <= 64:
             return -(-n // 16) * 16
-        return -(-n // 64) * 64 if n <= 512 else -(-n // 256) * 256
+        if n <= 512:
+            return -(-n // 64) * 64
+        return -(-n // 128) * 128 if n <= 1024 else -(-n // 256) * 256
 
     def _fill_shape(self, n_seqs: int, n_rows: int, n_want: int):
         """``(rows, requests, wanted rows)`` that a step of any mix is filled up to, or None if it runs in its own
         shape: the requests to the next power of two that leaves room for one more (the rows that fill the step up
         need a request to belong to), the rows to their bucket, the wanted rows to a power of two; a step whose rows are
-        a bucket's already keeps its requests.  Beyond 512 rows a
-        step is filled by at most 64 rows: more would cost more than the launches that a replay saves."""
+        a bucket's already keeps its requests.  Beyond 1,024 rows a step is filled by at most 64 rows: more would cost
+        more than the launches that a replay saves (launched kernel by kernel a step takes the host some 2.4 ms, which
+        the device is busy for from about 1,000 rows on; a prompt of 640 tokens: 2.44 ms launched, 2.35 replayed in 768
+        rows)."""
         if self._row_bucket(n_rows) == n_rows:
             seqs, rows = n_seqs, n_rows  # the step has a shared size already (a portion of the token budget, say)
         else:
@@ -255,7 +259,7 @@ class StepFunction:
             while seqs < n_seqs + 1:
                 seqs *= 2
             rows = self._row_bucket(n_rows + seqs - n_seqs)
-        if rows > self.CAPTURE_MAX_ROWS or (n_rows > 512 and rows - n_rows > 64):
+        if rows > self.CAPTURE_MAX_ROWS or (n_rows > 1024 and rows - n_rows > 64):
             return None
         want = 0
         if n_want:

@@ -346,7 +346,8 @@ def test_a_step_filled_up_to_a_shared_size_gives_the_same_logits(tmp_path, which
     lm = load_model(d, dtype="float32", device="cpu", page_size=16, num_pages=24, max_requests=4, ops=EmulatedOps())
     sf = lm.step
     assert sf._fill_shape(1, 100, 1) == (128, 2, 1) and sf._fill_shape(3, 17, 3) == (32, 4, 4) and sf._fill_shape(4, 60, 0) == (64, 8, 0) and sf._fill_shape(4, 64, 0) == (64, 4, 0)
-    assert sf._fill_shape(1, 600, 1) is None and sf._fill_shape(1, 1000, 1) == (1024, 2, 1) and sf._fill_shape(1, 2048, 1) == (2048, 1, 1) and sf._fill_shape(2, 5000, 1) is None
+    assert sf._fill_shape(1, 600, 1) == (640, 2, 1) and sf._fill_shape(1, 1000, 1) == (1024, 2, 1) and sf._fill_shape(1, 1100, 1) is None
+    assert sf._fill_shape(1, 1230, 1) == (1280, 2, 1) and sf._fill_shape(1, 2048, 1) == (2048, 1, 1) and sf._fill_shape(2, 5000, 1) is None
     seqs = [random_prompt(n, sizes["vocab"], 20 + n) for n in (50, 23, 9)]
     refs = [P.forward(w, sizes, s) for s in seqs]
     slots = [lm.cache.admit() for _ in seqs]
