@@ -539,7 +539,10 @@ static int plan_tiled_splits(int M, int N, int K) {
     // rows: 49 us with 6 slices, 33 with 12 to 16).
     // (measured again at 33 and 64 rows of the three layer sizes: 1.5B down projection, K = 8,960, 9.0 us in 10
     // slices, 10.0 in 16, and its consumer sums fewer planes)
-    const int most = M <= 128 ? (K >= 16384 ? 16 : (K >= 8192 ? 10 : 8)) : 6;
+    // (and again once few blocks ran with four LDS buffers in turn: with its 56 column tiles in four slices the 7B down
+    // projection stays within a round of blocks and takes that kernel, 30 to 34 us at 16 to 64 rows with the sum of its
+    // planes, against 31 to 36 in thirteen; the 7B decode step at 16 to 64 requests 0.5 to 1 % shorter)
+    const int most = M <= 128 ? (K >= 16384 ? (M <= 64 ? 4 : 16) : (K >= 8192 ? 10 : 8)) : 6;
     // (a handful of tiles under few rows - a small projection in a decode step of 33 to 64 requests:
     // slices of 128, or the step's few blocks leave the chip idle)
     // (from K = 1,536 on slices of 256, which run with four LDS buffers in turn: 1.5B output projection at 64
