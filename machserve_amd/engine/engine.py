@@ -60,8 +60,9 @@ class Engine:
             if not 1 <= n <= min(self.scheduler.max_batch_tokens, lm.model.spec.max_positions) or lm.cache.slots.available() < 1:
                 continue
             slot = lm.cache.admit()
-            try:
-                lm.step([StepEntry(slot, [0] * n, [n - 1])], borrow_logits=True, capture_now=True)
+            try:  # as the engine runs a prompt that fits one step: sampled inside the step
+                if lm.step.step_and_sample([StepEntry(slot, [0] * n, [n - 1])], [0.0], [0], [1.0], [0], capture_now=True) is None:
+                    lm.step([StepEntry(slot, [0] * n, [n - 1])], borrow_logits=True, capture_now=True)
             except OutOfPages:
                 pass
             finally:
@@ -178,7 +179,17 @@ class Engine:
             if fast is not None:
                 from ..sampling import advance
                 return self.scheduler.update(plan, fast[0], fast[1], [advance(r.rng_state) for r in reqs])
-        logits = self.loaded.step(entries, borrow_logits=True)
+        declined = False
+        if try_fast and sampled_items and all(r.params.plain() for r in reqs):
+            # portions of prompts, alone or beside decoded tokens: the captured step of their shared size samples too
+            fast = self.loaded.step.step_and_sample(
+                entries, [r.params.temperature for r in reqs], [r.params.top_k for r in reqs],
+                [r.params.top_p for r in reqs], [r.rng_state for r in reqs])
+            if fast is not None:
+                from ..sampling import advance
+                return self.scheduler.update(plan, fast[0], fast[1], [advance(r.rng_state) for r in reqs])
+            declined = self.loaded.step.use_graphs  # its shape is counted there, and captured there when it has come often enough
+        logits = self.loaded.step(entries, borrow_logits=True, eager=declined)
         if not sampled_items:
             return self.scheduler.update(plan, [])
         tokens, logprobs, states, top = self.sampler.sample(logits, [r.params for r in reqs], [r.rng_state for r in reqs],

@@ -274,7 +274,11 @@ class StepFunction:
         # for given tokens per request, wanted rows and table widths the buffer's layout is always the same
         return (tuple(counts), n_want, tuple(sorted(widths.items())), sampled)
 
-    def _run_graph(self, key: tuple, built, sampling=None, after: Optional["LaunchedDecode"] = None, fill_rows: int = 0):
+    def _run_graph(self, key: tuple, built, sampling=None, after: Optional["LaunchedDecode"] = None, fill_rows: int = 0,
+                   samples_feed_tokens: bool = True):
+        """Replays the captured step of this key on ``built`` (captures it first if it has none).  With ``sampling`` the
+        graph also samples at its logits' rows; with ``samples_feed_tokens`` (a decode step: row i is sample i) the
+        samples are left in the step's token section as well, where the next replay finds its input."""
         host, offsets, widths = built
         extra: Dict[str, np.ndarray] = {}
         if sampling is not None:
@@ -337,7 +341,7 @@ class StepFunction:
                     dg.sampled = self.rt.ops.sample_packed(
                         dg.logits, sec("sample/temperature").view(torch.float32), sec("sample/top_k"),
                         sec("sample/top_p").view(torch.float32), sec("sample/state").view(torch.int64), True,
-                        also_tokens=sec("tokens"))
+                        also_tokens=sec("tokens") if samples_feed_tokens else None)
             dg.graph = graph
             self._graphs[key] = dg
             while len(self._graphs) > 1 and (len(self._graphs) > self.MAX_GRAPHS or self.graph_bytes() > self.MAX_GRAPH_BYTES):
@@ -404,20 +408,68 @@ class StepFunction:
         n = len(launched.slots)  # rows beyond belong to no request
         return launched.result[0, :n].tolist(), launched.result[1, :n].view(torch.float32).tolist()
 
+    def step_and_sample(self, entries: Sequence[StepEntry], temperatures, top_ks, top_ps, states, capture_now: bool = False):
+        """A step of any mix (portions of prompts, alone or beside decoded tokens) whose wanted rows are sampled inside
+        the captured step: ``temperatures`` ... ``states`` hold one value for every wanted row, in the order of the
+        entries.  Returns ``(tokens, logprobs)`` as host lists in that order: one small copy brings them, where the
+        logits' way is three uploads, two launches and two copies behind the step (0.1 ms: 7 % of a short prompt's
+        first token).  None, before anything is taken or run, if the step cannot take this path: it is plain decoding
+        (``decode_and_sample``), it is not filled up to a shared size, or that size has not come often enough to be
+        captured (the caller then runs it through ``__call__`` with ``eager`` and samples from the logits)."""
+        if not (self.use_graphs and self.model.observer is None and all(e.positions is None for e in entries)):
+            return None
+        if all(len(e.tokens) == 1 for e in entries) and len({e.slot for e in entries}) == len(entries):
+            return None
+        cache = self.cache
+        checked = self._check_entries(entries)
+        slots, counts, tokens, want, _ = checked
+        if not want or len(want) != len(temperatures):
+            return None
+        fill = self._fill_shape(len(slots), len(tokens), len(want))
+        if fill is None:
+            return None
+        pages = max(-(-(cache.length(sl) + n) // cache.page_size) for sl, n in zip(slots, counts))
+        width = self.TABLE_BUCKET
+        while width < pages:
+            width *= 2
+        # the graph's key holds every group's table width, which only the built step knows: how often the size has
+        # come is counted under the width asked for
+        seen_as = ("filled, sampled",) + fill + (width,)
+        if not self._ready(seen_as, 0 if capture_now else self.FILLED_CAPTURE_AFTER):
+            return None
+        self._seen[seen_as] = max(self._seen.get(seen_as, 0), self.FILLED_CAPTURE_AFTER)  # it runs from a graph from now on
+        self._take_pages(entries)
+        try:
+            built = cache.build_step(slots, counts, tokens, want, self.heads_per_kv, self.rows_per_block, width, 0,
+                                     self.position_axes, (), fill)
+        except CacheError as e:
+            raise StepError(str(e)) from e
+        key = seen_as + tuple(sorted(built[2].items()))
+        # the rows that fill the wanted rows up sample greedily and are dropped
+        pad = fill[2] - len(want)
+        sampling = tuple(list(v) + [f] * pad for v, f in ((temperatures, 0.0), (top_ks, 0), (top_ps, 1.0), (states, 0)))
+        sampled, _ = self._run_graph(key, built, sampling, None, fill_rows=fill[0] - len(tokens), samples_feed_tokens=False)
+        for e in entries:
+            cache.commit(e.slot, len(e.tokens))
+        both = sampled[:, :len(want)].cpu()  # the step's synchronisation
+        return both[0].tolist(), both[1].view(torch.float32).tolist()
+
     # ------------------------------------------------------------------ the step
-    def __call__(self, entries: Sequence[StepEntry], borrow_logits: bool = False, capture_now: bool = False) -> Optional[torch.Tensor]:
+    def __call__(self, entries: Sequence[StepEntry], borrow_logits: bool = False, capture_now: bool = False,
+                 eager: bool = False) -> Optional[torch.Tensor]:
         """Float32 logits ``[number of wanted places, vocab]`` in the order of the entries and
         of their ``want`` lists (None if nothing is wanted).  Takes the pages the new tokens
         need (raises ``OutOfPages`` before anything ran if they are not there), runs the
         model, and advances the requests' lengths.  With ``borrow_logits`` the result may be a
         buffer that the next step overwrites (the engine samples from it at once); with
         ``capture_now`` a step that may run from a captured graph is captured at once, not
-        when its shape has come a few times."""
+        when its shape has come a few times; with ``eager`` it is launched kernel by kernel whatever its shape
+        (a step that ``step_and_sample`` has declined: its shape is counted there)."""
         cache = self.cache
         checked = self._check_entries(entries)  # a step that is refused has taken nothing
         self._take_pages(entries)
         # a captured step takes positions from the cache, and shows no layer's stream to an observer
-        graphs = self.use_graphs and self.model.observer is None and all(e.positions is None for e in entries)
+        graphs = self.use_graphs and not eager and self.model.observer is None and all(e.positions is None for e in entries)
         if graphs and all(len(e.tokens) == 1 for e in entries) and len({e.slot for e in entries}) == len(entries):
             built, key, pad = self._decode_shape(checked, False)
             if self._ready(key, self.DECODE_CAPTURE_AFTER):

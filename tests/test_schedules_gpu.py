@@ -196,6 +196,64 @@ def test_temperature_sampling_through_the_entry_point_equals_the_plain_draws(tmp
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_a_step_of_any_mix_that_samples_inside_the_step(tmp_path, which, dtype):
+    """``step_and_sample``: portions of prompts beside decoded tokens, some rows greedy and some drawn at a temperature
+    with top-k and top-p, a portion that samples nothing in between; captured at its first coming and replayed with other
+    tokens.  The same tokens and log-probabilities as the sampler's kernel gives on the logits of ``__call__`` in a second
+    model of the same weights, step after step (the sampled tokens are fed to both, so their caches stay alike)."""
+    from machserve_amd.engine import StepEntry, load_model
+    d = make_model_dir(tmp_path, which)
+    sizes = read_for_plain(d)[1]
+    a = load_model(d, dtype=dtype, device=DEV, page_size=16, num_pages=40, max_requests=4)
+    b = load_model(d, dtype=dtype, device=DEV, page_size=16, num_pages=40, max_requests=4)
+    b.step.FILLED_CAPTURE_AFTER = 0   # the same filled sizes, hence the same kernels on the same shapes: the same logits bit by bit
+    ops = a.rt.ops
+    prompts = [random_prompt(n, sizes["vocab"], 700 + n) for n in (40, 23, 9, 31)]
+    sa, sb = [a.cache.admit() for _ in prompts], [b.cache.admit() for _ in prompts]
+    fed = [0] * 4
+    state = [11, 12, 13, 14]
+    # (request, tokens of it in this step, sampled?) per step; request 0 comes in three portions
+    plan = [[(0, 17, False), (1, 23, True)],
+            [(0, 16, False), (1, 1, True), (2, 9, True)],
+            [(0, 7, True), (1, 1, True), (2, 1, True), (3, 31, True)],
+            [(0, 17, False), (1, 23, True)]]   # the first step's shape again, replayed: other requests, other tokens
+    temp, top_k, top_p = [0.0, 0.9, 0.7, 0.0], [0, 0, 5, 0], [1.0, 0.8, 1.0, 1.0]
+    assert a.step.step_and_sample([StepEntry(sa[0], [1], [0]), StepEntry(sa[1], [2], [0])], [0.0, 0.0], [0, 0], [1.0, 1.0], [1, 2]) is None, \
+        "plain decoding is not this path's"
+    for i, step in enumerate(plan):
+        if i == 3:   # new requests in the slots of 0 and 1
+            for r in (0, 1):
+                a.cache.release(sa[r]), b.cache.release(sb[r])
+                sa[r], sb[r], fed[r] = a.cache.admit(), b.cache.admit(), 0
+                prompts[r] = random_prompt(len(prompts[r]), sizes["vocab"], 800 + r)
+        ea, eb, who = [], [], []
+        for r, n, sampled in step:
+            toks = prompts[r][fed[r]:fed[r] + n]
+            assert len(toks) == n
+            ea.append(StepEntry(sa[r], toks, [n - 1] if sampled else []))
+            eb.append(StepEntry(sb[r], toks, [n - 1] if sampled else []))
+            fed[r] += n
+            if sampled:
+                who.append(r)
+                prompts[r] = prompts[r] + [0]     # room for the token that is sampled now
+        got = a.step.step_and_sample(ea, [temp[r] for r in who], [top_k[r] for r in who], [top_p[r] for r in who],
+                                     [state[r] for r in who], capture_now=True)
+        assert got is not None, f"step {i} must take the path"
+        logits = b.step(eb)
+        tok, lp = ops.sample(logits, torch.tensor([temp[r] for r in who], device=DEV), torch.tensor([top_k[r] for r in who], dtype=torch.int32, device=DEV),
+                             torch.tensor([top_p[r] for r in who], device=DEV), torch.tensor([state[r] for r in who], dtype=torch.int64, device=DEV))
+        assert got[0] == tok.cpu().tolist(), f"step {i}: tokens {got[0]} against {tok.cpu().tolist()}"
+        assert (torch.tensor(got[1]) - lp.cpu()).abs().max().item() <= 1e-6, f"step {i}: log-probabilities"
+        for r, t in zip(who, got[0]):
+            prompts[r][fed[r]] = t
+            state[r] += 100
+        a.cache.check(), b.cache.check()
+    filled = [k for k in a.step._graphs if k[0] == "filled, sampled"]
+    assert len(filled) == 3, f"{len(filled)} graphs: the fourth step ran from the first one's"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("which", ["A", "B", "C"])
 def test_steps_of_any_mix_run_from_graphs_of_shared_sizes(tmp_path, which, dtype):
     """Prompts of many lengths, alone and beside requests that decode, each step filled up to a size that many steps
