@@ -18,6 +18,17 @@ __global__ __launch_bounds__(256) void embed_kernel(const int* __restrict__ toke
     for (int c = threadIdx.x; c < d; c += 256) dst[c] = to_f32(src[c]) * scale;
 }
 
+// tokens[rows[i]] = sampled[src[i]] for the i with 0 <= rows[i] < n_tokens and 0 <= src[i] < n_sampled: the input of
+// those rows of a step that the step before it sampled, taken on the device (the host has not seen them yet)
+__global__ __launch_bounds__(256) void feed_tokens_kernel(int* __restrict__ tokens, const int* __restrict__ sampled,
+                                                          const int* __restrict__ rows, const int* __restrict__ src, int n,
+                                                          int n_tokens, int n_sampled) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int r = rows[i], s = src[i];
+    if (r >= 0 && r < n_tokens && s >= 0 && s < n_sampled) tokens[r] = sampled[s];
+}
+
 // r = rows ? rows[i] : i;  v = x[r, :] + sum_p partials[p, r, :] (in order);  if partials are given
 // and no rows are gathered, x[r, :] = v is written back (the residual stream takes the pending
 // sums);  out[i, :] = v * rsqrt(mean(v^2) + eps) * w.
@@ -299,6 +310,14 @@ extern "C" int ms_embed(const int* tokens, const void* table, float* x, int T, i
     MS_REQUIRE(T > 0 && d > 0, "embed: empty problem T=%d d=%d", T, d);
     hipLaunchKernelGGL(embed_kernel, dim3(T), dim3(256), 0, stream, tokens, (const elem_t*)table, x, d, scale);
     return check_launch("embed");
+}
+
+extern "C" int ms_feed_tokens(int* tokens, const int* sampled, const int* rows, const int* src, int n, int n_tokens, int n_sampled,
+                              hipStream_t stream) {
+    MS_REQUIRE(n > 0 && n_tokens > 0 && n_sampled > 0, "feed_tokens: empty problem n=%d tokens=%d sampled=%d", n, n_tokens, n_sampled);
+    MS_REQUIRE(tokens && sampled && rows && src, "feed_tokens: a buffer is missing");
+    hipLaunchKernelGGL(feed_tokens_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, stream, tokens, sampled, rows, src, n, n_tokens, n_sampled);
+    return check_launch("feed_tokens");
 }
 
 // rows may be null (identity).  out is float when out_f32 != 0, else the element type.

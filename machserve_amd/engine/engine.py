@@ -95,13 +95,13 @@ class Engine:
         return self._run_plan(plan)
 
     def step_pipelined(self):
-        """Like :meth:`step`, but a step of decoded tokens is launched before the tokens of the step
-        before it have come back: it takes them on the device, and the host's share of a step (the
-        scheduler, the step's buffers, reading the samples) runs while the device works.  What is
-        returned is what has become known by now, which lags the launches by one step; what would
-        end a request is seen one step late, and the token computed for it in between is dropped.
-        Steps that are not plain decoding of the same requests (a prompt portion, an arrival, an
-        end, sampling with penalties) are run as :meth:`step` runs them, after what is in flight."""
+        """Like :meth:`step`, but a step is launched before the tokens of the step before it have come back: the
+        requests that decode take them on the device, and the host's share of a step (the scheduler, the step's buffers,
+        reading the samples) runs while the device works.  What is returned is what has become known by now, which lags
+        the launches by one step; what would end a request is seen one step late, and the token computed for it in
+        between is dropped.  Steps that cannot be launched so (sampling with penalties, biases or top log-probabilities,
+        a preemption, a shape that has no captured step yet) are run as :meth:`step` runs them, after what is in
+        flight."""
         sched = self.scheduler
         if self._inflight is None:
             plan = sched.schedule()
@@ -113,7 +113,7 @@ class Engine:
             return [], []
         prev_plan, prev = self._inflight
         plan = sched.schedule()
-        launched = self._launch(plan, prev) if self._continues(prev_plan, plan) else None
+        launched = self._launch(plan, (prev_plan, prev))
         emitted, done = sched.complete(prev_plan, *self.loaded.step.collect(prev))
         if launched:
             self._inflight = (plan, launched)
@@ -125,28 +125,47 @@ class Engine:
         em2, done2 = self._run_plan(plan, try_fast=launched is None)
         return emitted + em2, done + done2
 
-    def _continues(self, before: StepPlan, plan: StepPlan) -> bool:
-        """Whether ``plan`` decodes one token for exactly the requests of ``before``, in its order."""
-        return (not plan.preempted and not plan.admitted and len(plan.items) == len(before.items)
-                and all(a.request is b.request and a.sample and a.count == 1 for a, b in zip(plan.items, before.items)))
-
     def _launch(self, plan: StepPlan, after):
-        """Launch ``plan`` without waiting if it is plain decoding; None (nothing done) if it is not,
-        False if the step function declined."""
-        if not plan.items or not all(it.sample and it.count == 1 and it.request.params.plain() for it in plan.items):
-            return None
-        if after is None and any(it.request.pending for it in plan.items):
+        """Launch ``plan`` without waiting for it; ``after`` is the plan in flight and its launched step, or None.
+        None (nothing done) if the plan cannot be launched so, False if the step function declined.  A request's next
+        token that the host has not seen yet (``pending``) must be a sample of the step in flight: it is taken from
+        there on the device."""
+        if not plan.items or plan.preempted or not all(it.request.params.plain() for it in plan.items if it.sample):
             return None
         reqs = [it.request for it in plan.items]
-        # after another launch the tokens are taken on the device; the entries' own are placeholders
-        entries = [StepEntry(r.slot, [0] if after is not None else [r.tokens[it.start]], [0]) for r, it in zip(reqs, plan.items)]
-        launched = self.loaded.step.launch_decode(
-            entries, [r.params.temperature for r in reqs], [r.params.top_k for r in reqs], [r.params.top_p for r in reqs],
-            [r.rng_state for r in reqs], after)
+        prev_plan, prev = after if after is not None else (None, None)
+        where = {}
+        if prev_plan is not None:
+            k = 0
+            for it in prev_plan.items:
+                if it.sample:
+                    where[it.request.id] = k
+                    k += 1
+        feeds, entries = [], []
+        for i, (r, it) in enumerate(zip(reqs, plan.items)):
+            if it.start + it.count > len(r.tokens):
+                # its first token is still on the device: one token, sampled by the step in flight
+                if it.count != 1 or it.start != len(r.tokens) or r.pending != 1 or r.id not in where:
+                    return None
+                feeds.append((i, where[r.id]))
+                entries.append(StepEntry(r.slot, [0], [0] if it.sample else []))
+            else:
+                entries.append(StepEntry(r.slot, r.tokens[it.start:it.start + it.count], [it.count - 1] if it.sample else []))
+        sampled = [r for r, it in zip(reqs, plan.items) if it.sample]
+        if not sampled:
+            return None  # nothing comes back from it: it runs as it is
+        args = ([r.params.temperature for r in sampled], [r.params.top_k for r in sampled], [r.params.top_p for r in sampled],
+                [r.rng_state for r in sampled])
+        step = self.loaded.step
+        if all(it.sample and it.count == 1 for it in plan.items):
+            same = prev is not None and len(feeds) == len(entries) and all(e == s for e, s in feeds) and len(where) == len(entries)
+            launched = step.launch_decode(entries, *args, prev if feeds else None, None if (same or not feeds) else feeds)
+        else:
+            launched = step.launch_step(entries, *args, prev if feeds else None, feeds or None)
         if launched is None:
             return False
         from ..sampling import advance
-        for r in reqs:
+        for r in sampled:
             r.rng_state = advance(r.rng_state)  # one draw a sampled row, whatever the token
         self.scheduler.begin(plan)
         self.steps += 1

@@ -275,10 +275,13 @@ class StepFunction:
         return (tuple(counts), n_want, tuple(sorted(widths.items())), sampled)
 
     def _run_graph(self, key: tuple, built, sampling=None, after: Optional["LaunchedDecode"] = None, fill_rows: int = 0,
-                   samples_feed_tokens: bool = True):
+                   samples_feed_tokens: bool = True, feeds=None):
         """Replays the captured step of this key on ``built`` (captures it first if it has none).  With ``sampling`` the
         graph also samples at its logits' rows; with ``samples_feed_tokens`` (a decode step: row i is sample i) the
-        samples are left in the step's token section as well, where the next replay finds its input."""
+        samples are left in the step's token section as well, where the next replay finds its input.  ``after`` is the
+        launched step before this one, whose samples are this step's input: row for row if ``feeds`` is None (the same
+        requests in the same order), else for the pairs ``(row of this step, index among that step's samples)`` of
+        ``feeds``; the other rows' tokens are the entries' own."""
         host, offsets, widths = built
         extra: Dict[str, np.ndarray] = {}
         if sampling is not None:
@@ -287,6 +290,11 @@ class StepFunction:
             extra["sample/top_p"] = np.asarray(top_ps, dtype=np.float32).view(np.int32)
             extra["sample/top_k"] = np.asarray(top_ks, dtype=np.int32)
             extra["sample/state"] = np.asarray(states, dtype=np.uint64).view(np.int32)
+            # which rows take their token from the step before, and from where among its samples: at most one a request
+            cap = offsets["seq_slot"][1]
+            extra["feed/rows"], extra["feed/src"] = np.full(cap, -1, dtype=np.int32), np.zeros(cap, dtype=np.int32)
+            for i, (row, src) in enumerate(feeds or ()):
+                extra["feed/rows"][i], extra["feed/src"][i] = row, src
         dg = self._graphs.get(key)
         if dg is not None:
             self._graphs.move_to_end(key)
@@ -306,7 +314,7 @@ class StepFunction:
         for k, a in extra.items():
             staged[dg.offsets[k][0]:dg.offsets[k][0] + a.size] = a
         start, size = dg.offsets["tokens"]
-        if after is not None and after.graph is dg:
+        if after is not None and feeds is None and after.graph is dg:
             # the sampling kernel of this graph's last replay left its tokens in the graph's own
             # token section: everything but that section is uploaded
             if start:
@@ -314,9 +322,13 @@ class StepFunction:
             dg.dev[start + size:].copy_(dg.pinned[start + size:], non_blocking=True)
         else:
             dg.dev.copy_(dg.pinned, non_blocking=True)
-            if after is not None:  # another graph ran that step (the block tables have grown a bucket)
+            if after is not None and feeds is None:  # another graph ran that step (the block tables have grown a bucket)
                 dg.dev[start:start + size].copy_(after.sampled[0])
         dg.copied.record()
+        if after is not None and feeds:
+            def part(k):
+                return dg.dev[dg.offsets[k][0]:dg.offsets[k][0] + dg.offsets[k][1]]
+            self.rt.ops.feed_tokens(part("tokens"), after.sampled[0], part("feed/rows"), part("feed/src"))
         if dg.graph is None:
             ctx = self._context_from(dg.dev, dg.offsets, widths)
             # Everything is loaded and compiled before the capture: one run of the step outside it.  That run and the
@@ -365,10 +377,12 @@ class StepFunction:
         return None if launched is None else self.collect(launched)
 
     def launch_decode(self, entries: Sequence[StepEntry], temperatures, top_ks, top_ps, states,
-                      after: Optional["LaunchedDecode"] = None) -> Optional["LaunchedDecode"]:
+                      after: Optional["LaunchedDecode"] = None, feeds=None) -> Optional["LaunchedDecode"]:
         """The same step, launched and not waited for.  With ``after`` - the launched step before
-        this one, of the same requests in the same order - the tokens are that step's samples,
-        taken on the device: the host need not have seen them.  None if the step cannot take this
+        this one - the tokens are that step's samples, taken on the device: the host need not have seen
+        them.  Without ``feeds`` that step held the same requests in the same order; with ``feeds``, pairs of
+        (entry of this step, index among that step's samples), only the listed entries take their token
+        from it and the others bring their own.  None if the step cannot take this
         path or its shape has not come often enough to be captured; ``OutOfPages`` before anything
         ran if the pages are not there."""
         if not (self.use_graphs and self.model.observer is None
@@ -376,7 +390,7 @@ class StepFunction:
                 and len({e.slot for e in entries}) == len(entries)):
             return None
         slots = [e.slot for e in entries]
-        if after is not None and after.slots != slots:
+        if after is not None and feeds is None and after.slots != slots:
             raise StepError("a step fed from the device must hold the requests of the step before, in the same order")
         cache = self.cache
         checked = self._check_entries(entries)
@@ -387,11 +401,15 @@ class StepFunction:
         # the rows that fill the step up are rows of the scratch slot: they sample greedily (their token is some
         # token of the vocabulary, which is all that the next step's embedding needs of it) and are dropped
         filled = [list(v) + [fill] * pad for v, fill in ((temperatures, 0.0), (top_ks, 0), (top_ps, 1.0), (states, 0))]
-        sampled, graph = self._run_graph(key, built, tuple(filled), after, fill_rows=pad)
+        sampled, graph = self._run_graph(key, built, tuple(filled), after, fill_rows=pad, feeds=feeds)
         for e in entries:
             cache.commit(e.slot, 1)
-        # the samples go to a pinned buffer of their own (the graph's is overwritten by its next replay)
-        rows = len(slots) + pad
+        return self._launched(slots, sampled, graph)
+
+    def _launched(self, slots: List[int], sampled: torch.Tensor, graph) -> "LaunchedDecode":
+        """The samples of a step that was just replayed go to a pinned buffer of their own (the graph's is overwritten
+        by its next replay), behind the step on its stream; nothing is waited for."""
+        rows = sampled.shape[1]
         ring = self._results.get(rows)
         if ring is None:
             ring = self._results[rows] = [torch.empty((2, rows), dtype=torch.int32, pin_memory=True) for _ in range(3)]
@@ -416,6 +434,15 @@ class StepFunction:
         first token).  None, before anything is taken or run, if the step cannot take this path: it is plain decoding
         (``decode_and_sample``), it is not filled up to a shared size, or that size has not come often enough to be
         captured (the caller then runs it through ``__call__`` with ``eager`` and samples from the logits)."""
+        launched = self.launch_step(entries, temperatures, top_ks, top_ps, states, capture_now=capture_now)
+        return None if launched is None else self.collect(launched)
+
+    def launch_step(self, entries: Sequence[StepEntry], temperatures, top_ks, top_ps, states, after: Optional["LaunchedDecode"] = None,
+                    feeds=None, capture_now: bool = False) -> Optional["LaunchedDecode"]:
+        """``step_and_sample``, launched and not waited for (``collect`` brings the samples).  With ``after``, the
+        launched step before this one, and ``feeds``, pairs of (entry of this step, index among that step's
+        samples), the first token of the listed entries is that sample, taken on the device; such an entry has one
+        token, whose value here is a placeholder."""
         if not (self.use_graphs and self.model.observer is None and all(e.positions is None for e in entries)):
             return None
         if all(len(e.tokens) == 1 for e in entries) and len({e.slot for e in entries}) == len(entries):
@@ -448,11 +475,20 @@ class StepFunction:
         # the rows that fill the wanted rows up sample greedily and are dropped
         pad = fill[2] - len(want)
         sampling = tuple(list(v) + [f] * pad for v, f in ((temperatures, 0.0), (top_ks, 0), (top_ps, 1.0), (states, 0)))
-        sampled, _ = self._run_graph(key, built, sampling, None, fill_rows=fill[0] - len(tokens), samples_feed_tokens=False)
+        row_feeds = None
+        if after is not None and feeds:
+            first_row, at = [], 0
+            for n in counts:
+                first_row.append(at)
+                at += n
+            if any(counts[e] != 1 for e, _ in feeds):
+                raise StepError("an entry fed from the device brings one token")
+            row_feeds = [(first_row[e], src) for e, src in feeds]
+        sampled, graph = self._run_graph(key, built, sampling, after if row_feeds else None, fill_rows=fill[0] - len(tokens),
+                                         samples_feed_tokens=False, feeds=row_feeds)
         for e in entries:
             cache.commit(e.slot, len(e.tokens))
-        both = sampled[:, :len(want)].cpu()  # the step's synchronisation
-        return both[0].tolist(), both[1].view(torch.float32).tolist()
+        return self._launched([e.slot for e in entries for _ in e.want], sampled, graph)
 
     # ------------------------------------------------------------------ the step
     def __call__(self, entries: Sequence[StepEntry], borrow_logits: bool = False, capture_now: bool = False,

@@ -128,6 +128,17 @@ class HipOps:
                                                     self._stream()))
         return x
 
+    def feed_tokens(self, tokens: torch.Tensor, sampled: torch.Tensor, rows: torch.Tensor, src: torch.Tensor) -> None:
+        """``tokens[rows[i]] = sampled[src[i]]`` where ``rows[i]`` is no negative number: the rows of a step whose
+        input the step before it sampled take it on the device."""
+        n = rows.numel()
+        self._want(tokens, torch.int32, "feed_tokens tokens")
+        self._want(sampled, torch.int32, "feed_tokens sampled")
+        self._want(rows, torch.int32, "feed_tokens rows", n)
+        self._want(src, torch.int32, "feed_tokens src", n)
+        self._check(self._core, self._core.ms_feed_tokens(_ptr(tokens), _ptr(sampled), _ptr(rows), _ptr(src), _c_int(n),
+                                                          _c_int(tokens.numel()), _c_int(sampled.numel()), self._stream()))
+
     def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, rows: Optional[torch.Tensor] = None,
                 out_f32: bool = False, partials: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Norm of ``x + sum(partials)`` (of its ``rows`` if given).  With ``partials [P, T, d]`` and

@@ -574,28 +574,43 @@ def test_engine_reports_logprobs_and_top_logprobs(tmp_path):
 
 
 class _LaggedDecode:
-    """Stand-in on the CPU for the launched decode step of the device: what it samples stays out of
+    """Stand-in on the CPU for the launched steps of the device: what a step samples stays out of
     the engine's sight until ``collect``, and a step launched after another takes that step's tokens
-    from it directly, as the device does."""
+    from it directly, as the device does (row for row, or for the listed entries)."""
 
     def __init__(self, eng):
-        self.eng, self.fed_from_device = eng, 0
+        self.eng, self.fed_from_device, self.mixed = eng, 0, 0
         eng.loaded.step.launch_decode = self.launch_decode
+        eng.loaded.step.launch_step = self.launch_step
         eng.loaded.step.collect = lambda launched: (launched["tokens"], launched["logprobs"])
 
-    def launch_decode(self, entries, temperatures, top_ks, top_ps, states, after=None):
+    def _run(self, entries, temperatures, top_ks, top_ps, states, after, feeds):
         from machserve_amd.engine.step import StepEntry
         from machserve_amd.sampling import SamplingParams
-        if not all(len(e.tokens) == 1 for e in entries):
-            return None
+        entries = list(entries)
         if after is not None:
-            assert after["slots"] == [e.slot for e in entries]
-            entries = [StepEntry(e.slot, [t], e.want) for e, t in zip(entries, after["tokens"])]
+            if feeds is None:
+                assert after["slots"] == [e.slot for e in entries]
+                feeds = [(i, i) for i in range(len(entries))]
+            for i, src in feeds:
+                assert len(entries[i].tokens) == 1
+                entries[i] = StepEntry(entries[i].slot, [after["tokens"][src]], entries[i].want)
             self.fed_from_device += 1
         logits = self.eng.loaded.step(entries)
         params = [SamplingParams(temperature=t, top_k=k, top_p=p) for t, k, p in zip(temperatures, top_ks, top_ps)]
-        tokens, logprobs, _, _ = self.eng.sampler.sample(logits, params, list(states), [[] for _ in entries])
-        return {"slots": [e.slot for e in entries], "tokens": [int(t) for t in tokens], "logprobs": list(logprobs)}
+        tokens, logprobs, _, _ = self.eng.sampler.sample(logits, params, list(states), [[] for _ in params])
+        return {"slots": [e.slot for e in entries for _ in e.want], "tokens": [int(t) for t in tokens], "logprobs": list(logprobs)}
+
+    def launch_decode(self, entries, temperatures, top_ks, top_ps, states, after=None, feeds=None):
+        if not all(len(e.tokens) == 1 for e in entries):
+            return None
+        return self._run(entries, temperatures, top_ks, top_ps, states, after, feeds)
+
+    def launch_step(self, entries, temperatures, top_ks, top_ps, states, after=None, feeds=None, capture_now=False):
+        if all(len(e.tokens) == 1 for e in entries):
+            return None
+        self.mixed += 1
+        return self._run(entries, temperatures, top_ks, top_ps, states, after, feeds)
 
 
 @pytest.mark.parametrize("pages", [16, 4])
@@ -630,11 +645,12 @@ def test_pipelined_steps_give_what_synchronous_steps_give(tmp_path, pages):
         per_request = {i: [t for j, t in emitted if j == i] for i in ids}
         assert all(per_request[i] == done[i].generated for i in ids)
         return ([(done[i].generated, done[i].finish_reason, [round(x, 5) for x in done[i].logprobs]) for i in ids],
-                lag.fed_from_device, sum(done[i].preemptions for i in ids))
+                lag.fed_from_device, sum(done[i].preemptions for i in ids), lag.mixed)
 
-    plain, _, _ = run(False)
-    piped, from_device, preempted = run(True)
+    plain, _, _, _ = run(False)
+    piped, from_device, preempted, mixed = run(True)
     assert piped == plain and from_device > 3
+    assert mixed >= 2, "the prompts' steps and the step of the arrival beside the decoding requests were launched ahead too"
     assert (preempted > 0) == (pages == 4)
     assert [r for _, r, _ in plain] == ["length"] * 4
     # an end-of-sequence token and a stop sequence taken from the middle of what request 0 generates
@@ -642,10 +658,57 @@ def test_pipelined_steps_give_what_synchronous_steps_give(tmp_path, pages):
     eos = first[5]
     stop = [first[3:5]]
     for kw in ({"eos": eos}, {"stop": stop}, {"eos": plain[1][0][-1]}):
-        a, _, _ = run(False, **kw)
-        b, n_dev, _ = run(True, **kw)
+        a, _, _, _ = run(False, **kw)
+        b, n_dev, _, _ = run(True, **kw)
         assert a == b and n_dev > 0
         assert "stop" in [r for _, r, _ in a]
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_pipelined_steps_under_random_arrivals(tmp_path, seed):
+    """Requests of random lengths arriving at random steps under a small token budget and few pages, some ending at an
+    end-of-sequence token: steps of every mix launched one ahead (prompt portions beside requests that take their token
+    from the step in flight) give every request the tokens, log-probabilities and reason to finish of one step at a
+    time."""
+    from machserve_amd.engine import Engine, load_model
+    from machserve_amd.sampling import SamplingParams
+    d = make_model_dir(tmp_path, "B")
+    rnd = random.Random(70 + seed)
+    vocab = read_for_plain(d)[1]["vocab"]
+    n = 9
+    prompts = [random_prompt(rnd.randint(2, 45), vocab, 900 + 17 * seed + i) for i in range(n)]
+    max_new = [rnd.randint(1, 12) for _ in range(n)]
+    arrive = sorted(rnd.randint(0, 25) for _ in range(n))
+    temps = [rnd.choice([0.0, 0.8]) for _ in range(n)]
+    budget, pages = rnd.choice([16, 24, 48]), rnd.choice([10, 14, 30])
+
+    def run(pipelined, eos):
+        lm = load_model(d, dtype="float32", device="cpu", page_size=16, num_pages=pages, max_requests=3, ops=EmulatedOps())
+        eng = Engine(lm, max_batch_tokens=budget)
+        lag = _LaggedDecode(eng)
+        ids, step = [], 0
+        while len(ids) < n or eng.has_work():
+            while len(ids) < n and arrive[len(ids)] <= step:
+                i = len(ids)
+                ids.append(eng.add(prompts[i], max_new[i], SamplingParams(temperature=temps[i], seed=5 + i), eos=eos))
+            if eng.has_work():
+                eng.step_pipelined() if pipelined else eng.step()
+            step += 1
+            lm.cache.check()
+            assert step < 2000
+        assert all(g.pool.available() == g.pool.num_pages for g in lm.cache.groups.values())
+        done = eng.scheduler.finished
+        return [(done[i].generated, done[i].finish_reason, [round(x, 5) for x in done[i].logprobs]) for i in ids], lag
+
+    plain, _ = run(False, None)
+    piped, lag = run(True, None)
+    assert piped == plain
+    assert lag.mixed > 0 and lag.fed_from_device > 0
+    # a token that some request generates in its middle ends every request that meets it
+    longest = max(plain, key=lambda r: len(r[0]))[0]
+    if len(longest) >= 3:
+        eos = longest[len(longest) // 2]
+        assert run(True, eos)[0] == run(False, eos)[0]
 
 
 def test_cancel_while_a_step_is_in_flight(tmp_path):
