@@ -69,7 +69,8 @@ class StepFunction:
     TABLE_BUCKET = 8        # captured block tables are this many pages wide, or a multiple
     MAX_GRAPHS = 256        # captured steps kept; the one unused longest goes first
     # ... and the most memory they may hold for good between them: each keeps its step buffer and its results (the
-    # logits [rows, vocabulary] in 32-bit are nearly all of it: 39 MB at 64 rows of a 152k vocabulary).  What a
+    # logits [rows, vocabulary] in 32-bit are nearly all of it, 39 MB at 64 rows of a 152k vocabulary, where the
+    # caller gets logits; a step that samples inside keeps the samples only).  What a
     # captured step needs only while it runs comes from one pool that all captures share, since they run one
     # after another on one stream.  This reserve is device memory beside the weights and the page pools.
     MAX_GRAPH_BYTES = 2 << 30
@@ -354,6 +355,11 @@ class StepFunction:
                         dg.logits, sec("sample/temperature").view(torch.float32), sec("sample/top_k"),
                         sec("sample/top_p").view(torch.float32), sec("sample/state").view(torch.int64), True,
                         also_tokens=sec("tokens") if samples_feed_tokens else None)
+            if sampling is not None:
+                # Nobody reads a sampling step's logits outside it: their memory (nearly all that such a step would hold
+                # for good: 78 MB at 128 sampled rows of a 152k vocabulary) goes back to the pool that the captured
+                # steps share, like every other buffer a step needs only while it runs.
+                dg.logits = None
             dg.graph = graph
             self._graphs[key] = dg
             while len(self._graphs) > 1 and (len(self._graphs) > self.MAX_GRAPHS or self.graph_bytes() > self.MAX_GRAPH_BYTES):
