@@ -54,10 +54,10 @@ class _DecodeGraph:
 
 @dataclass
 class LaunchedDecode:
-    """A decode step that runs on the device: its requests' slots, the device tensor that will hold
-    its samples (int32 ``[2, B]``: tokens, bits of the logprobs), the pinned copy of it, the
-    event after that copy, and the captured graph that ran it (whose token section holds the
-    sampled tokens as well)."""
+    """A step that samples inside (a decode step, or a step of any mix) and runs on the device: the slot of
+    every sampled row's request, the device tensor that will hold its samples (int32 ``[2, B]``: tokens, bits
+    of the logprobs; rows beyond the slots belong to nobody), the pinned copy of it, the event after that
+    copy, and the captured graph that ran it (a decode step's token section holds the sampled tokens as well)."""
     slots: List[int]
     sampled: torch.Tensor
     result: torch.Tensor
