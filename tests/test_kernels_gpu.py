@@ -795,6 +795,20 @@ def test_top_logprobs():
     assert tok3.shape == (4, 3) and torch.equal(tok3.cpu(), tok[:, :3])
 
 
+def test_feed_tokens():
+    """The rows of a step whose input the step before it sampled take it on the device: listed rows only, entries of
+    row -1 (the list is filled up to a fixed length) and anything outside either buffer change nothing."""
+    ops = ops_for(torch.float32)
+    tokens = torch.arange(100, 120, dtype=torch.int32, device=DEV)
+    sampled = torch.tensor([7, 8, 9, 10, 11], dtype=torch.int32, device=DEV)
+    rows = torch.tensor([3, 0, 19, -1, -1, 25, 4, -1], dtype=torch.int32, device=DEV)
+    src = torch.tensor([4, 0, 2, 1, 0, 1, 9, 0], dtype=torch.int32, device=DEV)
+    ops.feed_tokens(tokens, sampled, rows, src)
+    want = list(range(100, 120))
+    want[3], want[0], want[19] = 11, 7, 9       # row 25 is beyond the tokens, sample 9 beyond the samples
+    assert tokens.cpu().tolist() == want
+
+
 def test_logit_edit():
     ops = ops_for(torch.float32)
     x = torch.zeros(2, 10, device=DEV)
